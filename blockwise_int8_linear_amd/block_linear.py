@@ -1,0 +1,123 @@
+"""Drop-in for the reference's block_linear.py: ``BlockInt8Linear`` (an ``nn.Linear`` whose forward and
+backward run blockwise-int8 GEMMs), its autograd function and the model-surgery helper, rewired onto the
+HIP operators of ``ops.py``.
+
+Differences from the reference that do not change results:
+  * the backward pass quantizes the transposes of W, X and G with one fused kernel each instead of
+    ``.t().contiguous()`` followed by the row quantizer (block_linear.py:93-94, :100-103);
+  * ``ctx.save_for_backward`` is called, not assigned over (block_linear.py:73);
+  * switching the module back to training mode drops the cached int8 weights, so a later ``eval()``
+    re-quantizes the current weights (the reference keeps serving the first cache, block_linear.py:138-139).
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from .ops import (
+    dequantize_block_rowwise,
+    int8_matmul_block64_rowwise_dequantize,
+    quantize_block_rowwise,
+    quantize_block_transposed,
+)
+
+
+def replace_linear_with_blockwise_int8(model):
+    """Swap the DIRECT child ``nn.Linear`` modules of `model` for ``BlockInt8Linear`` sharing the same
+    weight/bias storage (block_linear.py:16-32; use ``model.apply(...)`` to recurse)."""
+    to_be_replaced = [name for name, module in model.named_children()
+                      if isinstance(module, nn.Linear) and not isinstance(module, BlockInt8Linear)]
+    for name in to_be_replaced:
+        module = model._modules[name]
+        new = BlockInt8Linear(module.in_features, module.out_features, module.bias is not None,
+                              module.weight.device, module.weight.dtype)
+        new.weight.data = module.weight.data
+        if module.bias is not None:
+            new.bias.data = module.bias.data
+        new.train(module.training)
+        model._modules[name] = new
+    return model
+
+
+class blockwise_int8_linear(torch.autograd.Function):
+    """y = x @ W.T + bias with both operands block-quantized on the fly (block_linear.py:69-112)."""
+
+    @staticmethod
+    def forward(ctx, X_3D, W, bias):
+        X = X_3D.reshape(-1, X_3D.size(-1))
+        ctx.save_for_backward(X, W)
+        X_int8, state_X = quantize_block_rowwise(X)
+        W_int8, state_W = quantize_block_rowwise(W)
+        out = int8_matmul_block64_rowwise_dequantize(X_int8, W_int8.t(), state_X, state_W, bias)
+        return out.view(*X_3D.size()[:-1], -1)
+
+    @staticmethod
+    def backward(ctx, G_3D):
+        G = G_3D.reshape(-1, G_3D.size(-1))
+        grad_X = grad_W = grad_bias = None
+        X, W = ctx.saved_tensors
+        if ctx.needs_input_grad[0]:
+            # grad_X [M,K] = G [M,N] @ W [N,K]: contraction over N, so W is requantized along N
+            g_int8, g_state = quantize_block_rowwise(G)
+            Wt_int8, w_state = quantize_block_transposed(W)                 # [K,N], [N/B,K]
+            grad_X = int8_matmul_block64_rowwise_dequantize(g_int8, Wt_int8.t(), g_state, w_state)
+            grad_X = grad_X.view(*G_3D.size()[:-1], -1)
+        if ctx.needs_input_grad[1]:
+            # grad_W [N,K] = G.T [N,M] @ X [M,K]: contraction over the tokens, both requantized along M
+            x_int8, x_state = quantize_block_transposed(X)                  # [K,M], [M/B,K]
+            gt_int8, gt_state = quantize_block_transposed(G)                # [N,M], [M/B,N]
+            grad_W = int8_matmul_block64_rowwise_dequantize(gt_int8, x_int8.t(), gt_state, x_state)
+        if ctx.needs_input_grad[2]:
+            grad_bias = G.sum(dim=0)
+        return grad_X, grad_W, grad_bias
+
+
+class BlockInt8Linear(nn.Linear):
+    """``nn.Linear`` replacement (block_linear.py:114-152).  Training mode: ``blockwise_int8_linear``.
+    Eval mode: weights quantized once into the buffers ``W_int8`` [N,K] int8 and ``state_W``
+    [ceil(K/B),N], activations quantized per call, one fused GEMM."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None):
+        super().__init__(in_features, out_features, bias, device, dtype)
+
+    def prepare_for_eval(self):
+        W_int8, state_W = quantize_block_rowwise(self.weight.detach())
+        self.register_buffer("W_int8", W_int8)
+        self.register_buffer("state_W", state_W)
+
+    def weight_quant_training(self, x=None):
+        """Replace the weight by its quantize->dequantize image (block_linear.py:130-135).  As in the
+        reference the attribute becomes a plain tensor, no longer a Parameter."""
+        W_int8, state_W = quantize_block_rowwise(self.weight.detach())
+        del self.weight
+        self.weight = dequantize_block_rowwise(W_int8, state_W)
+
+    def infer(self, x):
+        if getattr(self, "W_int8", None) is None:
+            self.prepare_for_eval()
+        X = x.reshape(-1, x.size(-1))
+        X_int8, state_X = quantize_block_rowwise(X)
+        return int8_matmul_block64_rowwise_dequantize(
+            X_int8, self.W_int8.t(), state_X, self.state_W, self.bias
+        ).view(*x.size()[:-1], -1)
+
+    def forward(self, x):
+        if not self.training:
+            return self.infer(x)
+        return blockwise_int8_linear.apply(x, self.weight, self.bias)
+
+    def train(self, mode: bool = True):
+        if mode and "W_int8" in self._buffers:
+            del self._buffers["W_int8"]
+            del self._buffers["state_W"]
+        return super().train(mode)
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        # a checkpoint written after the first eval call carries the cached int8 weights
+        for name in ("W_int8", "state_W"):
+            if prefix + name in state_dict and name not in self._buffers:
+                self.register_buffer(name, torch.empty_like(state_dict[prefix + name], device=self.weight.device))
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
+
+BlockLinear = BlockInt8Linear

@@ -1,0 +1,200 @@
+// Block quantize of the transpose (bi8_quantize_transposed): x [R,C] -> codes [C,R], scales [ceil(R/B), C],
+// blocks running down the columns of x.  The backward pass of the reference materializes x.t().contiguous()
+// and then calls the row quantizer (block_linear.py:93-94, :100-103): two extra full passes over HBM.
+// Here one workgroup reads a 128-row x 64-column tile once with 128-bit row loads, keeps it in LDS as
+// fp32, reduces and quantizes down the columns, transposes the codes through LDS and writes them as
+// 128-byte runs of the output rows.  Results are identical to the two-step form.
+#include "bi8_common.h"
+
+namespace {
+
+constexpr int kTR = 128;           // tile rows (source rows = output columns)
+constexpr int kTC = 64;            // tile columns (source columns = output rows)
+constexpr int kThreads = 256;
+constexpr int kPitch = kTC + 1;    // fp32 tile pitch: column walks hit distinct banks
+constexpr int kQPitch = kTR + 4;   // code tile pitch in bytes (33 dwords)
+
+template <int DT> struct Vec {
+    static constexpr int kElems = (DT == BI8_F32) ? 4 : 8;
+};
+
+template <int DT> __device__ __forceinline__ void unpack(const bi8_v4u &raw, float *f) {
+    if constexpr (DT == BI8_F32) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[e] = bi8_u2f(raw[e]);
+    } else if constexpr (DT == BI8_BF16) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f[2 * e] = bi8_u2f(raw[e] << 16);
+            f[2 * e + 1] = bi8_u2f(raw[e] & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f[2 * e] = bi8_from_f16_bits(raw[e] & 0xffffu);
+            f[2 * e + 1] = bi8_from_f16_bits(raw[e] >> 16);
+        }
+    }
+}
+
+// B in {32, 64, 128}: thread (c = tid % 64, g = tid / 64) owns source rows 32g .. 32g+31 of column c.
+template <int DT, int B>
+__global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__restrict__ x, int8_t *__restrict__ qT,
+                                                               float *__restrict__ scalesT, int64_t R, int64_t C,
+                                                               int64_t ldx, int64_t ldq, int tiles_c) {
+    constexpr int VEC = Vec<DT>::kElems;
+    constexpr int64_t ES = 16 / VEC;
+    constexpr int LPR = kTC / VEC;                 // lanes per tile row
+    constexpr int RPP = kThreads / LPR;            // rows per load pass
+    constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
+    constexpr int GPB = B / 32;                    // 32-row groups per block
+    __shared__ float s_x[kTR * kPitch];
+    __shared__ float s_max[4][kTC];
+    __shared__ __attribute__((aligned(16))) uint8_t s_q[kTC * kQPitch];
+
+    const int tid = threadIdx.x;
+    const int64_t tile_r = blockIdx.x / tiles_c;
+    const int tile_c = blockIdx.x % tiles_c;
+    const int64_t r0 = tile_r * kTR;
+    const int64_t c0 = (int64_t)tile_c * kTC;
+    const char *xb = (const char *)x;
+
+    // phase 1: rows of the tile -> fp32 in LDS
+#pragma unroll
+    for (int p = 0; p < kTR / RPP; ++p) {
+        const int r = p * RPP + tid / LPR;
+        const int cc = (tid % LPR) * VEC;
+        bi8_v4u raw = {0u, 0u, 0u, 0u};
+        if (r0 + r < R && c0 + cc < C) raw = __builtin_nontemporal_load((const bi8_v4u *)(xb + ((r0 + r) * ldx + c0 + cc) * ES));
+        float f[VEC];
+        unpack<DT>(raw, f);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) s_x[r * kPitch + cc + e] = f[e];
+    }
+    __syncthreads();
+
+    // phase 2: column maxima over this thread's 32 rows, then over the block's row groups
+    const int c = tid & 63;
+    const int g = tid >> 6;
+    float v[32];
+    float m = 0.0f;
+    bool special = false;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        v[i] = s_x[(g * 32 + i) * kPitch + c];
+        m = __builtin_fmaxf(m, __builtin_fabsf(v[i]));
+        special |= (v[i] != v[i]);
+    }
+    if constexpr (GPB > 1) {
+        s_max[g][c] = m;
+        __syncthreads();
+        const int gb = g & ~(GPB - 1);
+#pragma unroll
+        for (int k = 0; k < GPB; ++k) m = __builtin_fmaxf(m, s_max[gb + k][c]);
+    }
+    if ((g & (GPB - 1)) == 0) {
+        const int64_t jb = (r0 + g * 32) / B;
+        if (r0 + g * 32 < R && c0 + c < C) scalesT[jb * C + c0 + c] = m;
+    }
+
+    // phase 3: codes of this thread's 32 rows -> byte tile [column][row]
+    special |= !bi8_scale_is_ordinary(m);
+    uint32_t code[32];
+    if (__builtin_expect(special, 0)) {
+#pragma unroll
+        for (int i = 0; i < 32; ++i) code[i] = bi8_code_slow(v[i], m);
+    } else {
+        const float y = 1.0f / m;
+#pragma unroll
+        for (int i = 0; i < 32; ++i) code[i] = bi8_code_fast<NCORR>(v[i], m, y);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        *(uint32_t *)&s_q[c * kQPitch + g * 32 + 4 * i] = bi8_pack4(code[4 * i], code[4 * i + 1], code[4 * i + 2], code[4 * i + 3]);
+    __syncthreads();
+
+    // phase 4: 16 codes per lane, 8 lanes per output row
+#pragma unroll
+    for (int p = 0; p < (kTC * kTR / 16) / kThreads; ++p) {
+        const int idx = p * kThreads + tid;
+        const int oc = idx / (kTR / 16);           // output row inside the tile = source column
+        const int seg = idx % (kTR / 16);
+        const int64_t orow = c0 + oc;
+        const int64_t ocol = r0 + seg * 16;
+        if (orow < C && ocol < R) {
+            const uint32_t *src = (const uint32_t *)&s_q[oc * kQPitch + seg * 16];
+            bi8_v4u w = {src[0], src[1], src[2], src[3]};
+            int8_t *dst = qT + orow * ldq + ocol;
+            if (ocol + 16 <= R) {
+                __builtin_nontemporal_store(w, (bi8_v4u *)dst);
+            } else {
+                for (int e = 0; e < (int)(R - ocol); ++e) dst[e] = (int8_t)((w[e >> 2] >> (8 * (e & 3))) & 0xffu);
+            }
+        }
+    }
+}
+
+// Any block size / alignment: one thread per (output row, block); consecutive threads read consecutive columns.
+template <int DT>
+__global__ __launch_bounds__(kThreads) void quantize_cols_generic(const void *__restrict__ x, int8_t *__restrict__ qT,
+                                                                  float *__restrict__ scalesT, int64_t R, int64_t C,
+                                                                  int64_t ldx, int64_t ldq, int64_t nblk, int block) {
+    const int64_t units = C * nblk;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    for (int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x; u < units; u += stride) {
+        const int64_t j = u / C, c = u % C;
+        const int64_t ra = j * block;
+        const int64_t n = (R - ra < block) ? (R - ra) : block;
+        float m = 0.0f;
+        for (int64_t i = 0; i < n; ++i) m = __builtin_fmaxf(m, __builtin_fabsf(bi8_load_elem<DT>(x, (ra + i) * ldx + c)));
+        scalesT[j * C + c] = m;
+        for (int64_t i = 0; i < n; ++i)
+            qT[c * ldq + ra + i] = (int8_t)(bi8_code_slow(bi8_load_elem<DT>(x, (ra + i) * ldx + c), m) & 0xffu);
+    }
+}
+
+template <int DT, int B>
+int launch_tile(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq, hipStream_t st) {
+    const int64_t tiles_c = (C + kTC - 1) / kTC;
+    const int64_t tiles_r = (R + kTR - 1) / kTR;
+    if (tiles_c * tiles_r > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((quantize_cols_tile<DT, B>), dim3((unsigned)(tiles_c * tiles_r)), dim3(kThreads), 0, st, x, qT, scalesT, R, C,
+                       ldx, ldq, (int)tiles_c);
+    return bi8_launch_rc();
+}
+
+template <int DT>
+int dispatch(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq, int block, hipStream_t st) {
+    constexpr int VEC = Vec<DT>::kElems;
+    const bool tile_ok = C % VEC == 0 && ldx % VEC == 0 && ldq % 16 == 0 && bi8_aligned(x, 16) && bi8_aligned(qT, 16);
+    if (tile_ok) {
+        switch (block) {
+        case 32: return launch_tile<DT, 32>(x, qT, scalesT, R, C, ldx, ldq, st);
+        case 64: return launch_tile<DT, 64>(x, qT, scalesT, R, C, ldx, ldq, st);
+        case 128: return launch_tile<DT, 128>(x, qT, scalesT, R, C, ldx, ldq, st);
+        }
+    }
+    const int64_t nblk = (R + block - 1) / block;
+    int64_t grid = (C * nblk + kThreads - 1) / kThreads;
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL((quantize_cols_generic<DT>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, qT, scalesT, R, C, ldx, ldq, nblk,
+                       block);
+    return bi8_launch_rc();
+}
+
+}  // namespace
+
+extern "C" int bi8_quantize_transposed(const void *x, int x_dtype, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx,
+                                       int64_t ldq, int block, void *stream) {
+    if (x_dtype < 0 || x_dtype > 2) return BI8_ERR_BAD_DTYPE;
+    if (block < 1 || block > (1 << 20)) return BI8_ERR_BAD_BLOCK;
+    if (R < 0 || C < 0 || ldx < C || ldq < R) return BI8_ERR_BAD_SHAPE;
+    if (R == 0 || C == 0) return BI8_OK;
+    if (!x || !qT || !scalesT) return BI8_ERR_NULL_POINTER;
+    hipStream_t st = (hipStream_t)stream;
+    switch (x_dtype) {
+    case BI8_F32: return dispatch<BI8_F32>(x, qT, scalesT, R, C, ldx, ldq, block, st);
+    case BI8_BF16: return dispatch<BI8_BF16>(x, qT, scalesT, R, C, ldx, ldq, block, st);
+    default: return dispatch<BI8_F16>(x, qT, scalesT, R, C, ldx, ldq, block, st);
+    }
+}

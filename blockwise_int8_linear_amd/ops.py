@@ -1,0 +1,155 @@
+"""Operator launchers with the reference's names, signatures and output layouts
+(triton_functions.py:221-233, :492-500, :142-168), running hand-written gfx950 kernels through the
+C ABI of libbi8.so.  Like the reference's launchers they allocate their outputs with torch.empty on the
+input's device, enqueue on the current stream and return without synchronizing.
+
+There is one code path: device tensors, HIP kernels.  A CPU tensor trips the same assertion as in the
+reference (``assert x.is_cuda``); a missing libbi8.so raises.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from . import block_linear_config
+
+_DT = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+def ceil_div(n: int, d: int) -> int:
+    return -(n // -d)
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _float_operand(x: torch.Tensor) -> torch.Tensor:
+    if x.dtype not in _DT:
+        raise TypeError(f"unsupported dtype {x.dtype}: expected float32, bfloat16 or float16")
+    return x if x.stride(-1) == 1 or x.numel() == 0 else x.contiguous()
+
+
+def _rows(x: torch.Tensor) -> torch.Tensor:
+    """2-D tensor whose rows are contiguous (leading dimension = stride(0))."""
+    if x.numel() and (x.stride(1) != 1 or (x.shape[0] > 1 and x.stride(0) < x.shape[1])):
+        return x.contiguous()
+    return x
+
+
+def _ld(x: torch.Tensor) -> int:
+    return x.stride(0) if x.shape[0] > 1 else max(x.shape[1], 1)
+
+
+def _scales_out(s: torch.Tensor) -> torch.Tensor:
+    t = block_linear_config.SHARED_EXP_TORCH_TYPE
+    return s if t == torch.float32 else s.to(t)       # the reference's store casts to the scale dtype (:216, :227)
+
+
+def _scales_in(s: torch.Tensor) -> torch.Tensor:
+    s = s if s.dtype == torch.float32 else s.float()
+    return s if s.is_contiguous() else s.contiguous()
+
+
+def quantize_block_rowwise(x: torch.Tensor, fblock_size=None):
+    """x [M,K] -> (int8 codes [M,K], absmax scales [ceil(K/B), M]); triton_functions.py:221-233."""
+    fblock_size = fblock_size or block_linear_config.GROUP_SIZE
+    m, k = x.shape
+    assert x.is_cuda
+    x = _rows(_float_operand(x))
+    output = torch.empty((m, k), device=x.device, dtype=torch.int8)
+    # output_maxs is transposed: block-major, row-minor (:226-227)
+    output_maxs = torch.empty((ceil_div(k, fblock_size), m), device=x.device, dtype=torch.float32)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bi8_quantize_rowwise(x.data_ptr(), _DT[x.dtype], output.data_ptr(), output_maxs.data_ptr(),
+                                              m, k, _ld(x), max(k, 1), fblock_size, _stream(x))
+    _lib.check(rc, "bi8_quantize_rowwise")
+    return output, _scales_out(output_maxs)
+
+
+def quantize_block_transposed(x: torch.Tensor, fblock_size=None):
+    """Same result as ``quantize_block_rowwise(x.t().contiguous())`` (block_linear.py:93-94, :100-103) in one
+    pass over x:  x [R,C] -> (int8 [C,R], scales [ceil(R/B), C])."""
+    fblock_size = fblock_size or block_linear_config.GROUP_SIZE
+    r, c = x.shape
+    assert x.is_cuda
+    x = _rows(_float_operand(x))
+    output = torch.empty((c, r), device=x.device, dtype=torch.int8)
+    output_maxs = torch.empty((ceil_div(r, fblock_size), c), device=x.device, dtype=torch.float32)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bi8_quantize_transposed(x.data_ptr(), _DT[x.dtype], output.data_ptr(), output_maxs.data_ptr(),
+                                                 r, c, _ld(x), max(r, 1), fblock_size, _stream(x))
+    _lib.check(rc, "bi8_quantize_transposed")
+    return output, _scales_out(output_maxs)
+
+
+def dequantize_block_rowwise(x: torch.Tensor, state_x: torch.Tensor, fblock_size=None):
+    """int8 [M,K] + scales [ceil(K/B), M] -> [M,K] of INPUT_OUTPUT_TORCH_TYPE; triton_functions.py:492-500."""
+    fblock_size = fblock_size or block_linear_config.GROUP_SIZE
+    out_dtype = block_linear_config.INPUT_OUTPUT_TORCH_TYPE
+    assert x.is_cuda
+    assert x.dtype == torch.int8, "codes must be int8"
+    M, K = x.shape
+    assert tuple(state_x.shape) == (ceil_div(K, fblock_size), M), "scale shape must be [ceil(K/block), M]"
+    x = _rows(x)
+    state_x = _scales_in(state_x)
+    output = torch.empty((M, K), device=x.device, dtype=out_dtype)
+    with torch.cuda.device(x.device):
+        rc = _lib.load().bi8_dequantize_rowwise(x.data_ptr(), state_x.data_ptr(), output.data_ptr(), _DT[out_dtype],
+                                                M, K, _ld(x), max(K, 1), fblock_size, _stream(x))
+    _lib.check(rc, "bi8_dequantize_rowwise")
+    return output
+
+
+def _gemm_operands(a: torch.Tensor, b: torch.Tensor):
+    assert a.is_cuda and b.is_cuda
+    assert a.dtype == torch.int8 and b.dtype == torch.int8, "operands must be int8 codes"
+    assert a.shape[1] == b.shape[0], "incompatible dimensions"
+    a = _rows(a)
+    # b is [K,N]; the kernel wants its transpose [N,K] with contiguous rows, which is what the reference's
+    # callers pass (W_int8.t(), block_linear.py:80).  Anything else is copied into that layout once.
+    w = b.t()
+    w = _rows(w)
+    return a, w
+
+
+def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
+    """a int8 [M,K], b int8 [K,N] (any strides), state_x [K/B, M], state_w [K/B, N], bias [N] or None
+    -> [M,N] of INPUT_OUTPUT_TORCH_TYPE; triton_functions.py:142-168.  B = GROUP_SIZE at call time."""
+    block = block_linear_config.GROUP_SIZE
+    out_dtype = block_linear_config.INPUT_OUTPUT_TORCH_TYPE
+    a, w = _gemm_operands(a, b)
+    M, K = a.shape
+    N = w.shape[0]
+    nblk = ceil_div(K, block)
+    assert tuple(state_x.shape) == (nblk, M) and tuple(state_w.shape) == (nblk, N), "scale shapes must be [ceil(K/block), rows]"
+    state_x, state_w = _scales_in(state_x), _scales_in(state_w)
+    c = torch.empty((M, N), device=a.device, dtype=out_dtype)
+    bias_ptr, bias_dt = None, 0
+    if bias is not None:
+        assert bias.is_cuda and bias.numel() == N
+        if bias.dtype not in _DT:
+            bias = bias.float()
+        bias = bias.contiguous()
+        bias_ptr, bias_dt = bias.data_ptr(), _DT[bias.dtype]
+    with torch.cuda.device(a.device):
+        rc = _lib.load().bi8_gemm_nt_dequant(a.data_ptr(), w.data_ptr(), state_x.data_ptr(), state_w.data_ptr(),
+                                             bias_ptr, bias_dt, c.data_ptr(), _DT[out_dtype], M, N, K,
+                                             _ld(a), _ld(w), max(N, 1), block, _stream(a))
+    _lib.check(rc, "bi8_gemm_nt_dequant")
+    return c
+
+
+def int8_matmul_block_partials(a, b, fblock_size=None):
+    """The GEMM kernel's int32 block partials, before any scaling: int32 [ceil(K/B), M, N]
+    (what ``tl.dot`` yields at triton_functions.py:115).  Parity/debug operator."""
+    block = fblock_size or block_linear_config.GROUP_SIZE
+    a, w = _gemm_operands(a, b)
+    M, K = a.shape
+    N = w.shape[0]
+    p = torch.empty((ceil_div(K, block), M, N), device=a.device, dtype=torch.int32)
+    with torch.cuda.device(a.device):
+        rc = _lib.load().bi8_gemm_nt_partials(a.data_ptr(), w.data_ptr(), p.data_ptr(), M, N, K, _ld(a), _ld(w),
+                                              block, _stream(a))
+    _lib.check(rc, "bi8_gemm_nt_partials")
+    return p

@@ -1,0 +1,109 @@
+/*
+ * libbi8 -- blockwise int8 linear hot path for AMD MI355X (gfx950), C ABI.
+ *
+ * The reference (LiuTaowen-Tony/blockwise_int8_linear) has no FFI: its operator boundary is three
+ * Python launchers in triton_functions.py that allocate their outputs with torch.empty and start a
+ * Triton kernel on the current stream.  Each entry point below replaces the device work of one of
+ * those launchers; the Python side (blockwise_int8_linear_amd/ops.py) keeps the launchers' names,
+ * signatures and output layouts and only allocates and forwards pointers.
+ *
+ * Conventions
+ *   - plain pointers to DEVICE memory, element counts as int64_t, leading dimensions in ELEMENTS;
+ *   - the library never allocates, frees or synchronizes; every call only enqueues kernels on
+ *     `stream` (a hipStream_t passed as void*, NULL = the default stream) and returns;
+ *   - re-entrant, no global mutable state, callable from any host thread;
+ *   - return value 0 = success, BI8_ERR_* for rejected arguments (nothing was launched),
+ *     BI8_ERR_HIP_BASE + hipError_t when the launch itself failed;
+ *   - `block` is the quantization group size along the contraction dimension
+ *     (block_linear_config.GROUP_SIZE, block_linear_config.py:3): a power of two, 16..1024 for the
+ *     quantizers and 32..256 for the GEMM;
+ *   - scales use the reference's layout: fp32 [ceil(K/block), rows], block-major / row-minor
+ *     (triton_functions.py:214-216, :227), and hold the block ABSMAX (not absmax/127).
+ */
+#ifndef BI8_H
+#define BI8_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of the floating-point operands (block_linear_config.INPUT_OUTPUT_TORCH_TYPE) */
+#define BI8_F32 0
+#define BI8_BF16 1
+#define BI8_F16 2
+
+#define BI8_OK 0
+#define BI8_ERR_NULL_POINTER 1
+#define BI8_ERR_BAD_DTYPE 2
+#define BI8_ERR_BAD_BLOCK 3
+#define BI8_ERR_BAD_SHAPE 4   /* negative size, or a leading dimension smaller than the row length */
+#define BI8_ERR_TOO_LARGE 5   /* a dimension exceeds what one launch can index */
+#define BI8_ERR_HIP_BASE 1000 /* BI8_ERR_HIP_BASE + hipError_t */
+
+/* ABI version of this header (bumped on any signature change). */
+int bi8_version(void);
+
+/* Static, NUL-terminated description of a return code. */
+const char *bi8_strerror(int code);
+
+/*
+ * Block quantize along rows.  Replaces quantize_block_rowwise / _quantize_block_rowwise
+ * (triton_functions.py:221-233 / :193-216).
+ *   x       [M,K] of x_dtype, row-major, leading dimension ldx
+ *   q       int8 [M,K], leading dimension ldq:   rint_even(127 * (x / absmax)), two fp32 roundings
+ *   scales  fp32 [ceil(K/block), M]:             absmax of each (row, block)
+ * An all-zero block gets scale 0 and codes 0; NaN elements are ignored by the maximum and get code 0.
+ */
+int bi8_quantize_rowwise(const void *x, int x_dtype, int8_t *q, float *scales,
+                         int64_t M, int64_t K, int64_t ldx, int64_t ldq, int block, void *stream);
+
+/*
+ * Block quantize of the TRANSPOSE, without materializing it.  Replaces the pair
+ * `t = x.t().contiguous(); quantize_block_rowwise(t)` of the backward pass (block_linear.py:93-94,
+ * :100-103).
+ *   x        [R,C] of x_dtype, row-major, leading dimension ldx
+ *   qT       int8 [C,R], leading dimension ldq;  blocks run down the columns of x
+ *   scalesT  fp32 [ceil(R/block), C]
+ */
+int bi8_quantize_transposed(const void *x, int x_dtype, int8_t *qT, float *scalesT,
+                            int64_t R, int64_t C, int64_t ldx, int64_t ldq, int block, void *stream);
+
+/*
+ * Block dequantize.  Replaces dequantize_block_rowwise / _dequantize_block_rowwise
+ * (triton_functions.py:492-500 / :468-490):  out = (scale * float(q)) * fp32(1/127), cast to out_dtype.
+ */
+int bi8_dequantize_rowwise(const int8_t *q, const float *scales, void *out, int out_dtype,
+                           int64_t M, int64_t K, int64_t ldq, int64_t ldo, int block, void *stream);
+
+/*
+ * int8 GEMM with the per-K-block dequantize fused into the K loop.  Replaces
+ * int8_matmul_block64_rowwise_dequantize / _int8_matmul_block64_rowwise_dequantize
+ * (triton_functions.py:142-168 / :70-139), SPLIT_K = 1 semantics.
+ *   A   int8 [M,K], leading dimension lda      (quantized activations)
+ *   W   int8 [N,K], leading dimension ldw      (the reference passes the view W.t(): both operands
+ *                                               are contiguous along K, block_linear.py:80)
+ *   sA  fp32 [ceil(K/block), M],  sW  fp32 [ceil(K/block), N]
+ *   C[m,n] = cast( sum_j sW[j,n] * sA[j,m] * P_j[m,n] / 127^2 ),  P_j = int32 dot over K-block j;
+ *   then, if bias != NULL (bias [N] of bias_dtype):  C = C + cast(bias), evaluated in c_dtype
+ *   (triton_functions.py:127-131).  fp32 accumulation order over j is ascending; the products inside
+ *   one term may be associated differently from the reference (results agree to ~1e-6 relative).
+ */
+int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float *sA, const float *sW,
+                        const void *bias, int bias_dtype, void *C, int c_dtype,
+                        int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                        int block, void *stream);
+
+/*
+ * The int32 block partial products of the same kernel, before any scaling (what tl.dot yields at
+ * triton_functions.py:115):  P int32 [ceil(K/block), M, N], contiguous.  Parity/debug entry point.
+ */
+int bi8_gemm_nt_partials(const int8_t *A, const int8_t *W, int32_t *P,
+                         int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw,
+                         int block, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BI8_H */

@@ -1,0 +1,147 @@
+"""CPU-side checks of the boundary: libbi8.so loads and exports exactly what include/bi8.h declares, the
+ctypes signatures agree with the header, argument validation answers before any launch, and the Python
+layer keeps the reference's names, defaults and error behaviour.  No kernel is launched here."""
+import ctypes
+import inspect
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+import torch.nn as nn
+
+import blockwise_int8_linear_amd as pkg
+from blockwise_int8_linear_amd import _lib, block_linear_config, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _header_decls():
+    text = open(os.path.join(ROOT, "include", "bi8.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = {}
+    for m in re.finditer(r"(?:int|const char \*)\s*(bi8_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        args = [a.strip() for a in m.group(2).split(",")] if m.group(2).strip() != "void" else []
+        decls[m.group(1)] = args
+    return decls
+
+
+def test_library_exports_every_declared_symbol():
+    decls = _header_decls()
+    assert set(decls) == {"bi8_version", "bi8_strerror", "bi8_quantize_rowwise", "bi8_quantize_transposed",
+                          "bi8_dequantize_rowwise", "bi8_gemm_nt_dequant", "bi8_gemm_nt_partials"}
+    lib = _lib.load()
+    for name in decls:
+        assert hasattr(lib, name), f"{name} not exported"
+    # and nothing else with the library's prefix leaks out
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = {l.split()[-1] for l in out.splitlines() if " T " in l and l.split()[-1].startswith("bi8_")}
+    assert exported == set(decls)
+
+
+def test_ctypes_signatures_match_header():
+    decls = _header_decls()
+    assert set(decls) == set(_lib.SIGNATURES)
+    for name, args in decls.items():
+        res, argtypes = _lib.SIGNATURES[name]
+        assert len(args) == len(argtypes), name
+        for a, t in zip(args, argtypes):
+            if "*" in a:
+                assert t is ctypes.c_void_p, (name, a)
+            elif a.startswith("int64_t"):
+                assert t is ctypes.c_int64, (name, a)
+            else:
+                assert a.startswith("int ") and t is ctypes.c_int, (name, a)
+
+
+def test_version_and_error_strings():
+    lib = _lib.load()
+    assert lib.bi8_version() == _lib.ABI_VERSION == 1
+    assert lib.bi8_strerror(0) == b"success"
+    assert b"block" in lib.bi8_strerror(3)
+    with pytest.raises(_lib.Bi8Error, match="leading dimension"):
+        _lib.check(4, "x")
+
+
+def test_argument_validation_happens_before_any_launch():
+    """bad arguments are rejected on the host; none of these calls reaches the GPU runtime"""
+    lib = _lib.load()
+    p = ctypes.c_void_p(0x1000)
+    assert lib.bi8_quantize_rowwise(p, 7, p, p, 4, 128, 128, 128, 128, None) == 2          # dtype
+    assert lib.bi8_quantize_rowwise(p, 1, p, p, 4, 128, 128, 128, 0, None) == 3            # block
+    assert lib.bi8_quantize_rowwise(p, 1, p, p, 4, 128, 64, 128, 128, None) == 4           # ldx < K
+    assert lib.bi8_quantize_rowwise(p, 1, p, p, -1, 128, 128, 128, 128, None) == 4
+    assert lib.bi8_quantize_rowwise(None, 1, p, p, 4, 128, 128, 128, 128, None) == 1       # null
+    assert lib.bi8_quantize_rowwise(None, 1, None, None, 0, 128, 128, 128, 128, None) == 0  # empty: nothing to do
+    assert lib.bi8_quantize_transposed(p, 1, p, p, 4, 128, 128, 2, 128, None) == 4         # ldq < R
+    assert lib.bi8_dequantize_rowwise(p, p, p, 3, 4, 128, 128, 128, 128, None) == 2
+    assert lib.bi8_gemm_nt_dequant(p, p, p, p, None, 0, p, 1, 4, 4, 128, 64, 128, 4, 128, None) == 4
+    assert lib.bi8_gemm_nt_dequant(p, p, p, p, p, 9, p, 1, 4, 4, 128, 128, 128, 4, 128, None) == 2
+    assert lib.bi8_gemm_nt_dequant(None, None, None, None, None, 0, None, 1, 0, 4, 128, 128, 128, 4, 128, None) == 0
+    assert lib.bi8_gemm_nt_partials(p, p, None, 4, 4, 128, 128, 128, 128, None) == 1
+
+
+def test_python_api_mirrors_reference_names_and_defaults():
+    # triton_functions.py:221, :492, :142 and block_linear.py:16, :69, :114
+    assert list(inspect.signature(ops.quantize_block_rowwise).parameters) == ["x", "fblock_size"]
+    assert list(inspect.signature(ops.dequantize_block_rowwise).parameters) == ["x", "state_x", "fblock_size"]
+    assert list(inspect.signature(ops.int8_matmul_block64_rowwise_dequantize).parameters) == ["a", "b", "state_x", "state_w", "bias"]
+    assert inspect.signature(ops.int8_matmul_block64_rowwise_dequantize).parameters["bias"].default is None
+    assert list(inspect.signature(pkg.BlockInt8Linear.__init__).parameters) == ["self", "in_features", "out_features", "bias", "device", "dtype"]
+    for name in ("prepare_for_eval", "infer", "forward", "weight_quant_training"):
+        assert callable(getattr(pkg.BlockInt8Linear, name))
+    assert issubclass(pkg.BlockInt8Linear, nn.Linear) and issubclass(pkg.blockwise_int8_linear, torch.autograd.Function)
+    # block_linear_config.py:3-5
+    assert block_linear_config.GROUP_SIZE == 128
+    assert block_linear_config.SHARED_EXP_TORCH_TYPE == torch.float32
+    assert block_linear_config.INPUT_OUTPUT_TORCH_TYPE == torch.bfloat16
+
+
+def test_cpu_tensors_are_rejected_like_the_reference():
+    x = torch.zeros(4, 128)
+    with pytest.raises(AssertionError):                     # `assert x.is_cuda`, triton_functions.py:229
+        ops.quantize_block_rowwise(x)
+    with pytest.raises(AssertionError):                     # :496
+        ops.dequantize_block_rowwise(torch.zeros(4, 128, dtype=torch.int8), torch.zeros(1, 4))
+    with pytest.raises(AssertionError):
+        ops.int8_matmul_block64_rowwise_dequantize(torch.zeros(4, 128, dtype=torch.int8), torch.zeros(128, 4, dtype=torch.int8),
+                                                   torch.zeros(1, 4), torch.zeros(1, 4))
+    lin = pkg.BlockInt8Linear(128, 4)
+    with pytest.raises(AssertionError):                     # no silent CPU fallback in the module either
+        lin(x)
+
+
+def test_model_surgery_on_cpu_modules():
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = nn.Linear(8, 16)
+            self.seq = nn.Sequential(nn.Linear(16, 16), nn.ReLU())
+
+    net = Net().eval()
+    w = net.a.weight.data_ptr()
+    pkg.replace_linear_with_blockwise_int8(net)
+    assert isinstance(net.a, pkg.BlockInt8Linear) and net.a.weight.data_ptr() == w and not net.a.training
+    assert type(net.seq[0]) is nn.Linear
+    assert set(net.a.state_dict()) == {"weight", "bias"}
+    net.apply(pkg.replace_linear_with_blockwise_int8)
+    assert isinstance(net.seq[0], pkg.BlockInt8Linear)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libbi8.so"))
+    with pytest.raises(_lib.Bi8Error, match="no CPU or PyTorch fallback"):
+        _lib.load()
+
+
+def test_recip_division_is_exact():
+    """the quantizer's reciprocal-multiply division, restated in C with fmaf(): exhaustive over all pairs of
+    16-bit inputs (one correction), sampled for binary32 (two corrections) -- see tests/c/recip_division_check.c"""
+    src = os.path.join(ROOT, "tests", "c", "recip_division_check.c")
+    exe = "/tmp/bi8_recip_division_check"
+    subprocess.run(["gcc", "-O2", "-ffp-contract=off", "-fopenmp", src, "-o", exe, "-lm"], check=True)
+    res = subprocess.run([exe, "50000000"], capture_output=True, text=True)
+    assert res.returncode == 0, res.stdout
+    assert res.stdout.count(" 0 mismatches") == 3, res.stdout

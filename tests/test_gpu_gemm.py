@@ -1,0 +1,203 @@
+"""GPU parity of the int8 block GEMM with fused dequantize against the CPU checker: int32 block partials
+bit-exact, outputs within rel 1e-3 (fp32 out) / 1e-2 (bf16, fp16 out).  All calls go through the C ABI."""
+import pytest
+import torch
+
+import oracle
+from oracle import oracle_torch
+from util import DTYPES, f32_from_bits, load_golden
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {"f32": 1e-3, "bf16": 1e-2, "f16": 1e-2}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import blockwise_int8_linear_amd as pkg
+    from blockwise_int8_linear_amd import _lib
+    _lib.load()
+    return pkg
+
+
+class cfg_as:
+    def __init__(self, ops, block=None, out=None):
+        self.cfg, self.block, self.out = ops.block_linear_config, block, out
+
+    def __enter__(self):
+        self.old = (self.cfg.GROUP_SIZE, self.cfg.INPUT_OUTPUT_TORCH_TYPE)
+        if self.block:
+            self.cfg.GROUP_SIZE = self.block
+        if self.out:
+            self.cfg.INPUT_OUTPUT_TORCH_TYPE = self.out
+
+    def __exit__(self, *a):
+        self.cfg.GROUP_SIZE, self.cfg.INPUT_OUTPUT_TORCH_TYPE = self.old
+
+
+def _codes(g, *shape):
+    return torch.randint(-127, 128, shape, generator=g, dtype=torch.int32).to(torch.int8)
+
+
+def _reference(A, W, sa, sw, B, bias, out_dtype):
+    """checker output and the magnitude sum_j |term_j| that bounds fp32 re-association error"""
+    P = oracle_torch.gemm_nt_partials(A, W, B)
+    ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw, B, bias, out_dtype)
+    mag = torch.zeros(P.shape[1:], dtype=torch.float64)
+    for j in range(P.shape[0]):
+        mag += P[j].abs().double() * sa[j].double()[:, None] * sw[j].double()[None, :]
+    return P, ref, mag / (127.0 * 127.0)
+
+
+def _assert_close(C, ref, mag, tol):
+    err = (C.double() - ref.double()).abs()
+    bound = tol * ref.double().abs() + 4e-6 * mag + 1e-30
+    if not (err <= bound).all():
+        i = (err - bound).argmax()
+        raise AssertionError(f"max violation at flat index {i.item()}: got {C.view(-1)[i].item()} want {ref.view(-1)[i].item()} "
+                             f"(err {err.view(-1)[i].item():.3e}, bound {bound.view(-1)[i].item():.3e})")
+
+
+def test_gemm_golden(ops):
+    for case in load_golden("kat_gemm.json"):
+        A = torch.tensor(case["A"], dtype=torch.int8)
+        W = torch.tensor(case["W"], dtype=torch.int8)
+        sa = torch.stack([f32_from_bits(r) for r in case["sa_bits"]])
+        sw = torch.stack([f32_from_bits(r) for r in case["sw_bits"]])
+        with cfg_as(ops, case["block"], torch.float32):
+            P = ops.int8_matmul_block_partials(A.to(DEV), W.to(DEV).t())
+            C = ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa.to(DEV), sw.to(DEV))
+        assert P.cpu().tolist() == case["P"]
+        exp = torch.tensor(case["C_f32"], dtype=torch.float64)
+        assert ((C.cpu().double() - exp).abs() <= 1e-5 * exp.abs() + 1e-12).all()
+
+
+# (M, N, K): ragged shapes from the reference's commented list (triton_functions.py:583-588), then shapes that
+# select each tile of the main kernel (K multiple of 128): 64x128, 128x128, 256x256
+SHAPES = [(253, 257, 234), (129, 266, 75), (389, 138, 45), (256, 512, 512), (1, 384, 256), (16, 1000, 1024),
+          (64, 128, 128), (100, 300, 384), (300, 500, 512), (1024, 512, 512), (3584, 3584, 256), (3500, 3700, 384)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("block", [32, 64, 128])
+def test_partials_bit_exact(ops, shape, block):
+    M, N, K = shape
+    g = torch.Generator().manual_seed(M + N + K + block)
+    A, W = _codes(g, M, K), _codes(g, N, K)
+    P = ops.int8_matmul_block_partials(A.to(DEV), W.to(DEV).t(), block)
+    ref = oracle_torch.gemm_nt_partials(A, W, block)
+    assert P.dtype == torch.int32 and P.shape == ref.shape
+    assert torch.equal(P.cpu(), ref)
+    if M * N * K <= 64 * 1024 * 1024:
+        assert torch.equal(ref, oracle.gemm_nt_partials(A, W, block, threads=True))
+
+
+def test_partials_saturated(ops):
+    A = torch.full((130, 256), 127, dtype=torch.int8)
+    W = torch.full((70, 256), -127, dtype=torch.int8)
+    P = ops.int8_matmul_block_partials(A.to(DEV), W.to(DEV).t(), 128)
+    assert (P == -128 * 127 * 127).all()
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("block", [32, 64, 128])
+@pytest.mark.parametrize("out", ["f32", "bf16"])
+def test_gemm_dequant_parity(ops, shape, block, out):
+    M, N, K = shape
+    g = torch.Generator().manual_seed(M * 3 + N + K + block)
+    A, W = _codes(g, M, K), _codes(g, N, K)
+    nblk = -(-K // block)
+    sa = torch.rand(nblk, M, generator=g) * 4 + 0.01
+    sw = torch.rand(nblk, N, generator=g) * 0.1 + 1e-4
+    bias = torch.randn(N, generator=g)
+    _, ref, mag = _reference(A, W, sa, sw, block, None, DTYPES[out])
+    with cfg_as(ops, block, DTYPES[out]):
+        Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
+        C = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sad, swd)
+        Cb = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sad, swd, bias.to(DEV))
+    assert C.dtype == DTYPES[out] and C.shape == (M, N)
+    _assert_close(C.cpu(), ref, mag, TOL[out])
+    # bias is added after the cast, in the output dtype (triton_functions.py:127-131): an exact identity
+    assert torch.equal(Cb, C + bias.to(DEV).to(DTYPES[out]))
+
+
+def test_gemm_fp16_out_and_bias_dtypes(ops):
+    g = torch.Generator().manual_seed(1)
+    M, N, K, B = 200, 260, 512, 128
+    A, W = _codes(g, M, K), _codes(g, N, K)
+    sa = torch.rand(K // B, M, generator=g); sw = torch.rand(K // B, N, generator=g) * 0.05
+    _, ref, mag = _reference(A, W, sa, sw, B, None, torch.float16)
+    with cfg_as(ops, B, torch.float16):
+        C = ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa.to(DEV), sw.to(DEV))
+        _assert_close(C.cpu(), ref, mag, TOL["f16"])
+        for bd in (torch.float32, torch.bfloat16, torch.float16):
+            bias = torch.randn(N, generator=g).to(bd)
+            Cb = ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa.to(DEV), sw.to(DEV), bias.to(DEV))
+            assert torch.equal(Cb, C + bias.to(DEV).to(torch.float16))
+
+
+def test_operand_layouts(ops):
+    """b given as a contiguous [K,N] tensor, operands that are column slices of wider buffers, misaligned views"""
+    g = torch.Generator().manual_seed(2)
+    M, N, K, B = 150, 200, 384, 128
+    Abig, Wbig = _codes(g, M, K + 64).to(DEV), _codes(g, N, K + 48).to(DEV)
+    sa = torch.rand(K // B, M, generator=g).to(DEV); sw = torch.rand(K // B, N, generator=g).to(DEV)
+    with cfg_as(ops, B, torch.float32):
+        A, W = Abig[:, 16:16 + K], Wbig[:, 32:32 + K]                        # aligned starts, ld > K
+        base = ops.int8_matmul_block64_rowwise_dequantize(A.contiguous(), W.contiguous().t(), sa, sw)
+        assert torch.equal(ops.int8_matmul_block64_rowwise_dequantize(A, W.t(), sa, sw), base)
+        assert torch.equal(ops.int8_matmul_block64_rowwise_dequantize(A, W.t().contiguous(), sa, sw), base)
+        A2, W2 = Abig[:, 3:3 + K], Wbig[:, 5:5 + K]                          # misaligned -> fallback kernel
+        ref = ops.int8_matmul_block64_rowwise_dequantize(A2.contiguous(), W2.contiguous().t(), sa, sw)
+        got = ops.int8_matmul_block64_rowwise_dequantize(A2, W2.t(), sa, sw)
+        assert torch.allclose(got, ref, rtol=1e-5, atol=1e-6)
+        with pytest.raises(AssertionError, match="incompatible dimensions"):
+            ops.int8_matmul_block64_rowwise_dequantize(A, W[:, :-1].t(), sa, sw)
+
+
+def test_end_to_end_vs_dense_config1(ops):
+    """X fp32 [256,1024] ~N(0,1); W fp32 [1024,1024] ~N(0,0.02); block 64; fp32 out, compared to the fp32
+    matmul and to the checker's forward."""
+    g = torch.Generator().manual_seed(0)
+    X = torch.randn(256, 1024, generator=g); W = torch.randn(1024, 1024, generator=g) * 0.02
+    with cfg_as(ops, 64, torch.float32):
+        xq, sx = ops.quantize_block_rowwise(X.to(DEV))
+        wq, sw = ops.quantize_block_rowwise(W.to(DEV))
+        out = ops.int8_matmul_block64_rowwise_dequantize(xq, wq.t(), sx, sw)
+        P = ops.int8_matmul_block_partials(xq, wq.t())
+    xqo, sxo = oracle.quantize_block_rowwise(X, 64); wqo, swo = oracle.quantize_block_rowwise(W, 64)
+    assert torch.equal(xq.cpu(), xqo) and torch.equal(wq.cpu(), wqo) and torch.equal(sx.cpu(), sxo) and torch.equal(sw.cpu(), swo)
+    Pref, ref, mag = _reference(xqo, wqo, sxo, swo, 64, None, torch.float32)
+    assert torch.equal(P.cpu(), Pref)
+    _assert_close(out.cpu(), ref, mag, 1e-3)
+    dense = X @ W.t()
+    rel = (out.cpu() - dense).norm() / dense.norm()
+    assert 1e-3 < rel < 3e-2
+
+
+@pytest.mark.parametrize("block", [128])
+def test_headline_shape_8192(ops, block):
+    """M=N=K=8192, bf16 out.  Too big for the scalar checker, so: (i) 96 sampled rows and 96 sampled columns
+    against the checker, (ii) every block partial of a 256x256 corner bit-exact, (iii) the result of a row
+    subset equals the same rows of the full result (tiles are independent)."""
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(8192, 8192, generator=g).to(torch.bfloat16)
+    w = (torch.randn(8192, 8192, generator=g) * 0.02).to(torch.bfloat16)
+    with cfg_as(ops, block, torch.bfloat16):
+        xq, sx = ops.quantize_block_rowwise(x.to(DEV))
+        wq, sw = ops.quantize_block_rowwise(w.to(DEV))
+        C = ops.int8_matmul_block64_rowwise_dequantize(xq, wq.t(), sx, sw)
+        rows = torch.randperm(8192, generator=g)[:96]
+        cols = torch.randperm(8192, generator=g)[:96]
+        xq_c, wq_c, sx_c, sw_c = xq.cpu(), wq.cpu(), sx.cpu(), sw.cpu()
+        _, ref, mag = _reference(xq_c[rows], wq_c, sx_c[:, rows].contiguous(), sw_c, block, None, torch.bfloat16)
+        _assert_close(C[rows.to(DEV)].cpu(), ref, mag, 1e-2)
+        _, ref, mag = _reference(xq_c, wq_c[cols], sx_c, sw_c[:, cols].contiguous(), block, None, torch.bfloat16)
+        _assert_close(C[:, cols.to(DEV)].cpu(), ref, mag, 1e-2)
+        sub = ops.int8_matmul_block64_rowwise_dequantize(xq[4096:4096 + 512], wq.t(), sx[:, 4096:4096 + 512].contiguous(), sw)
+        assert torch.equal(sub, C[4096:4096 + 512])
+        P = ops.int8_matmul_block_partials(xq[-256:], wq[-256:].t())
+    assert torch.equal(P.cpu(), oracle_torch.gemm_nt_partials(xq_c[-256:], wq_c[-256:], block))
+    dense = (x[rows].float() @ w.float().t())
+    rel = (C[rows.to(DEV)].cpu().float() - dense).norm() / dense.norm()
+    assert rel < 3e-2
