@@ -1,0 +1,178 @@
+"""Benchmark of the blockwise int8 hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (the configuration the headline metric is quoted on): int8 block GEMM with fused dequantize at
+M = N = K = 8192, block 128, bf16 out, operands = block-quantized bf16 N(0,1) activations and 0.02*N(0,1)
+weights (seed 0), already resident in HBM; next to it the block quantize -> dequantize round trip of a bf16
+[8192,8192] tensor with 0.1% x50 outliers at blocks 32/64/128.  A "step" is one GEMM launch through the
+drop-in operator.  Prints ONE JSON line.
+
+Kernel durations are measured with HIP events recorded on the stream the kernels are launched on (torch's
+current stream), around runs of back-to-back launches.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+INT8_PEAK_TOPS = 5033.2        # 256 CUs x 8192 int8 ops/clk/CU x 2.4 GHz (AMD quotes 5.0 POP/s dense)
+HBM_PEAK_GBS = 8000.0          # HBM3E, 8 TB/s
+
+
+def event_ms(fn, iters: int) -> float:
+    """average duration of one `fn()` launch: `iters` back-to-back launches between two events"""
+    import torch
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def bench_quantize(pkg, torch, iters: int):
+    """block quantize / dequantize of bf16 [8192,8192] with outliers, through the C ABI with preallocated outputs"""
+    from blockwise_int8_linear_amd import _lib
+    lib = _lib.load()
+    M = K = 8192
+    E = M * K
+    gen = torch.Generator(device="cuda").manual_seed(0)
+    x = torch.randn(M, K, device="cuda", generator=gen, dtype=torch.float32)
+    gen1 = torch.Generator(device="cuda").manual_seed(1)
+    pos = torch.randint(0, E, (E // 1000,), device="cuda", generator=gen1)
+    x.view(-1)[pos] *= 50.0
+    x = x.to(torch.bfloat16)
+    st = torch.cuda.current_stream().cuda_stream
+    out = {}
+    for B in (32, 64, 128):
+        q = torch.empty(M, K, device="cuda", dtype=torch.int8)
+        s = torch.empty(K // B, M, device="cuda", dtype=torch.float32)
+        d = torch.empty(M, K, device="cuda", dtype=torch.bfloat16)
+
+        def fq():
+            rc = lib.bi8_quantize_rowwise(x.data_ptr(), 1, q.data_ptr(), s.data_ptr(), M, K, K, K, B, st)
+            assert rc == 0
+
+        def fd():
+            rc = lib.bi8_dequantize_rowwise(q.data_ptr(), s.data_ptr(), d.data_ptr(), 1, M, K, K, K, B, st)
+            assert rc == 0
+
+        for f in (fq, fd):
+            for _ in range(5):
+                f()
+        torch.cuda.synchronize()
+        tq = min(event_ms(fq, iters) for _ in range(3))
+        td = min(event_ms(fd, iters) for _ in range(3))
+        nbytes = E * 3 + 4 * E // B                 # read 2 B + write 1 B per element (or the reverse) + scales
+        mse = ((d.float() - x.float()) ** 2).mean().item()
+        out[f"block{B}"] = {
+            "bytes": nbytes,
+            "quantize_us": round(tq * 1e3, 2), "quantize_GBps": round(nbytes / tq / 1e6, 1),
+            "quantize_frac_hbm": round(nbytes / tq / 1e6 / HBM_PEAK_GBS, 4),
+            "dequantize_us": round(td * 1e3, 2), "dequantize_GBps": round(nbytes / td / 1e6, 1),
+            "dequantize_frac_hbm": round(nbytes / td / 1e6 / HBM_PEAK_GBS, 4),
+            "roundtrip_mse": mse,
+        }
+    return out
+
+
+def cpu_baseline(torch, xq_rows, wq, sx_rows, sw, B, budget_s: float = 20.0):
+    """the PyTorch CPU restatement of the reference math (oracle/oracle_torch.py) on a bounded row sample of the
+    same GEMM, on this host's cores"""
+    from oracle import oracle_torch
+    rows = xq_rows.shape[0]
+    N, K = wq.shape
+    t0 = time.perf_counter()
+    oracle_torch.int8_matmul_block_dequantize(xq_rows, wq, sx_rows, sw, B, None, torch.bfloat16)
+    dt = time.perf_counter() - t0
+    return {
+        "value": round(2.0 * rows * N * K / dt / 1e12, 4), "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"oracle/oracle_torch.py (PyTorch eager, fp32 bmm per K-block + fp32 rescale) on the first {rows} rows of the "
+                  f"same 8192^3 problem: {rows}x{N}x{K}, block {B}, bf16 out; {dt:.2f} s on {torch.get_num_threads()} threads "
+                  f"({os.cpu_count()} logical CPUs)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--size", type=int, default=8192, help="M = N = K of the GEMM (the metric is quoted at 8192)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-quantize", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build is a one-GPU path (no collectives, no sharding); run it with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import blockwise_int8_linear_amd as pkg
+    from blockwise_int8_linear_amd import _lib
+    _lib.load()                                     # fails loudly if libbi8.so is not built
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    torch.cuda.set_device(0)
+    cfg = pkg.block_linear_config
+    B = cfg.GROUP_SIZE
+    assert B == 128 and cfg.INPUT_OUTPUT_TORCH_TYPE == torch.bfloat16
+    S = args.size
+
+    torch.manual_seed(0)
+    x = torch.randn(S, S, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn(S, S, device="cuda", dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    xq, sx = pkg.quantize_block_rowwise(x)
+    wq, sw = pkg.quantize_block_rowwise(w)
+    wqt = wq.t()
+    del x, w
+
+    def step():
+        return pkg.int8_matmul_block64_rowwise_dequantize(xq, wqt, sx, sw)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    ops_per_launch = 2.0 * S * S * S
+    kern_ms = min(event_ms(step, max(args.steps // 2, 5)) for _ in range(3))
+    achieved = ops_per_launch / kern_ms / 1e9       # TOPS
+
+    res = {
+        "metric": "int8 block GEMM TOPS (% int8 MFMA peak) at 8192^3; quantize GB/s (% HBM)",
+        "value": round(ops_per_launch / wall_ms / 1e9, 2), "unit": "TOPS",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": f"int8 block GEMM + fused dequantize, M=N=K={S}, block {B}, bf16 out; A = quantize(bf16 N(0,1)), "
+                               f"W = quantize(bf16 0.02*N(0,1)), seed 0; one launch per step via "
+                               f"int8_matmul_block64_rowwise_dequantize",
+                   "block": B, "out_dtype": "bf16"},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": None,
+                     "kernel": "gemm_tile<256,256,4,2,128,bf16>", "ops_per_launch": ops_per_launch,
+                     "avg_launch_ms": round(kern_ms, 4)},
+    }
+    if not args.no_quantize:
+        res["quantize_roundtrip"] = bench_quantize(pkg, torch, 50)
+    if not args.no_cpu_baseline:
+        rows = min(2048, S)
+        res["cpu_baseline"] = cpu_baseline(torch, xq[:rows].cpu(), wq.cpu(), sx[:, :rows].contiguous().cpu(), sw.cpu(), B)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

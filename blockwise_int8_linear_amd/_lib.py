@@ -9,7 +9,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libbi8.so")
+# BI8_LIBRARY overrides the location of the shared object (e.g. an experimental build)
+LIB_PATH = os.environ.get("BI8_LIBRARY") or os.path.join(_HERE, "libbi8.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "bi8.h")
 ABI_VERSION = 1
 

@@ -15,6 +15,8 @@
 //     compact patch of output tiles.
 // Shapes the main kernel cannot take (K not a multiple of 128, rows not 16-byte aligned, other block
 // sizes) go to gemm_generic: same MFMA, operands gathered straight from global memory with byte loads.
+#include <type_traits>
+
 #include "bi8_common.h"
 
 namespace {
@@ -71,26 +73,37 @@ __device__ __forceinline__ float load_bias(const GemmArgs &g, int64_t n) {
     return bi8_from_f16_bits(((const uint16_t *)g.bias)[n]);
 }
 
-// BM x BN output tile per workgroup, WM x WN waves, BLK = quantization block (32, 64 or 128).
+// LDS map of gemm_tile: operand regions first, each with two stage buffers, so that every ds_read of the
+// main loop is "per-lane base register + immediate".
+template <int BM, int BN, int BLK> struct TileLds {
+    static constexpr int NBS = kStageK / BLK;        // K-blocks per stage
+    static constexpr int kABuf = BM * kStageK, kWBuf = BN * kStageK;
+    static constexpr int kSABuf = NBS * BM * 4, kSWBuf = NBS * BN * 4;
+    static constexpr int kAReg = 0;
+    static constexpr int kWReg = kAReg + 2 * kABuf;
+    static constexpr int kSAReg = kWReg + 2 * kWBuf;
+    static constexpr int kSWReg = kSAReg + 2 * kSABuf;
+    static constexpr int kBytes = kSWReg + 2 * kSWBuf;
+};
+
+// BM x BN output tile per workgroup, WM x WN waves (each TM x TN subtiles of 32x32), BLK = quantization block.
 template <int BM, int BN, int WM, int WN, int BLK, int CDT, bool PARTIALS>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
+    using L = TileLds<BM, BN, BLK>;
     constexpr int NW = WM * WN;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int NBS = kStageK / BLK;             // K-blocks per stage
+    constexpr int NBS = L::NBS;
     constexpr int KSB = BLK / 32;                  // MFMA k-steps per K-block
-    constexpr int kAOff = 0;
-    constexpr int kWOff = BM * kStageK;
-    constexpr int kSAOff = (BM + BN) * kStageK;
-    constexpr int kSWOff = kSAOff + NBS * BM * 4;
-    constexpr int kStageBytes = kSWOff + NBS * BN * 4;
+    constexpr int NSUB = TM * TN;
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
     static_assert(BM % 64 == 0 && BN % 64 == 0, "scale rows are loaded 64 floats per wave instruction");
+    static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "operand rows split evenly over the waves");
 
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, h = lane >> 5;
 
@@ -98,15 +111,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
     tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
     const int nstages = (int)(g.K / kStageK);
-    const int64_t nblk = g.K / BLK;
 
-    // ---- loader: this lane's source rows (clamped into the matrix) and swizzled source chunk ----
-    // wave-instruction i covers tile rows 8i .. 8i+7; lane -> (row 8i + lane/8, LDS chunk lane%8),
-    // which holds source chunk (lane%8) ^ (lane/8).
+    // ---- loader state: per-lane source pointers, advanced by one stage after every issue ----
+    // wave-instruction i covers tile rows 8i .. 8i+7; lane -> (row 8i + lane/8, LDS chunk lane%8), which
+    // holds source chunk (lane%8) ^ (lane/8).  Rows outside the matrix are clamped to its last row.
     const int ld_row = lane >> 3;
     const int ld_chunk = (lane & 7) ^ ld_row;
-    constexpr int kAInstr = BM / 8, kWInstr = BN / 8;
-    constexpr int kAIter = (kAInstr + NW - 1) / NW, kWIter = (kWInstr + NW - 1) / NW;
+    constexpr int kAIter = BM / 8 / NW, kWIter = BN / 8 / NW;
     const int8_t *a_src[kAIter];
     const int8_t *w_src[kWIter];
 #pragma unroll
@@ -121,52 +132,67 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
         if (r > g.N - 1) r = g.N - 1;
         w_src[it] = g.W + r * g.ldw + ld_chunk * 16;
     }
-    // scale rows: 64 floats per wave instruction; instruction i < BM/64 -> sA, else sW (per K-block of the stage)
-    constexpr int kSAInstr = BM / 64, kSWInstr = BN / 64;
-    int64_t sa_col = m0 + lane, sw_col = n0 + lane;
+    // scale rows: 64 floats per wave instruction; instruction i -> K-block i / kSPer of the stage, and inside
+    // it the first BM/64 instructions fetch sA, the rest sW
+    constexpr int kSPer = BM / 64 + BN / 64;
+    constexpr int kSInstr = PARTIALS ? 0 : NBS * kSPer;
+    constexpr int kSIter = (kSInstr + NW - 1) / NW;
+    const float *s_src[kSIter > 0 ? kSIter : 1];
+    int s_dst[kSIter > 0 ? kSIter : 1];
+    int64_t s_step[kSIter > 0 ? kSIter : 1];
+#pragma unroll
+    for (int it = 0; it < kSIter; ++it) {
+        const int i = wave + it * NW;
+        const int b = i / kSPer, r = i % kSPer;
+        if (r < BM / 64) {
+            int64_t m = m0 + r * 64 + lane;
+            if (m > g.M - 1) m = g.M - 1;
+            s_src[it] = g.sA + (int64_t)b * g.M + m;
+            s_dst[it] = L::kSAReg + (b * BM + r * 64) * 4;
+            s_step[it] = (int64_t)NBS * g.M;
+        } else {
+            int64_t n = n0 + (r - BM / 64) * 64 + lane;
+            if (n > g.N - 1) n = g.N - 1;
+            s_src[it] = g.sW + (int64_t)b * g.N + n;
+            s_dst[it] = L::kSWReg + (b * BN + (r - BM / 64) * 64) * 4;
+            s_step[it] = (int64_t)NBS * g.N;
+        }
+    }
 
-    auto issue_stage = [&](int s, int buf) {
-        uint8_t *base = lds + buf * kStageBytes;
-        const int64_t k0 = (int64_t)s * kStageK;
+    auto issue_stage = [&](int buf) {             // buf is wave-uniform: the LDS destinations are scalars
 #pragma unroll
         for (int it = 0; it < kAIter; ++it) {
-            const int i = wave + it * NW;
-            if (kAInstr % NW == 0 || i < kAInstr) lds_dma16(a_src[it] + k0, base + kAOff + i * 1024);
+            lds_dma16(a_src[it], lds + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024);
+            a_src[it] += kStageK;
         }
 #pragma unroll
         for (int it = 0; it < kWIter; ++it) {
-            const int i = wave + it * NW;
-            if (kWInstr % NW == 0 || i < kWInstr) lds_dma16(w_src[it] + k0, base + kWOff + i * 1024);
+            lds_dma16(w_src[it], lds + L::kWReg + buf * L::kWBuf + (wave + it * NW) * 1024);
+            w_src[it] += kStageK;
         }
-        if constexpr (!PARTIALS) {
-            constexpr int kSInstr = NBS * (kSAInstr + kSWInstr);
 #pragma unroll
-            for (int it = 0; it < (kSInstr + NW - 1) / NW; ++it) {
-                const int i = wave + it * NW;
-                if (i < kSInstr) {
-                    const int b = i / (kSAInstr + kSWInstr);
-                    const int r = i % (kSAInstr + kSWInstr);
-                    const int64_t jb = (int64_t)s * NBS + b;
-                    if (r < kSAInstr) {
-                        int64_t m = sa_col + r * 64;
-                        if (m > g.M - 1) m = g.M - 1;
-                        lds_dma4(g.sA + jb * g.M + m, base + kSAOff + (b * BM + r * 64) * 4);
-                    } else {
-                        int64_t n = sw_col + (r - kSAInstr) * 64;
-                        if (n > g.N - 1) n = g.N - 1;
-                        lds_dma4(g.sW + jb * g.N + n, base + kSWOff + (b * BN + (r - kSAInstr) * 64) * 4);
-                    }
-                }
+        for (int it = 0; it < kSIter; ++it) {
+            const int i = wave + it * NW;
+            if (i < kSInstr) {
+                const bool is_a = (i % kSPer) < BM / 64;
+                lds_dma4(s_src[it], lds + s_dst[it] + buf * (is_a ? L::kSABuf : L::kSWBuf));
+                s_src[it] += s_step[it];
             }
         }
     };
 
-    // ---- operand fragment addresses: row r = ... + l32, chunk (2*ks + h) ^ (r & 7) ----
+    // ---- operand fragment addresses of the buffer being computed.  Row r = ... + l32, 16-byte chunk
+    // (2*ks + h) ^ (r & 7): address(ks) = base ^ (ks << 5).  One register per ks; subtile offsets are immediates.
     const int frag_sw = ((h ^ (lane & 7)) << 4);
-    const int a_frag = kAOff + (wm * (BM / WM) + l32) * kStageK + frag_sw;
-    const int w_frag = kWOff + (wn * (BN / WN) + l32) * kStageK + frag_sw;
-    const int sa_frag = kSAOff + (wm * (BM / WM) + 4 * h) * 4;
-    const int sw_frag = kSWOff + (wn * (BN / WN) + l32) * 4;
+    int a_addr[4], w_addr[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        a_addr[ks] = (L::kAReg + (wm * (BM / WM) + l32) * kStageK + frag_sw) ^ (ks << 5);
+        w_addr[ks] = (L::kWReg + (wn * (BN / WN) + l32) * kStageK + frag_sw) ^ (ks << 5);
+    }
+    int sa_addr = L::kSAReg + (wm * (BM / WM) + 4 * h) * 4;
+    int sw_addr = L::kSWReg + (wn * (BN / WN) + l32) * 4;
+    int flip = 1;                                  // +1: the next stage is in buffer 1, -1: in buffer 0
 
     float acc[TM][TN][16];
 #pragma unroll
@@ -176,74 +202,123 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
 
-    auto compute_stage = [&](int s, int buf) {
-        const uint8_t *base = lds + buf * kStageBytes;
-        bi8_v4i af[TM][4], wf[TN][4];
+    // The last subtile of a stage is folded into the accumulator during the first MFMAs of the NEXT stage
+    // (after the barrier, while the new operands are still on their way from LDS).
+    bi8_v16i pend_p = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    bi8_v4f pend_sx[4];
 #pragma unroll
-        for (int a = 0; a < TM; ++a)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) af[a][ks] = *(const bi8_v4i *)(base + ((a_frag + a * 32 * kStageK) ^ (ks << 5)));
-#pragma unroll
-        for (int b = 0; b < TN; ++b)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) wf[b][ks] = *(const bi8_v4i *)(base + ((w_frag + b * 32 * kStageK) ^ (ks << 5)));
+    for (int i = 0; i < 4; ++i) pend_sx[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    float pend_sw = 0.0f;
 
+    auto fold = [&](const bi8_v16i &pt, const bi8_v4f *sx, float sw, float *dst) {
 #pragma unroll
-        for (int blk = 0; blk < NBS; ++blk) {
-            float swv[TN];
-            if constexpr (!PARTIALS) {
-#pragma unroll
-                for (int b = 0; b < TN; ++b) swv[b] = *(const float *)(base + sw_frag + (blk * BN + b * 32) * 4);
-            }
-#pragma unroll
-            for (int a = 0; a < TM; ++a) {
-                bi8_v4f sxv[4];
-                if constexpr (!PARTIALS) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) sxv[i] = *(const bi8_v4f *)(base + sa_frag + (blk * BM + a * 32 + 8 * i) * 4);
-                }
-#pragma unroll
-                for (int b = 0; b < TN; ++b) {
-                    bi8_v16i p = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-                    for (int ks = 0; ks < KSB; ++ks)
-                        p = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a][blk * KSB + ks], wf[b][blk * KSB + ks], p, 0, 0, 0);
-                    if constexpr (PARTIALS) {
-                        const int64_t jb = (int64_t)s * NBS + blk;
-                        const int64_t n = n0 + wn * (BN / WN) + b * 32 + l32;
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const int64_t m = m0 + wm * (BM / WM) + a * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                            if (m < g.M && n < g.N) g.P[(jb * g.M + m) * g.N + n] = p[r];
-                        }
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            const float t = (float)p[r] * sxv[r >> 2][r & 3];
-                            acc[a][b][r] = __builtin_fmaf(t, swv[b], acc[a][b][r]);
-                        }
-                    }
-                }
-            }
+        for (int r = 0; r < 16; ++r) {
+            const float f = (float)pt[r] * sx[r >> 2][r & 3];
+            dst[r] = __builtin_fmaf(f, sw, dst[r]);
         }
     };
 
-    issue_stage(0, 0);
-    for (int s = 0; s < nstages; ++s) {
+    // One stage = NBS K-blocks x NSUB subtiles ("items").  The MFMAs of item t are issued before the fp32
+    // fold of item t-1, so the matrix pipe works while the vector ALU converts and accumulates.
+    auto compute_stage = [&](int s) {
+        bi8_v4i af[TM][4], wf[TN][4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int a = 0; a < TM; ++a) af[a][ks] = *(const bi8_v4i *)(lds + a_addr[ks] + a * 32 * kStageK);
+#pragma unroll
+            for (int b = 0; b < TN; ++b) wf[b][ks] = *(const bi8_v4i *)(lds + w_addr[ks] + b * 32 * kStageK);
+        }
+        float swv[2][TN];
+        bi8_v4f sxv[2][TM][4];
+        auto load_scales = [&](int blk) {
+#pragma unroll
+            for (int b = 0; b < TN; ++b) swv[blk & 1][b] = *(const float *)(lds + sw_addr + (blk * BN + b * 32) * 4);
+#pragma unroll
+            for (int a = 0; a < TM; ++a)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) sxv[blk & 1][a][i] = *(const bi8_v4f *)(lds + sa_addr + (blk * BM + a * 32 + 8 * i) * 4);
+        };
+        auto chain = [&](int t) {
+            const int blk = t / NSUB, a = (t % NSUB) / TN, b = t % TN;
+            bi8_v16i acc_i = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < KSB; ++ks)
+                acc_i = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a][blk * KSB + ks], wf[b][blk * KSB + ks], acc_i, 0, 0, 0);
+            return acc_i;
+        };
+        constexpr int NITEM = NBS * NSUB;
+        if constexpr (PARTIALS) {
+#pragma unroll
+            for (int t = 0; t < NITEM; ++t) {
+                const int blk = t / NSUB, a = (t % NSUB) / TN, b = t % TN;
+                const bi8_v16i pt = chain(t);
+                const int64_t jb = (int64_t)s * NBS + blk;
+                const int64_t n = n0 + wn * (BN / WN) + b * 32 + l32;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int64_t m = m0 + wm * (BM / WM) + a * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+                    if (m < g.M && n < g.N) g.P[(jb * g.M + m) * g.N + n] = pt[r];
+                }
+            }
+        } else {
+            bi8_v16i p[2];
+#pragma unroll
+            for (int t = 0; t < NITEM; ++t) {
+                const int blk = t / NSUB;
+                if (t % NSUB == 0) load_scales(blk);
+                p[t & 1] = chain(t);
+                if (t == 0) {
+                    fold(pend_p, pend_sx, pend_sw, acc[TM - 1][TN - 1]);
+                } else {
+                    const int u = t - 1, ub = u / NSUB, ua = (u % NSUB) / TN, un = u % TN;
+                    fold(p[u & 1], sxv[ub & 1][ua], swv[ub & 1][un], acc[ua][un]);
+                }
+#pragma unroll
+                for (int ks = 0; ks < KSB; ++ks) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA of item t
+                    __builtin_amdgcn_sched_group_barrier(0x002, 48 / KSB, 0);       // a slice of item t-1's fold
+                }
+            }
+            pend_p = p[(NITEM - 1) & 1];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pend_sx[i] = sxv[(NBS - 1) & 1][TM - 1][i];
+            pend_sw = swv[(NBS - 1) & 1][TN - 1];
+        }
+        // point the fragment addresses at the other buffer
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            a_addr[ks] += flip * L::kABuf;
+            w_addr[ks] += flip * L::kWBuf;
+        }
+        sa_addr += flip * L::kSABuf;
+        sw_addr += flip * L::kSWBuf;
+        flip = -flip;
+    };
+
+    issue_stage(0);
+    int fill = 1;
+    for (int s = 0; s + 1 < nstages; ++s) {
         __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): this wave's direct-to-LDS loads have landed
         __syncthreads();                           // ... and everyone's; the other buffer is free again
-        if (s + 1 < nstages) issue_stage(s + 1, (s + 1) & 1);
-        compute_stage(s, s & 1);
+        issue_stage(fill);
+        fill ^= 1;
+        compute_stage(s);
     }
-    (void)nblk;
+    if (nstages > 0) {
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        compute_stage(nstages - 1);
+    }
+    if constexpr (!PARTIALS) fold(pend_p, pend_sx, pend_sw, acc[TM - 1][TN - 1]);
 
     if constexpr (!PARTIALS) {
         const float div = (float)(1.0 / (127.0 * 127.0));
+        const bool has_bias = g.bias != nullptr;
 #pragma unroll
         for (int b = 0; b < TN; ++b) {
             const int64_t n = n0 + wn * (BN / WN) + b * 32 + l32;
             const bool n_ok = n < g.N;
-            const bool has_bias = g.bias != nullptr;
             const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
 #pragma unroll
             for (int a = 0; a < TM; ++a)
@@ -323,9 +398,7 @@ __global__ __launch_bounds__(256) void gemm_generic(const GemmArgs g, int block)
 
 template <int BM, int BN, int WM, int WN, int BLK, int CDT, bool PARTIALS>
 int launch_tile(GemmArgs g, hipStream_t st) {
-    constexpr int NBS = kStageK / BLK;
-    constexpr int kStageBytes = (BM + BN) * kStageK + NBS * (BM + BN) * 4;
-    constexpr int kLds = 2 * kStageBytes;
+    constexpr int kLds = TileLds<BM, BN, BLK>::kBytes;
     const int64_t tm = (g.M + BM - 1) / BM, tn = (g.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     g.tiles_m = (int)tm;
@@ -350,10 +423,15 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
 
 // tile shape by problem shape: the big tile when there is enough work to fill 256 CUs with it
 template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipStream_t st) {
-    const int64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256);
-    if (g.M > 128 && big >= 192) return launch_tile<256, 256, 4, 2, BLK, CDT, PARTIALS>(g, st);
+#ifdef BI8_FORCE_TILE
+    if (BI8_FORCE_TILE == 0) return launch_tile<256, 128, 4, 2, BLK, CDT, PARTIALS>(g, st);
+    if (BI8_FORCE_TILE == 1) return launch_tile<128, 128, 2, 2, BLK, CDT, PARTIALS>(g, st);
+    if (BI8_FORCE_TILE == 2) return launch_tile<64, 128, 1, 2, BLK, CDT, PARTIALS>(g, st);
+#endif
+    const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
+    if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, BLK, CDT, PARTIALS>(g, st);
     if (g.M > 64) return launch_tile<128, 128, 2, 2, BLK, CDT, PARTIALS>(g, st);
-    return launch_tile<64, 128, 1, 4, BLK, CDT, PARTIALS>(g, st);
+    return launch_tile<64, 128, 1, 2, BLK, CDT, PARTIALS>(g, st);
 }
 
 template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hipStream_t st) {
