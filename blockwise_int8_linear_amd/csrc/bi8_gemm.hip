@@ -9,8 +9,8 @@
 //     registers, converted and folded into an fp32 accumulator as soon as the block's MFMAs are issued;
 //   - A and W tiles (128 bytes of K per row per stage) and the stage's scale rows go HBM -> LDS directly
 //     (global_load_lds, 16 bytes per lane), two stages in flight, one barrier per stage;
-//   - LDS rows are 128 bytes with the 16-byte chunk index XOR-ed with (row & 7), which makes both the
-//     direct-to-LDS writes and the MFMA operand reads (ds_read_b128) conflict-free;
+//   - LDS rows are 128 bytes with the 16-byte chunk index XOR-ed with ((row >> 1) & 7): 16 consecutive rows of
+//     one chunk column cover all 64 banks, so the MFMA operand reads (ds_read_b128) run at full LDS rate;
 //   - the workgroup index is remapped so that the 32 workgroups resident on one XCD (one L2) cover a
 //     compact patch of output tiles.
 // Shapes the main kernel cannot take (K not a multiple of 128, rows not 16-byte aligned, other block
@@ -23,13 +23,19 @@ namespace {
 
 constexpr int kStageK = 128;       // bytes of K per LDS stage
 
-__device__ __forceinline__ void lds_dma16(const void *gsrc, void *lds_dst) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gsrc,
-                                     (__attribute__((address_space(3))) void *)lds_dst, 16, 0, 0);
+// Raw buffer resource over [base, base + bytes): loads beyond the end return zeros.
+typedef __amdgpu_buffer_rsrc_t bi8_rsrc;
+__device__ __forceinline__ bi8_rsrc bi8_make_rsrc(const void *base, int64_t bytes) {
+    const int n = bytes > 0x7fffffffLL ? 0x7fffffff : (int)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, n, 0x00020000);
 }
-__device__ __forceinline__ void lds_dma4(const void *gsrc, void *lds_dst) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gsrc,
-                                     (__attribute__((address_space(3))) void *)lds_dst, 4, 0, 0);
+// 64 lanes x 16 (or 4) bytes from buffer offset voff + soff to LDS at lds_dst + lane * 16 (or 4); lds_dst and
+// soff are wave-uniform.
+__device__ __forceinline__ void bi8_buffer_to_lds16(bi8_rsrc r, void *lds_dst, uint32_t voff, uint32_t soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_dst, 16, voff, soff, 0, 0);
+}
+__device__ __forceinline__ void bi8_buffer_to_lds4(bi8_rsrc r, void *lds_dst, uint32_t voff, uint32_t soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_dst, 4, voff, soff, 0, 0);
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs.  Give XCD x the x-th contiguous eighth of a
@@ -73,23 +79,25 @@ __device__ __forceinline__ float load_bias(const GemmArgs &g, int64_t n) {
     return bi8_from_f16_bits(((const uint16_t *)g.bias)[n]);
 }
 
-// LDS map of gemm_tile: operand regions first, each with two stage buffers, so that every ds_read of the
-// main loop is "per-lane base register + immediate".
-template <int BM, int BN, int BLK> struct TileLds {
+// LDS map of gemm_tile: one region per operand, each a ring of kBufs stage buffers.
+template <int BM, int BN, int BLK, int NBUF> struct TileLds {
+    static constexpr int kBufs = NBUF;
     static constexpr int NBS = kStageK / BLK;        // K-blocks per stage
     static constexpr int kABuf = BM * kStageK, kWBuf = BN * kStageK;
     static constexpr int kSABuf = NBS * BM * 4, kSWBuf = NBS * BN * 4;
     static constexpr int kAReg = 0;
-    static constexpr int kWReg = kAReg + 2 * kABuf;
-    static constexpr int kSAReg = kWReg + 2 * kWBuf;
-    static constexpr int kSWReg = kSAReg + 2 * kSABuf;
-    static constexpr int kBytes = kSWReg + 2 * kSWBuf;
+    static constexpr int kWReg = kAReg + kBufs * kABuf;
+    static constexpr int kSAReg = kWReg + kBufs * kWBuf;
+    static constexpr int kSWReg = kSAReg + kBufs * kSABuf;
+    static constexpr int kBytes = kSWReg + kBufs * kSWBuf;
+    static constexpr bool kFits = kBytes <= 160 * 1024;   // LDS per CU
 };
 
 // BM x BN output tile per workgroup, WM x WN waves (each TM x TN subtiles of 32x32), BLK = quantization block.
-template <int BM, int BN, int WM, int WN, int BLK, int CDT, bool PARTIALS>
+template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
 __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
-    using L = TileLds<BM, BN, BLK>;
+    using L = TileLds<BM, BN, BLK, NBUF>;
+    constexpr int kBufs = NBUF;
     constexpr int NW = WM * WN;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int NBS = L::NBS;
@@ -112,87 +120,85 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
     const int nstages = (int)(g.K / kStageK);
 
-    // ---- loader state: per-lane source pointers, advanced by one stage after every issue ----
+    // ---- loader: buffer loads straight into LDS.  One buffer resource per operand, based at this tile's
+    // first row and sized to the end of the matrix, so rows past the edge read as zeros; a 32-bit per-lane
+    // offset per wave instruction (constant over the K loop) and the K position in a scalar register.
     // wave-instruction i covers tile rows 8i .. 8i+7; lane -> (row 8i + lane/8, LDS chunk lane%8), which
-    // holds source chunk (lane%8) ^ (lane/8).  Rows outside the matrix are clamped to its last row.
+    // holds source chunk (lane%8) ^ ((row >> 1) & 7).  Every wave's instruction indices i = wave + it*NW have
+    // the parity of `wave` (NW is even), so (row >> 1) & 7 = (4 * (wave & 1) + lane/16) & 7.
+    static_assert(NW % 2 == 0, "swizzle term must not depend on the iteration");
     const int ld_row = lane >> 3;
-    const int ld_chunk = (lane & 7) ^ ld_row;
+    const int ld_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
     constexpr int kAIter = BM / 8 / NW, kWIter = BN / 8 / NW;
-    const int8_t *a_src[kAIter];
-    const int8_t *w_src[kWIter];
+    const int64_t a_rows = (g.M - m0 < BM) ? (g.M - m0) : BM, w_rows = (g.N - n0 < BN) ? (g.N - n0) : BN;
+    const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
+    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
+    uint32_t a_off[kAIter], w_off[kWIter];
 #pragma unroll
-    for (int it = 0; it < kAIter; ++it) {
-        int64_t r = m0 + (wave + it * NW) * 8 + ld_row;
-        if (r > g.M - 1) r = g.M - 1;
-        a_src[it] = g.A + r * g.lda + ld_chunk * 16;
-    }
+    for (int it = 0; it < kAIter; ++it) a_off[it] = (uint32_t)(((wave + it * NW) * 8 + ld_row) * g.lda + ld_chunk * 16);
 #pragma unroll
-    for (int it = 0; it < kWIter; ++it) {
-        int64_t r = n0 + (wave + it * NW) * 8 + ld_row;
-        if (r > g.N - 1) r = g.N - 1;
-        w_src[it] = g.W + r * g.ldw + ld_chunk * 16;
-    }
+    for (int it = 0; it < kWIter; ++it) w_off[it] = (uint32_t)(((wave + it * NW) * 8 + ld_row) * g.ldw + ld_chunk * 16);
     // scale rows: 64 floats per wave instruction; instruction i -> K-block i / kSPer of the stage, and inside
-    // it the first BM/64 instructions fetch sA, the rest sW
+    // it the first BM/64 instructions fetch sA, the rest sW.  Waves beyond the last instruction repeat an
+    // earlier one (same bytes to the same place) rather than branch around it.
     constexpr int kSPer = BM / 64 + BN / 64;
     constexpr int kSInstr = PARTIALS ? 0 : NBS * kSPer;
     constexpr int kSIter = (kSInstr + NW - 1) / NW;
-    const float *s_src[kSIter > 0 ? kSIter : 1];
-    int s_dst[kSIter > 0 ? kSIter : 1];
-    int64_t s_step[kSIter > 0 ? kSIter : 1];
+    constexpr int kSI = kSIter > 0 ? kSIter : 1;
+    const int64_t nblk = g.K / BLK;
+    const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, PARTIALS ? 0 : ((nblk - 1) * g.M + (g.M - m0)) * 4);
+    const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, PARTIALS ? 0 : ((nblk - 1) * g.N + (g.N - n0)) * 4);
+    uint32_t s_off[kSI];
+    int s_dst[kSI], s_bufstep[kSI];
+    bool s_is_a[kSI];
 #pragma unroll
     for (int it = 0; it < kSIter; ++it) {
-        const int i = wave + it * NW;
+        const int i = (wave + it * NW) % (kSInstr > 0 ? kSInstr : 1);
         const int b = i / kSPer, r = i % kSPer;
-        if (r < BM / 64) {
-            int64_t m = m0 + r * 64 + lane;
-            if (m > g.M - 1) m = g.M - 1;
-            s_src[it] = g.sA + (int64_t)b * g.M + m;
+        s_is_a[it] = r < BM / 64;
+        if (s_is_a[it]) {
+            s_off[it] = (uint32_t)((b * g.M + r * 64 + lane) * 4);
             s_dst[it] = L::kSAReg + (b * BM + r * 64) * 4;
-            s_step[it] = (int64_t)NBS * g.M;
+            s_bufstep[it] = L::kSABuf;
         } else {
-            int64_t n = n0 + (r - BM / 64) * 64 + lane;
-            if (n > g.N - 1) n = g.N - 1;
-            s_src[it] = g.sW + (int64_t)b * g.N + n;
+            s_off[it] = (uint32_t)((b * g.N + (r - BM / 64) * 64 + lane) * 4);
             s_dst[it] = L::kSWReg + (b * BN + (r - BM / 64) * 64) * 4;
-            s_step[it] = (int64_t)NBS * g.N;
+            s_bufstep[it] = L::kSWBuf;
         }
     }
+    uint32_t k_pos = 0;                            // K offset of the next stage to load (bytes)
+    uint32_t sa_pos = 0, sw_pos = 0;               // scale-row offsets of the next stage (bytes)
 
-    auto issue_stage = [&](int buf) {             // buf is wave-uniform: the LDS destinations are scalars
+    constexpr int kLoadsPerStage = kAIter + kWIter + kSIter;     // VMEM instructions one wave issues per stage
+    auto issue_stage = [&](int buf) {             // buf is wave-uniform: LDS destinations and K position are scalars
+#ifdef BI8_ABL_NODMA
+        return;
+#endif
 #pragma unroll
-        for (int it = 0; it < kAIter; ++it) {
-            lds_dma16(a_src[it], lds + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024);
-            a_src[it] += kStageK;
-        }
+        for (int it = 0; it < kAIter; ++it) bi8_buffer_to_lds16(a_rsrc, lds + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024, a_off[it], k_pos);
 #pragma unroll
-        for (int it = 0; it < kWIter; ++it) {
-            lds_dma16(w_src[it], lds + L::kWReg + buf * L::kWBuf + (wave + it * NW) * 1024);
-            w_src[it] += kStageK;
-        }
+        for (int it = 0; it < kWIter; ++it) bi8_buffer_to_lds16(w_rsrc, lds + L::kWReg + buf * L::kWBuf + (wave + it * NW) * 1024, w_off[it], k_pos);
+        k_pos += kStageK;
 #pragma unroll
         for (int it = 0; it < kSIter; ++it) {
-            const int i = wave + it * NW;
-            if (i < kSInstr) {
-                const bool is_a = (i % kSPer) < BM / 64;
-                lds_dma4(s_src[it], lds + s_dst[it] + buf * (is_a ? L::kSABuf : L::kSWBuf));
-                s_src[it] += s_step[it];
-            }
+            if (s_is_a[it]) bi8_buffer_to_lds4(sa_rsrc, lds + s_dst[it] + buf * s_bufstep[it], s_off[it], sa_pos);
+            else bi8_buffer_to_lds4(sw_rsrc, lds + s_dst[it] + buf * s_bufstep[it], s_off[it], sw_pos);
         }
+        sa_pos += (uint32_t)(NBS * g.M * 4);
+        sw_pos += (uint32_t)(NBS * g.N * 4);
     };
 
-    // ---- operand fragment addresses of the buffer being computed.  Row r = ... + l32, 16-byte chunk
-    // (2*ks + h) ^ (r & 7): address(ks) = base ^ (ks << 5).  One register per ks; subtile offsets are immediates.
-    const int frag_sw = ((h ^ (lane & 7)) << 4);
+    // ---- operand fragment addresses (buffer 0).  Row r = ... + l32, 16-byte chunk (2*ks + h) ^ ((r >> 1) & 7):
+    // address(ks) = base ^ (ks << 5).  One register per ks; buffer and subtile offsets are immediates.
+    const int frag_sw = ((h ^ ((l32 >> 1) & 7)) << 4);
     int a_addr[4], w_addr[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
         a_addr[ks] = (L::kAReg + (wm * (BM / WM) + l32) * kStageK + frag_sw) ^ (ks << 5);
         w_addr[ks] = (L::kWReg + (wn * (BN / WN) + l32) * kStageK + frag_sw) ^ (ks << 5);
     }
-    int sa_addr = L::kSAReg + (wm * (BM / WM) + 4 * h) * 4;
-    int sw_addr = L::kSWReg + (wn * (BN / WN) + l32) * 4;
-    int flip = 1;                                  // +1: the next stage is in buffer 1, -1: in buffer 0
+    const int sa_addr = L::kSAReg + (wm * (BM / WM) + 4 * h) * 4;
+    const int sw_addr = L::kSWReg + (wn * (BN / WN) + l32) * 4;
 
     float acc[TM][TN][16];
 #pragma unroll
@@ -202,57 +208,94 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
 
-    // The last subtile of a stage is folded into the accumulator during the first MFMAs of the NEXT stage
-    // (after the barrier, while the new operands are still on their way from LDS).
-    bi8_v16i pend_p = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    bi8_v4f pend_sx[4];
+    // Loop-carried pipeline state.  The last subtile ("item") of a stage is folded into the accumulator
+    // during the first MFMAs of the NEXT stage (after the barrier, while the new operands are still on their
+    // way from LDS), so its int32 partial and its scales stay live across the stage boundary.
+    constexpr int NITEM = NBS * NSUB;
+    static_assert(NITEM % 2 == 0, "the two partial buffers alternate consistently across stages");
+    bi8_v16i p[2];
+    constexpr int kMagicBits = 0x4B400000;        // bit pattern of 1.5 * 2^23
+    const int mg = PARTIALS ? 0 : kMagicBits;
+    const bi8_v16i magic = {mg, mg, mg, mg, mg, mg, mg, mg, mg, mg, mg, mg, mg, mg, mg, mg};
+    p[0] = p[1] = magic;                           // "partial 0" for the fold that precedes the first stage
+    float swv[2][TN], swc[2][TN];                  // [K-block parity][column subtile]: scale b and -(1.5*2^23)*b
+    bi8_v4f sxv[2][TM][4];                         // [K-block parity][row subtile][row group of 8]
 #pragma unroll
-    for (int i = 0; i < 4; ++i) pend_sx[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
-    float pend_sw = 0.0f;
+    for (int q = 0; q < 2; ++q) {
+#pragma unroll
+        for (int b = 0; b < TN; ++b) swv[q][b] = swc[q][b] = 0.0f;
+#pragma unroll
+        for (int a = 0; a < TM; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sxv[q][a][i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    }
 
-    auto fold = [&](const bi8_v16i &pt, const bi8_v4f *sx, float sw, float *dst) {
+    // Fold elements [16*ks/KSB, 16*(ks+1)/KSB) of an item's partial into the accumulator, two vector ops each.
+    // The MFMA chain starts from kMagicBits in every accumulator lane, so the int32 result P + kMagicBits,
+    // read as a float, IS the number 1.5*2^23 + P (exact for |P| < 2^22): no int->float conversion.  With the
+    // column scale b rounded to 22 significant bits, c = -(1.5*2^23)*b is exact, and fma(f, b, c) = fl(b*P)
+    // with a single rounding; the second fma applies the row scale and accumulates.
+    auto fold_slice = [&](const bi8_v16i &pt, const bi8_v4f *sx, float sw, float swc, float *dst, int ks) {
+#ifdef BI8_ABL_NOFOLD
+        asm volatile("" ::"v"(pt));
+        return;
+#endif
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float f = (float)pt[r] * sx[r >> 2][r & 3];
-            dst[r] = __builtin_fmaf(f, sw, dst[r]);
+        for (int r = ks * (16 / KSB); r < (ks + 1) * (16 / KSB); ++r) {
+            const float u = __builtin_fmaf(bi8_u2f((uint32_t)pt[r]), sw, swc);
+            dst[r] = __builtin_fmaf(u, sx[r >> 2][r & 3], dst[r]);
         }
     };
 
-    // One stage = NBS K-blocks x NSUB subtiles ("items").  The MFMAs of item t are issued before the fp32
-    // fold of item t-1, so the matrix pipe works while the vector ALU converts and accumulates.
-    auto compute_stage = [&](int s) {
+    // One stage = NBS K-blocks x NSUB subtiles ("items"), KSB MFMAs each.  The instruction order below is the
+    // schedule: sched_barrier(0) fences keep the compiler from reordering across steps.  Step (t, ks) issues
+    // one MFMA of item t and folds one slice of item t-1, so the matrix pipe and the vector ALU overlap;
+    // operand reads are issued at the top of the stage in order of first use, scale reads as soon as the
+    // registers they overwrite have been consumed.
+    auto compute_stage = [&](int buf, int s) {     // buf is wave-uniform
+        const int oa = buf * L::kABuf, ow = buf * L::kWBuf, osa = buf * L::kSABuf, osw = buf * L::kSWBuf;
         bi8_v4i af[TM][4], wf[TN][4];
+        auto load_scales = [&](int blk, int a0, int a1, int b0, int b1) {
+#pragma unroll
+            for (int b = b0; b < b1; ++b) swv[blk & 1][b] = *(const float *)(lds + (sw_addr + osw) + (blk * BN + b * 32) * 4);
+#pragma unroll
+            for (int a = a0; a < a1; ++a)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    sxv[blk & 1][a][i] = *(const bi8_v4f *)(lds + (sa_addr + osa) + (blk * BM + a * 32 + 8 * i) * 4);
+        };
+        // column scale -> 22 significant bits (relative change <= 2^-22) and its product with -1.5*2^23 (exact)
+        auto prep_scales = [&](int blk, int b0, int b1) {
+#pragma unroll
+            for (int b = b0; b < b1; ++b) {
+                const float bq = bi8_u2f((bi8_f2u(swv[blk & 1][b]) + 2u) & ~3u);
+                swv[blk & 1][b] = bq;
+                swc[blk & 1][b] = -BI8_MAGIC * bq;
+            }
+        };
+        // operands in order of first use: item (a, b) needs af[a][*] and wf[b][*]
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-#pragma unroll
-            for (int a = 0; a < TM; ++a) af[a][ks] = *(const bi8_v4i *)(lds + a_addr[ks] + a * 32 * kStageK);
-#pragma unroll
-            for (int b = 0; b < TN; ++b) wf[b][ks] = *(const bi8_v4i *)(lds + w_addr[ks] + b * 32 * kStageK);
+            af[0][ks] = *(const bi8_v4i *)(lds + (a_addr[ks] + oa));
+            wf[0][ks] = *(const bi8_v4i *)(lds + (w_addr[ks] + ow));
         }
-        float swv[2][TN];
-        bi8_v4f sxv[2][TM][4];
-        auto load_scales = [&](int blk) {
 #pragma unroll
-            for (int b = 0; b < TN; ++b) swv[blk & 1][b] = *(const float *)(lds + sw_addr + (blk * BN + b * 32) * 4);
+        for (int b = 1; b < TN; ++b)
 #pragma unroll
-            for (int a = 0; a < TM; ++a)
+            for (int ks = 0; ks < 4; ++ks) wf[b][ks] = *(const bi8_v4i *)(lds + (w_addr[ks] + ow) + b * 32 * kStageK);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) sxv[blk & 1][a][i] = *(const bi8_v4f *)(lds + sa_addr + (blk * BM + a * 32 + 8 * i) * 4);
-        };
-        auto chain = [&](int t) {
-            const int blk = t / NSUB, a = (t % NSUB) / TN, b = t % TN;
-            bi8_v16i acc_i = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int a = 1; a < TM; ++a)
 #pragma unroll
-            for (int ks = 0; ks < KSB; ++ks)
-                acc_i = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a][blk * KSB + ks], wf[b][blk * KSB + ks], acc_i, 0, 0, 0);
-            return acc_i;
-        };
-        constexpr int NITEM = NBS * NSUB;
+            for (int ks = 0; ks < 4; ++ks) af[a][ks] = *(const bi8_v4i *)(lds + (a_addr[ks] + oa) + a * 32 * kStageK);
+
         if constexpr (PARTIALS) {
 #pragma unroll
             for (int t = 0; t < NITEM; ++t) {
                 const int blk = t / NSUB, a = (t % NSUB) / TN, b = t % TN;
-                const bi8_v16i pt = chain(t);
+                bi8_v16i pt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int ks = 0; ks < KSB; ++ks)
+                    pt = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a][blk * KSB + ks], wf[b][blk * KSB + ks], pt, 0, 0, 0);
                 const int64_t jb = (int64_t)s * NBS + blk;
                 const int64_t n = n0 + wn * (BN / WN) + b * 32 + l32;
 #pragma unroll
@@ -262,55 +305,82 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
                 }
             }
         } else {
-            bi8_v16i p[2];
+            // The pending item of the previous stage reads parity (NBS-1)&1, row subtile TM-1, column TN-1.
+            constexpr bool kClash = ((NBS - 1) & 1) == 0;          // K-block 0 of this stage reuses those registers
+            load_scales(0, 0, kClash ? TM - 1 : TM, 0, kClash ? TN - 1 : TN);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int t = 0; t < NITEM; ++t) {
-                const int blk = t / NSUB;
-                if (t % NSUB == 0) load_scales(blk);
-                p[t & 1] = chain(t);
-                if (t == 0) {
-                    fold(pend_p, pend_sx, pend_sw, acc[TM - 1][TN - 1]);
-                } else {
-                    const int u = t - 1, ub = u / NSUB, ua = (u % NSUB) / TN, un = u % TN;
-                    fold(p[u & 1], sxv[ub & 1][ua], swv[ub & 1][un], acc[ua][un]);
-                }
+                const int blk = t / NSUB, a = (t % NSUB) / TN, b = t % TN;
+                // item t-1 (for t = 0: the last item of the previous stage)
+                const int u = (t + NITEM - 1) % NITEM, ub = u / NSUB, ua = (u % NSUB) / TN, un = u % TN;
 #pragma unroll
                 for (int ks = 0; ks < KSB; ++ks) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);              // one MFMA of item t
-                    __builtin_amdgcn_sched_group_barrier(0x002, 48 / KSB, 0);       // a slice of item t-1's fold
+                    // at the top of a stage the fold goes first: its inputs are ready, the operands are not yet
+                    if (t == 0) fold_slice(p[u & 1], sxv[ub & 1][ua], swv[ub & 1][un], swc[ub & 1][un], acc[ua][un], ks);
+#ifdef BI8_ABL_NOMFMA
+                    asm volatile("" ::"v"(af[a][blk * KSB + ks]), "v"(wf[b][blk * KSB + ks]));
+#else
+                    if (ks == 0)
+                        p[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a][blk * KSB], wf[b][blk * KSB], magic, 0, 0, 0);
+                    else
+                        p[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a][blk * KSB + ks], wf[b][blk * KSB + ks], p[t & 1], 0, 0, 0);
+#endif
+                    if (t != 0) fold_slice(p[u & 1], sxv[ub & 1][ua], swv[ub & 1][un], swc[ub & 1][un], acc[ua][un], ks);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (t == 0) {
+                    if (kClash) {
+                        load_scales(0, TM - 1, TM, 0, 0);
+                        load_scales(0, 0, 0, TN - 1, TN);
+                    }
+                    prep_scales(0, 0, TN);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                // the registers of parity (blk+1)&1 were last read by the fold that just finished when t opens a block
+                if (t % NSUB == 0 && blk + 1 < NBS) {
+                    load_scales(blk + 1, 0, TM, 0, TN);
+                    prep_scales(blk + 1, 0, TN);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
             }
-            pend_p = p[(NITEM - 1) & 1];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pend_sx[i] = sxv[(NBS - 1) & 1][TM - 1][i];
-            pend_sw = swv[(NBS - 1) & 1][TN - 1];
         }
-        // point the fragment addresses at the other buffer
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            a_addr[ks] += flip * L::kABuf;
-            w_addr[ks] += flip * L::kWBuf;
-        }
-        sa_addr += flip * L::kSABuf;
-        sw_addr += flip * L::kSWBuf;
-        flip = -flip;
     };
 
-    issue_stage(0);
-    int fill = 1;
-    for (int s = 0; s + 1 < nstages; ++s) {
-        __builtin_amdgcn_s_waitcnt(0x0F70);        // vmcnt(0): this wave's direct-to-LDS loads have landed
-        __syncthreads();                           // ... and everyone's; the other buffer is free again
-        issue_stage(fill);
-        fill ^= 1;
-        compute_stage(s);
-    }
-    if (nstages > 0) {
-        __builtin_amdgcn_s_waitcnt(0x0F70);
+    // Ring of kBufs stage buffers.  Before computing stage s every wave waits until only the loads of later
+    // stages are still outstanding (its own direct-to-LDS loads of stage s have landed), then the barrier makes
+    // that true for all waves and frees the buffer computed one stage earlier.
+    auto sync_stage = [&](auto pending_c) {
+        constexpr int kPending = decltype(pending_c)::value;       // VMEM instructions allowed to stay in flight
+        static_assert(kPending < 64, "vmcnt is a 6-bit field");
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));   // vmcnt(kPending) only
         __syncthreads();
-        compute_stage(nstages - 1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // kBufs - 1 stages of loads are in flight while one stage is computed
+    using InFlight = std::integral_constant<int, (kBufs - 2) * kLoadsPerStage>;
+    using Drained = std::integral_constant<int, 0>;
+#pragma unroll
+    for (int q = 0; q < kBufs - 1; ++q)
+        if (q < nstages) issue_stage(q);
+    int s = 0, buf = 0, fill = kBufs - 1;
+    for (; s + kBufs - 1 < nstages; ++s) {         // steady state: start the loads of stage s+kBufs-1, compute stage s
+        sync_stage(InFlight{});
+        issue_stage(fill);
+        compute_stage(buf, s);
+        buf = (buf == kBufs - 1) ? 0 : buf + 1;
+        fill = (fill == kBufs - 1) ? 0 : fill + 1;
     }
-    if constexpr (!PARTIALS) fold(pend_p, pend_sx, pend_sw, acc[TM - 1][TN - 1]);
+    for (; s < nstages; ++s) {                     // drain: nothing left to start; wait for everything each time
+        sync_stage(Drained{});
+        compute_stage(buf, s);
+        buf = (buf == kBufs - 1) ? 0 : buf + 1;
+    }
+    if constexpr (!PARTIALS)
+#pragma unroll
+        for (int ks = 0; ks < KSB; ++ks)
+            fold_slice(p[(NITEM - 1) & 1], sxv[(NBS - 1) & 1][TM - 1], swv[(NBS - 1) & 1][TN - 1], swc[(NBS - 1) & 1][TN - 1], acc[TM - 1][TN - 1], ks);
 
     if constexpr (!PARTIALS) {
         const float div = (float)(1.0 / (127.0 * 127.0));
@@ -396,14 +466,15 @@ __global__ __launch_bounds__(256) void gemm_generic(const GemmArgs g, int block)
     }
 }
 
-template <int BM, int BN, int WM, int WN, int BLK, int CDT, bool PARTIALS>
+template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
 int launch_tile(GemmArgs g, hipStream_t st) {
-    constexpr int kLds = TileLds<BM, BN, BLK>::kBytes;
+    constexpr int kLds = TileLds<BM, BN, BLK, NBUF>::kBytes;
+    static_assert(TileLds<BM, BN, BLK, NBUF>::kFits, "tile does not fit the LDS");
     const int64_t tm = (g.M + BM - 1) / BM, tn = (g.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     g.tiles_m = (int)tm;
     g.tiles_n = (int)tn;
-    auto kern = gemm_tile<BM, BN, WM, WN, BLK, CDT, PARTIALS>;
+    auto kern = gemm_tile<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>;
     if (kLds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
         if (e != hipSuccess) return bi8_hip_rc(e);
@@ -423,15 +494,19 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
 
 // tile shape by problem shape: the big tile when there is enough work to fill 256 CUs with it
 template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipStream_t st) {
+    constexpr bool kBigFits = TileLds<256, 128, BLK, 3>::kFits;
 #ifdef BI8_FORCE_TILE
-    if (BI8_FORCE_TILE == 0) return launch_tile<256, 128, 4, 2, BLK, CDT, PARTIALS>(g, st);
-    if (BI8_FORCE_TILE == 1) return launch_tile<128, 128, 2, 2, BLK, CDT, PARTIALS>(g, st);
-    if (BI8_FORCE_TILE == 2) return launch_tile<64, 128, 1, 2, BLK, CDT, PARTIALS>(g, st);
+    if constexpr (kBigFits) if (BI8_FORCE_TILE == 0) return launch_tile<256, 128, 4, 2, 3, BLK, CDT, PARTIALS>(g, st);
+    if (BI8_FORCE_TILE == 1) return launch_tile<128, 128, 2, 2, 2, BLK, CDT, PARTIALS>(g, st);
+    if (BI8_FORCE_TILE == 2) return launch_tile<64, 128, 1, 2, 3, BLK, CDT, PARTIALS>(g, st);
+    if (BI8_FORCE_TILE == 3) return launch_tile<128, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
 #endif
-    const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
-    if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, BLK, CDT, PARTIALS>(g, st);
-    if (g.M > 64) return launch_tile<128, 128, 2, 2, BLK, CDT, PARTIALS>(g, st);
-    return launch_tile<64, 128, 1, 2, BLK, CDT, PARTIALS>(g, st);
+    if constexpr (kBigFits) {
+        const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
+        if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, 3, BLK, CDT, PARTIALS>(g, st);
+    }
+    if (g.M > 64) return launch_tile<128, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
+    return launch_tile<64, 128, 1, 2, 3, BLK, CDT, PARTIALS>(g, st);
 }
 
 template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hipStream_t st) {
