@@ -1,70 +1,79 @@
 // Block dequantize (bi8_dequantize_rowwise): out = (scale * float(code)) * fp32(1/127), cast on store.
-// Replaces _dequantize_block_rowwise, triton_functions.py:468-490.  HBM-bound: one lane = 16 codes
-// (one 128-bit load) -> 16 outputs (two or four 128-bit stores).  Same tiling as the quantizer: a
-// workgroup owns 16 rows x 1024 codes and first pulls its scales in through LDS, so the block-major /
-// row-minor scale array is read as runs of 16 consecutive rows.
+// Replaces _dequantize_block_rowwise, triton_functions.py:468-490.  HBM-bound: one lane = one 128-bit store
+// of outputs (8 bf16/f16 or 4 fp32) per step, so every wave store covers 1 KiB of contiguous output.  Same
+// tiling as the quantizer: a workgroup owns 16 rows x 2 KiB of output row and first pulls its scales in
+// through LDS, so the block-major / row-minor scale array is read as runs of 16 consecutive rows.
 #include "bi8_common.h"
 
 namespace {
 
 constexpr int kRows = 16;
-constexpr int kTileK = 1024;       // codes per tile row = 64 lanes x 16
 constexpr int kThreads = 256;
 
-template <int DT> __device__ __forceinline__ void store16(void *out, int64_t idx, const float *v) {
+// One lane = kOut outputs = one 16-byte store (8 bf16/f16 or 4 fp32), so every store instruction of a wave
+// writes 1 KiB of contiguous output; the codes come in as one 8- or 4-byte load per lane.
+template <int DT> struct Out {
+    static constexpr int kElems = (DT == BI8_F32) ? 4 : 8;
+};
+
+template <int DT> __device__ __forceinline__ void store_vec(void *out, int64_t idx, const float *v) {
     if constexpr (DT == BI8_F32) {
-        bi8_v4f *dst = (bi8_v4f *)((float *)out + idx);
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            bi8_v4f w = {v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3]};
-            __builtin_nontemporal_store(w, dst + g);
-        }
+        bi8_v4f w = {v[0], v[1], v[2], v[3]};
+        __builtin_nontemporal_store(w, (bi8_v4f *)((float *)out + idx));
     } else {
-        bi8_v4u *dst = (bi8_v4u *)((uint16_t *)out + idx);
+        bi8_v4u w;
 #pragma unroll
-        for (int g = 0; g < 2; ++g) {
-            bi8_v4u w;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                uint32_t lo, hi;
-                if constexpr (DT == BI8_BF16) {
-                    lo = bi8_bf16_bits(v[8 * g + 2 * e]);
-                    hi = bi8_bf16_bits(v[8 * g + 2 * e + 1]);
-                } else {
-                    lo = bi8_f16_bits(v[8 * g + 2 * e]);
-                    hi = bi8_f16_bits(v[8 * g + 2 * e + 1]);
-                }
-                w[e] = lo | (hi << 16);
+        for (int e = 0; e < 4; ++e) {
+            uint32_t lo, hi;
+            if constexpr (DT == BI8_BF16) {
+                lo = bi8_bf16_bits(v[2 * e]);
+                hi = bi8_bf16_bits(v[2 * e + 1]);
+            } else {
+                lo = bi8_f16_bits(v[2 * e]);
+                hi = bi8_f16_bits(v[2 * e + 1]);
             }
-            __builtin_nontemporal_store(w, dst + g);
+            w[e] = lo | (hi << 16);
         }
+        __builtin_nontemporal_store(w, (bi8_v4u *)((uint16_t *)out + idx));
     }
 }
 
-// LOG2B: log2 of the block size (>= 4, so that one lane's 16 codes share a scale)
+constexpr int kLoads = 8;          // wave-loads per lane per tile
+
+// workgroup tile: 16 rows x (2 * 64 * kOut) codes; wave w owns rows 4w .. 4w+3, two chunks of 64 * kOut codes each
 template <int DT>
 __global__ __launch_bounds__(kThreads) void dequantize_rows_vec(const int8_t *__restrict__ q, const float *__restrict__ scales,
                                                                 void *__restrict__ out, int64_t M, int64_t K, int64_t ldq,
                                                                 int64_t ldo, int64_t nblk, int log2b, int tiles_k) {
-    __shared__ float s_tile[kTileK / 16][kRows + 1];
+    constexpr int VEC = Out<DT>::kElems;
+    constexpr int TE = 2 * BI8_WAVE * VEC;         // codes per tile row
+    __shared__ float s_tile[TE / 8][kRows + 1];    // block size >= 8 on this path
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int64_t tile_m = blockIdx.x / tiles_k;
     const int tile_k = blockIdx.x % tiles_k;
     const int64_t row0 = tile_m * kRows;
-    const int64_t col0 = (int64_t)tile_k * kTileK;
-    const int nb = kTileK >> log2b;                 // blocks per tile row
+    const int64_t col0 = (int64_t)tile_k * TE;
+    const int nb = (TE >> log2b) > 0 ? (TE >> log2b) : 1;      // blocks per tile row
     const int64_t jb0 = col0 >> log2b;
 
-    bi8_v4u raw[4];
+    uint32_t raw[kLoads][VEC / 4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t row = row0 + wave * 4 + i;
-        const int64_t col = col0 + lane * 16;
-        bi8_v4u v = {0u, 0u, 0u, 0u};
-        if (row < M && col < K) v = __builtin_nontemporal_load((const bi8_v4u *)(q + row * ldq + col));
-        raw[i] = v;
+    for (int i = 0; i < kLoads; ++i) {
+        const int64_t row = row0 + wave * 4 + (i >> 1);
+        const int64_t col = col0 + ((i & 1) * BI8_WAVE + lane) * VEC;
+#pragma unroll
+        for (int e = 0; e < VEC / 4; ++e) raw[i][e] = 0u;
+        if (row < M && col < K) {
+            if constexpr (VEC == 8) {
+                const bi8_v2u v = __builtin_nontemporal_load((const bi8_v2u *)(q + row * ldq + col));
+                raw[i][0] = v[0];
+                raw[i][1] = v[1];
+            } else {
+                raw[i][0] = __builtin_nontemporal_load((const uint32_t *)(q + row * ldq + col));
+            }
+        }
     }
     for (int t = tid; t < nb * kRows; t += kThreads) {
         const int j = t / kRows, r = t % kRows;
@@ -76,21 +85,22 @@ __global__ __launch_bounds__(kThreads) void dequantize_rows_vec(const int8_t *__
 
     const float inv127 = (float)(1.0 / 127.0);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t row = row0 + wave * 4 + i;
-        const int64_t col = col0 + lane * 16;
+    for (int i = 0; i < kLoads; ++i) {
+        const int64_t row = row0 + wave * 4 + (i >> 1);
+        const int incol = ((i & 1) * BI8_WAVE + lane) * VEC;
+        const int64_t col = col0 + incol;
         if (row < M && col < K) {
-            const float s = s_tile[(lane * 16) >> log2b][wave * 4 + i];
-            float v[16];
+            const float s = s_tile[incol >> log2b][wave * 4 + (i >> 1)];
+            float v[VEC];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
+            for (int e = 0; e < VEC / 4; ++e) {
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
                     const int code = (int)(raw[i][e] << (24 - 8 * b)) >> 24;     // sign-extended byte b
                     v[4 * e + b] = (s * (float)code) * inv127;                   // two roundings, left to right
                 }
             }
-            store16<DT>(out, row * ldo + col, v);
+            store_vec<DT>(out, row * ldo + col, v);
         }
     }
 }
@@ -112,10 +122,12 @@ __global__ __launch_bounds__(kThreads) void dequantize_rows_generic(const int8_t
 template <int DT>
 int dispatch(const int8_t *q, const float *scales, void *out, int64_t M, int64_t K, int64_t ldq, int64_t ldo, int block,
              hipStream_t st) {
-    const bool vec_ok = bi8_pow2(block) && block >= 16 && block <= kTileK && K % 16 == 0 && ldq % 16 == 0 && ldo % 16 == 0 &&
-                        bi8_aligned(q, 16) && bi8_aligned(out, 16);
+    constexpr int VEC = Out<DT>::kElems;
+    constexpr int TE = 2 * BI8_WAVE * VEC;
+    const bool vec_ok = bi8_pow2(block) && block >= 8 && K % VEC == 0 && ldq % VEC == 0 && ldo % VEC == 0 &&
+                        bi8_aligned(q, VEC) && bi8_aligned(out, 16);
     if (vec_ok) {
-        const int64_t tiles_k = (K + kTileK - 1) / kTileK;
+        const int64_t tiles_k = (K + TE - 1) / TE;
         const int64_t tiles_m = (M + kRows - 1) / kRows;
         if (tiles_k * tiles_m > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
         const int64_t nblk = (K + block - 1) / block;
