@@ -171,9 +171,6 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
 
     constexpr int kLoadsPerStage = kAIter + kWIter + kSIter;     // VMEM instructions one wave issues per stage
     auto issue_stage = [&](int buf) {             // buf is wave-uniform: LDS destinations and K position are scalars
-#ifdef BI8_ABL_NODMA
-        return;
-#endif
 #pragma unroll
         for (int it = 0; it < kAIter; ++it) bi8_buffer_to_lds16(a_rsrc, lds + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024, a_off[it], k_pos);
 #pragma unroll
@@ -236,10 +233,6 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
     // column scale b rounded to 22 significant bits, c = -(1.5*2^23)*b is exact, and fma(f, b, c) = fl(b*P)
     // with a single rounding; the second fma applies the row scale and accumulates.
     auto fold_slice = [&](const bi8_v16i &pt, const bi8_v4f *sx, float sw, float swc, float *dst, int ks) {
-#ifdef BI8_ABL_NOFOLD
-        asm volatile("" ::"v"(pt));
-        return;
-#endif
 #pragma unroll
         for (int r = ks * (16 / KSB); r < (ks + 1) * (16 / KSB); ++r) {
             const float u = __builtin_fmaf(bi8_u2f((uint32_t)pt[r]), sw, swc);
@@ -273,20 +266,24 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
                 swc[blk & 1][b] = -BI8_MAGIC * bq;
             }
         };
-        // operands in order of first use: item (a, b) needs af[a][*] and wf[b][*]
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            af[0][ks] = *(const bi8_v4i *)(lds + (a_addr[ks] + oa));
-            wf[0][ks] = *(const bi8_v4i *)(lds + (w_addr[ks] + ow));
-        }
-#pragma unroll
-        for (int b = 1; b < TN; ++b)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) wf[b][ks] = *(const bi8_v4i *)(lds + (w_addr[ks] + ow) + b * 32 * kStageK);
-#pragma unroll
-        for (int a = 1; a < TM; ++a)
+        // Operands are read just in time: item (0,0)'s at the top of the stage, row subtile a / column subtile b
+        // during the item that precedes their first use, so the LDS traffic is spread over the stage.
+        auto load_a = [&](int a) {
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) af[a][ks] = *(const bi8_v4i *)(lds + (a_addr[ks] + oa) + a * 32 * kStageK);
+        };
+        auto load_w = [&](int b) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) wf[b][ks] = *(const bi8_v4i *)(lds + (w_addr[ks] + ow) + b * 32 * kStageK);
+        };
+        load_a(0);
+        load_w(0);
+        if constexpr (PARTIALS || NBS > 1) {       // these variants keep the simple order: everything up front
+#pragma unroll
+            for (int b = 1; b < TN; ++b) load_w(b);
+#pragma unroll
+            for (int a = 1; a < TM; ++a) load_a(a);
+        }
 
         if constexpr (PARTIALS) {
 #pragma unroll
@@ -314,18 +311,19 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
                 const int blk = t / NSUB, a = (t % NSUB) / TN, b = t % TN;
                 // item t-1 (for t = 0: the last item of the previous stage)
                 const int u = (t + NITEM - 1) % NITEM, ub = u / NSUB, ua = (u % NSUB) / TN, un = u % TN;
+                if constexpr (NBS == 1) {           // operands of the next item: column subtile b+1, then row subtile a+1
+                    if (a == 0 && b + 1 < TN) load_w(b + 1);
+                    if (b == TN - 1 && a + 1 < TM) load_a(a + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
 #pragma unroll
                 for (int ks = 0; ks < KSB; ++ks) {
                     // at the top of a stage the fold goes first: its inputs are ready, the operands are not yet
                     if (t == 0) fold_slice(p[u & 1], sxv[ub & 1][ua], swv[ub & 1][un], swc[ub & 1][un], acc[ua][un], ks);
-#ifdef BI8_ABL_NOMFMA
-                    asm volatile("" ::"v"(af[a][blk * KSB + ks]), "v"(wf[b][blk * KSB + ks]));
-#else
                     if (ks == 0)
                         p[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a][blk * KSB], wf[b][blk * KSB], magic, 0, 0, 0);
                     else
                         p[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[a][blk * KSB + ks], wf[b][blk * KSB + ks], p[t & 1], 0, 0, 0);
-#endif
                     if (t != 0) fold_slice(p[u & 1], sxv[ub & 1][ua], swv[ub & 1][un], swc[ub & 1][un], acc[ua][un], ks);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -337,6 +335,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
                     prep_scales(0, 0, TN);
                     __builtin_amdgcn_sched_barrier(0);
                 }
+
                 // the registers of parity (blk+1)&1 were last read by the fold that just finished when t opens a block
                 if (t % NSUB == 0 && blk + 1 < NBS) {
                     load_scales(blk + 1, 0, TM, 0, TN);
@@ -500,6 +499,7 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
     if (BI8_FORCE_TILE == 1) return launch_tile<128, 128, 2, 2, 2, BLK, CDT, PARTIALS>(g, st);
     if (BI8_FORCE_TILE == 2) return launch_tile<64, 128, 1, 2, 3, BLK, CDT, PARTIALS>(g, st);
     if (BI8_FORCE_TILE == 3) return launch_tile<128, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
+    if constexpr (BLK == 128) if (BI8_FORCE_TILE == 4) return launch_tile<256, 256, 4, 2, 2, BLK, CDT, PARTIALS>(g, st);
 #endif
     if constexpr (kBigFits) {
         const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
