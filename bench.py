@@ -40,40 +40,49 @@ def event_ms(fn, iters: int) -> float:
 
 
 def bench_quantize(pkg, torch, iters: int):
-    """block quantize / dequantize of bf16 [8192,8192] with outliers, through the C ABI with preallocated outputs"""
+    """block quantize / dequantize of bf16 [8192,8192] with outliers, through the C ABI with preallocated outputs.
+    Three independent sets of buffers are used in rotation (576 MiB in total), so that successive launches do
+    not find their operands in the 256 MiB memory-side cache left there by the launch before."""
     from blockwise_int8_linear_amd import _lib
     lib = _lib.load()
     M = K = 8192
     E = M * K
-    gen = torch.Generator(device="cuda").manual_seed(0)
-    x = torch.randn(M, K, device="cuda", generator=gen, dtype=torch.float32)
-    gen1 = torch.Generator(device="cuda").manual_seed(1)
-    pos = torch.randint(0, E, (E // 1000,), device="cuda", generator=gen1)
-    x.view(-1)[pos] *= 50.0
-    x = x.to(torch.bfloat16)
+    NSETS = 3
+    xs = []
+    for i in range(NSETS):
+        gen = torch.Generator(device="cuda").manual_seed(i)
+        x = torch.randn(M, K, device="cuda", generator=gen, dtype=torch.float32)
+        gen1 = torch.Generator(device="cuda").manual_seed(100 + i)
+        pos = torch.randint(0, E, (E // 1000,), device="cuda", generator=gen1)
+        x.view(-1)[pos] *= 50.0
+        xs.append(x.to(torch.bfloat16))
+        del x
     st = torch.cuda.current_stream().cuda_stream
     out = {}
     for B in (32, 64, 128):
-        q = torch.empty(M, K, device="cuda", dtype=torch.int8)
-        s = torch.empty(K // B, M, device="cuda", dtype=torch.float32)
-        d = torch.empty(M, K, device="cuda", dtype=torch.bfloat16)
+        qs = [torch.empty(M, K, device="cuda", dtype=torch.int8) for _ in range(NSETS)]
+        ss = [torch.empty(K // B, M, device="cuda", dtype=torch.float32) for _ in range(NSETS)]
+        ds = [torch.empty(M, K, device="cuda", dtype=torch.bfloat16) for _ in range(NSETS)]
+        turn = [0]
 
         def fq():
-            rc = lib.bi8_quantize_rowwise(x.data_ptr(), 1, q.data_ptr(), s.data_ptr(), M, K, K, K, B, st)
+            i = turn[0] = (turn[0] + 1) % NSETS
+            rc = lib.bi8_quantize_rowwise(xs[i].data_ptr(), 1, qs[i].data_ptr(), ss[i].data_ptr(), M, K, K, K, B, st)
             assert rc == 0
 
         def fd():
-            rc = lib.bi8_dequantize_rowwise(q.data_ptr(), s.data_ptr(), d.data_ptr(), 1, M, K, K, K, B, st)
+            i = turn[0] = (turn[0] + 1) % NSETS
+            rc = lib.bi8_dequantize_rowwise(qs[i].data_ptr(), ss[i].data_ptr(), ds[i].data_ptr(), 1, M, K, K, K, B, st)
             assert rc == 0
 
         for f in (fq, fd):
-            for _ in range(5):
+            for _ in range(2 * NSETS):
                 f()
         torch.cuda.synchronize()
         tq = min(event_ms(fq, iters) for _ in range(3))
         td = min(event_ms(fd, iters) for _ in range(3))
         nbytes = E * 3 + 4 * E // B                 # read 2 B + write 1 B per element (or the reverse) + scales
-        mse = ((d.float() - x.float()) ** 2).mean().item()
+        mse = ((ds[0].float() - xs[0].float()) ** 2).mean().item()
         out[f"block{B}"] = {
             "bytes": nbytes,
             "quantize_us": round(tq * 1e3, 2), "quantize_GBps": round(nbytes / tq / 1e6, 1),
@@ -82,23 +91,25 @@ def bench_quantize(pkg, torch, iters: int):
             "dequantize_frac_hbm": round(nbytes / td / 1e6 / HBM_PEAK_GBS, 4),
             "roundtrip_mse": mse,
         }
+        del qs, ss, ds
     return out
 
 
-def cpu_baseline(torch, xq_rows, wq, sx_rows, sw, B, budget_s: float = 20.0):
-    """the PyTorch CPU restatement of the reference math (oracle/oracle_torch.py) on a bounded row sample of the
-    same GEMM, on this host's cores"""
+def cpu_baseline(torch, xq, wq, sx, sw, B, chunk: int = 2048):
+    """the PyTorch CPU restatement of the reference math (oracle/oracle_torch.py) on this host's cores: the same
+    8192^3 problem, in row chunks so that the int32 partials of one chunk fit comfortably in memory"""
     from oracle import oracle_torch
-    rows = xq_rows.shape[0]
-    N, K = wq.shape
+    M, K = xq.shape
+    N = wq.shape[0]
     t0 = time.perf_counter()
-    oracle_torch.int8_matmul_block_dequantize(xq_rows, wq, sx_rows, sw, B, None, torch.bfloat16)
+    for r0 in range(0, M, chunk):
+        oracle_torch.int8_matmul_block_dequantize(xq[r0:r0 + chunk], wq, sx[:, r0:r0 + chunk].contiguous(), sw, B, None, torch.bfloat16)
     dt = time.perf_counter() - t0
     return {
-        "value": round(2.0 * rows * N * K / dt / 1e12, 4), "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"oracle/oracle_torch.py (PyTorch eager, fp32 bmm per K-block + fp32 rescale) on the first {rows} rows of the "
-                  f"same 8192^3 problem: {rows}x{N}x{K}, block {B}, bf16 out; {dt:.2f} s on {torch.get_num_threads()} threads "
-                  f"({os.cpu_count()} logical CPUs)",
+        "value": round(2.0 * M * N * K / dt / 1e12, 4), "unit": "TOPS", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"oracle/oracle_torch.py (PyTorch eager: fp32 bmm per K-block, exact for int8 codes, + fp32 rescale) on the whole "
+                  f"{M}x{N}x{K} problem, block {B}, bf16 out, in {M // chunk} row chunks: {dt:.1f} s on {torch.get_num_threads()} "
+                  f"threads ({os.cpu_count()} logical CPUs)",
     }
 
 
@@ -110,6 +121,9 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the GEMM (the metric is quoted at 8192)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-quantize", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a plain 256 MiB device-to-device copy 5 times (a kernel of known traffic, for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is a one-GPU path (no collectives, no sharding); run it with --gpus 1", file=sys.stderr)
@@ -126,6 +140,14 @@ def main():
     B = cfg.GROUP_SIZE
     assert B == 128 and cfg.INPUT_OUTPUT_TORCH_TYPE == torch.bfloat16
     S = args.size
+
+    if args.calibrate_copy:
+        src = torch.empty(256 * 1024 * 1024, device="cuda", dtype=torch.uint8).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     torch.manual_seed(0)
     x = torch.randn(S, S, device="cuda", dtype=torch.float32).to(torch.bfloat16)
@@ -163,14 +185,13 @@ def main():
                    "block": B, "out_dtype": "bf16"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": round(achieved / INT8_PEAK_TOPS, 4), "traffic": None,
-                     "kernel": "gemm_tile<256,256,4,2,128,bf16>", "ops_per_launch": ops_per_launch,
+                     "kernel": "gemm_tile<256,128,4,2,3,128,bf16> (256x128 tile, 8 waves, 3-deep LDS ring)", "ops_per_launch": ops_per_launch,
                      "avg_launch_ms": round(kern_ms, 4)},
     }
     if not args.no_quantize:
         res["quantize_roundtrip"] = bench_quantize(pkg, torch, 50)
     if not args.no_cpu_baseline:
-        rows = min(2048, S)
-        res["cpu_baseline"] = cpu_baseline(torch, xq[:rows].cpu(), wq.cpu(), sx[:, :rows].contiguous().cpu(), sw.cpu(), B)
+        res["cpu_baseline"] = cpu_baseline(torch, xq.cpu(), wq.cpu(), sx.cpu(), sw.cpu(), B)
     print(json.dumps(res))
 
 
