@@ -23,30 +23,50 @@ namespace {
 
 constexpr int kStageK = 128;       // bytes of K per LDS stage
 
-// Raw buffer resource over [base, base + bytes): loads beyond the end return zeros.
-typedef __amdgpu_buffer_rsrc_t bi8_rsrc;
+// Raw buffer resource (V#) over [base, base + bytes): loads beyond the end return zeros.
+typedef bi8_v4i bi8_rsrc;
 __device__ __forceinline__ bi8_rsrc bi8_make_rsrc(const void *base, int64_t bytes) {
+    const uint64_t a = (uint64_t)base;
     const int n = bytes > 0x7fffffffLL ? 0x7fffffff : (int)bytes;
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, n, 0x00020000);
+    // dword0-1: 48-bit base, stride 0; dword2: size in bytes; dword3: raw 32-bit-format buffer (gfx9 family)
+    return bi8_rsrc{(int)(uint32_t)a, (int)(uint32_t)((a >> 32) & 0xffffu), n, 0x00020000};
 }
-// 64 lanes x 16 (or 4) bytes from buffer offset voff + soff to LDS at lds_dst + lane * 16 (or 4); lds_dst and
-// soff are wave-uniform.
-__device__ __forceinline__ void bi8_buffer_to_lds16(bi8_rsrc r, void *lds_dst, uint32_t voff, uint32_t soff) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_dst, 16, voff, soff, 0, 0);
+__device__ __forceinline__ uint32_t bi8_lds_address(const void *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
 }
-__device__ __forceinline__ void bi8_buffer_to_lds4(bi8_rsrc r, void *lds_dst, uint32_t voff, uint32_t soff) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_dst, 4, voff, soff, 0, 0);
+// 64 lanes x 16 (or 4) bytes from buffer offset voff + soff straight into LDS at lds_addr + lane * 16 (or 4);
+// rsrc, lds_addr and soff are wave-uniform.  Written as inline asm on purpose: the loads complete
+// asynchronously and are fenced by this file's own `s_waitcnt vmcnt(n)`, which lets later stages stay in
+// flight across a barrier; through the compiler's builtin every barrier would wait for all of them.
+__device__ __forceinline__ void bi8_buffer_to_lds16(bi8_rsrc r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void bi8_buffer_to_lds4(bi8_rsrc r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff)
+                 : "memory", "m0");
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs.  Give XCD x the x-th contiguous eighth of a
 // tile order in which consecutive indices form kGroupM-row bands walked column by column.
 constexpr int kXcds = 8;
-constexpr int kGroupM = 4;
+#ifndef BI8_GROUP_M
+#define BI8_GROUP_M 4
+#endif
+constexpr int kGroupM = BI8_GROUP_M;
 __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tiles_n, int &tm, int &tn) {
     const int total = tiles_m * tiles_n;
     const int per = total / kXcds;                 // full rounds
     int idx;
+#ifdef BI8_NO_XCD_REMAP
+    if (false) idx = 0;
+#else
     if (pid < per * kXcds) idx = (pid % kXcds) * per + pid / kXcds;
+#endif
     else idx = pid;                                // remainder keeps its place at the end
     const int band = kGroupM * tiles_n;
     const int b = idx / band;
@@ -133,11 +153,11 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
     const int64_t a_rows = (g.M - m0 < BM) ? (g.M - m0) : BM, w_rows = (g.N - n0 < BN) ? (g.N - n0) : BN;
     const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
     const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
-    uint32_t a_off[kAIter], w_off[kWIter];
-#pragma unroll
-    for (int it = 0; it < kAIter; ++it) a_off[it] = (uint32_t)(((wave + it * NW) * 8 + ld_row) * g.lda + ld_chunk * 16);
-#pragma unroll
-    for (int it = 0; it < kWIter; ++it) w_off[it] = (uint32_t)(((wave + it * NW) * 8 + ld_row) * g.ldw + ld_chunk * 16);
+    // per-lane part of the offset (one register per operand); the rows of wave instruction `it` start
+    // (wave + it*NW) * 8 rows further down, which goes into the scalar offset together with the K position
+    const uint32_t a_off = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_off = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
+    const uint32_t a_wave = (uint32_t)(wave * 8 * g.lda), w_wave = (uint32_t)(wave * 8 * g.ldw);
+    const uint32_t a_step = (uint32_t)(NW * 8 * g.lda), w_step = (uint32_t)(NW * 8 * g.ldw);
     // scale rows: 64 floats per wave instruction; instruction i -> K-block i / kSPer of the stage, and inside
     // it the first BM/64 instructions fetch sA, the rest sW.  Waves beyond the last instruction repeat an
     // earlier one (same bytes to the same place) rather than branch around it.
@@ -148,41 +168,36 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
     const int64_t nblk = g.K / BLK;
     const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, PARTIALS ? 0 : ((nblk - 1) * g.M + (g.M - m0)) * 4);
     const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, PARTIALS ? 0 : ((nblk - 1) * g.N + (g.N - n0)) * 4);
-    uint32_t s_off[kSI];
+    uint32_t s_off[kSI], s_pos[kSI], s_inc[kSI];   // per-lane offset; scale-row position of the next stage and its step
     int s_dst[kSI], s_bufstep[kSI];
-    bool s_is_a[kSI];
+    bi8_rsrc s_rsrc[kSI];
 #pragma unroll
     for (int it = 0; it < kSIter; ++it) {
         const int i = (wave + it * NW) % (kSInstr > 0 ? kSInstr : 1);
         const int b = i / kSPer, r = i % kSPer;
-        s_is_a[it] = r < BM / 64;
-        if (s_is_a[it]) {
-            s_off[it] = (uint32_t)((b * g.M + r * 64 + lane) * 4);
-            s_dst[it] = L::kSAReg + (b * BM + r * 64) * 4;
-            s_bufstep[it] = L::kSABuf;
-        } else {
-            s_off[it] = (uint32_t)((b * g.N + (r - BM / 64) * 64 + lane) * 4);
-            s_dst[it] = L::kSWReg + (b * BN + (r - BM / 64) * 64) * 4;
-            s_bufstep[it] = L::kSWBuf;
-        }
+        const bool is_a = r < BM / 64;             // wave-uniform: everything below is selected, not branched
+        s_rsrc[it] = is_a ? sa_rsrc : sw_rsrc;
+        s_off[it] = is_a ? (uint32_t)((b * g.M + r * 64 + lane) * 4) : (uint32_t)((b * g.N + (r - BM / 64) * 64 + lane) * 4);
+        s_dst[it] = is_a ? L::kSAReg + (b * BM + r * 64) * 4 : L::kSWReg + (b * BN + (r - BM / 64) * 64) * 4;
+        s_bufstep[it] = is_a ? L::kSABuf : L::kSWBuf;
+        s_inc[it] = (uint32_t)(NBS * (is_a ? g.M : g.N) * 4);
+        s_pos[it] = 0;
     }
     uint32_t k_pos = 0;                            // K offset of the next stage to load (bytes)
-    uint32_t sa_pos = 0, sw_pos = 0;               // scale-row offsets of the next stage (bytes)
 
     constexpr int kLoadsPerStage = kAIter + kWIter + kSIter;     // VMEM instructions one wave issues per stage
+    const uint32_t lds_base = bi8_lds_address(lds);
     auto issue_stage = [&](int buf) {             // buf is wave-uniform: LDS destinations and K position are scalars
 #pragma unroll
-        for (int it = 0; it < kAIter; ++it) bi8_buffer_to_lds16(a_rsrc, lds + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024, a_off[it], k_pos);
+        for (int it = 0; it < kAIter; ++it) bi8_buffer_to_lds16(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024, a_off, k_pos + a_wave + it * a_step);
 #pragma unroll
-        for (int it = 0; it < kWIter; ++it) bi8_buffer_to_lds16(w_rsrc, lds + L::kWReg + buf * L::kWBuf + (wave + it * NW) * 1024, w_off[it], k_pos);
+        for (int it = 0; it < kWIter; ++it) bi8_buffer_to_lds16(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + it * NW) * 1024, w_off, k_pos + w_wave + it * w_step);
         k_pos += kStageK;
 #pragma unroll
         for (int it = 0; it < kSIter; ++it) {
-            if (s_is_a[it]) bi8_buffer_to_lds4(sa_rsrc, lds + s_dst[it] + buf * s_bufstep[it], s_off[it], sa_pos);
-            else bi8_buffer_to_lds4(sw_rsrc, lds + s_dst[it] + buf * s_bufstep[it], s_off[it], sw_pos);
+            bi8_buffer_to_lds4(s_rsrc[it], lds_base + s_dst[it] + buf * s_bufstep[it], s_off[it], s_pos[it]);
+            s_pos[it] += s_inc[it];
         }
-        sa_pos += (uint32_t)(NBS * g.M * 4);
-        sw_pos += (uint32_t)(NBS * g.N * 4);
     };
 
     // ---- operand fragment addresses (buffer 0).  Row r = ... + l32, 16-byte chunk (2*ks + h) ^ ((r >> 1) & 7):
@@ -346,20 +361,123 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
         }
     };
 
+    // vmcnt(n) alone: wait until at most n of this wave's VMEM instructions are outstanding
+    auto wait_vm = [&](auto pending_c) {
+        constexpr int kPending = decltype(pending_c)::value;
+        static_assert(kPending < 64, "vmcnt is a 6-bit field");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
+    };
+    using Drained = std::integral_constant<int, 0>;
+
+    constexpr bool kPipelined = !PARTIALS && NBS == 1 && TM == 2 && TN == 2 && kBufs == 2;
+    if constexpr (kPipelined) {
+        // ---- block-128 pipeline: two stage buffers, barrier in the MIDDLE of a stage ------------------------
+        // Stage s lives in buffer q = s & 1 and runs the four subtiles in the order (0,f) (0,g) (1,g) (1,f) with
+        // f = q, g = 1 - q.  All of its operands are in registers after the second subtile; then ONE barrier
+        // certifies for every wave that stage s+1 has landed and that buffer q is no longer read, the loads of
+        // stage s+2 start into buffer q, and the operands of stage s+1's first subtile (row subtile 0, column
+        // subtile g) are read during subtiles three and four into the registers that subtiles one and two have
+        // released.  No wave waits for LDS data right behind a barrier, the stage body is one basic block, and
+        // every LDS address is "base register + immediate".
+        // Stages past the end of K (the trip count is rounded up to even, and loads run two stages ahead) read
+        // their scales through the buffers' range check as zeros, so they add exactly 0 to the accumulators.
+        bi8_v4i A0[4], A1[4], Bq[2][4];
+        bi8_v4f sx0[4], sx1[4];
+        float sw2[2] = {0.0f, 0.0f}, swc2[2] = {0.0f, 0.0f}, pend_sw = 0.0f, pend_swc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sx0[i] = sx1[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        using InFlight1 = std::integral_constant<int, kLoadsPerStage>;
+
+        auto read_a = [&](bi8_v4i *dst, int a, int buf) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) dst[ks] = *(const bi8_v4i *)(lds + a_addr[ks] + buf * L::kABuf + a * 32 * kStageK);
+        };
+        auto read_w = [&](bi8_v4i *dst, int b, int buf) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) dst[ks] = *(const bi8_v4i *)(lds + w_addr[ks] + buf * L::kWBuf + b * 32 * kStageK);
+        };
+        auto read_sx = [&](bi8_v4f *dst, int a, int buf) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dst[i] = *(const bi8_v4f *)(lds + sa_addr + buf * L::kSABuf + (a * 32 + 8 * i) * 4);
+        };
+        // one subtile: four MFMAs, each followed by a slice of the previous subtile's fold
+        auto item = [&](bi8_v16i &pdst, const bi8_v4i *af, const bi8_v4i *wf, const bi8_v16i &psrc, const bi8_v4f *sx, float sw,
+                        float swcv, float *dst, bool fold_first) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                if (fold_first) fold_slice(psrc, sx, sw, swcv, dst, ks);
+                pdst = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[ks], wf[ks], ks == 0 ? magic : pdst, 0, 0, 0);
+                if (!fold_first) fold_slice(psrc, sx, sw, swcv, dst, ks);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        auto stage = [&](auto par_c) {
+            constexpr int F = decltype(par_c)::value, G = 1 - F;       // F is also this stage's buffer, G the next one's
+            // subtile (0,F): its operands were read during the previous stage
+            read_w(Bq[G], G, F);
+            read_sx(sx0, 0, F);
+            float swn[2];
+            swn[0] = *(const float *)(lds + sw_addr + F * L::kSWBuf);
+            swn[1] = *(const float *)(lds + sw_addr + F * L::kSWBuf + 32 * 4);
+            __builtin_amdgcn_sched_barrier(0);
+            item(p[0], A0, Bq[F], p[1], sx1, pend_sw, pend_swc, acc[1][G], true);      // folds the previous stage's (1,G)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {          // column scales -> 22 significant bits, and -(1.5*2^23) times them
+                sw2[b] = bi8_u2f((bi8_f2u(swn[b]) + 2u) & ~3u);
+                swc2[b] = -BI8_MAGIC * sw2[b];
+            }
+            // subtile (0,G)
+            read_a(A1, 1, F);
+            read_sx(sx1, 1, F);
+            __builtin_amdgcn_sched_barrier(0);
+            item(p[1], A0, Bq[G], p[0], sx0, sw2[F], swc2[F], acc[0][F], false);
+            // every operand of this stage is in registers (or on its way: lgkmcnt below); synchronize
+            __builtin_amdgcn_s_waitcnt(0xC07F);    // lgkmcnt(0) only
+            wait_vm(Drained{});                    // this wave's loads of stage s+1 have landed
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            issue_stage(F);                        // stage s+2 into the buffer just released
+            // subtile (1,G), meanwhile the next stage's row subtile 0
+            read_a(A0, 0, G);
+            __builtin_amdgcn_sched_barrier(0);
+            item(p[0], A1, Bq[G], p[1], sx0, sw2[G], swc2[G], acc[0][G], false);
+            // subtile (1,F), meanwhile the next stage's column subtile G (its first)
+            read_w(Bq[G], G, G);
+            __builtin_amdgcn_sched_barrier(0);
+            item(p[1], A1, Bq[F], p[0], sx1, sw2[G], swc2[G], acc[1][G], false);
+            pend_sw = sw2[F];
+            pend_swc = swc2[F];
+        };
+        using P0 = std::integral_constant<int, 0>;
+        using P1 = std::integral_constant<int, 1>;
+        // prologue: two stages of loads, wait for the first, read the first subtile's operands
+        issue_stage(0);
+        issue_stage(1);
+        wait_vm(InFlight1{});
+        __syncthreads();
+        read_a(A0, 0, 0);
+        read_w(Bq[0], 0, 0);
+        for (int s = 0; s < nstages; s += 2) {
+            stage(P0{});
+            stage(P1{});
+        }
+        wait_vm(Drained{});                        // nothing may still be writing LDS when the wave ends
+        // the last subtile of the last (possibly padding) stage: always (1,1)
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) fold_slice(p[1], sx1, pend_sw, pend_swc, acc[1][1], ks);
+    } else {
+    // ---- generic pipeline: barrier at the top of every stage ---------------------------------------------------
     // Ring of kBufs stage buffers.  Before computing stage s every wave waits until only the loads of later
     // stages are still outstanding (its own direct-to-LDS loads of stage s have landed), then the barrier makes
     // that true for all waves and frees the buffer computed one stage earlier.
     auto sync_stage = [&](auto pending_c) {
-        constexpr int kPending = decltype(pending_c)::value;       // VMEM instructions allowed to stay in flight
-        static_assert(kPending < 64, "vmcnt is a 6-bit field");
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));   // vmcnt(kPending) only
+        wait_vm(pending_c);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
     };
     // kBufs - 1 stages of loads are in flight while one stage is computed
     using InFlight = std::integral_constant<int, (kBufs - 2) * kLoadsPerStage>;
-    using Drained = std::integral_constant<int, 0>;
 #pragma unroll
     for (int q = 0; q < kBufs - 1; ++q)
         if (q < nstages) issue_stage(q);
@@ -380,6 +498,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
 #pragma unroll
         for (int ks = 0; ks < KSB; ++ks)
             fold_slice(p[(NITEM - 1) & 1], sxv[(NBS - 1) & 1][TM - 1], swv[(NBS - 1) & 1][TN - 1], swc[(NBS - 1) & 1][TN - 1], acc[TM - 1][TN - 1], ks);
+    }
 
     if constexpr (!PARTIALS) {
         const float div = (float)(1.0 / (127.0 * 127.0));
@@ -503,7 +622,7 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
 #endif
     if constexpr (kBigFits) {
         const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
-        if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, 3, BLK, CDT, PARTIALS>(g, st);
+        if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : 3, BLK, CDT, PARTIALS>(g, st);
     }
     if (g.M > 64) return launch_tile<128, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
     return launch_tile<64, 128, 1, 2, 3, BLK, CDT, PARTIALS>(g, st);
