@@ -519,6 +519,87 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
     }
 }
 
+// Skinny GEMM (M <= 32), HBM-bound on W: the whole problem is one pass over the N*K bytes of weight codes.
+// One workgroup = 32 output columns, 8 waves that split K in interleaved 128-byte stages; every wave gathers its
+// MFMA operands straight from global memory in operand layout (16 bytes per lane; the four k-steps of a stage
+// touch each 128-byte line of a weight row once), folds each K-block into 16 fp32 accumulators per lane, and the
+// eight partial accumulators are summed through LDS in wave order (deterministic).  Rows m >= M are zero operands.
+template <int BLK, int CDT>
+__global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
+    constexpr int NW = 8;
+    constexpr int NBS = kStageK / BLK, KSB = BLK / 32;
+    __shared__ float red[NW][16][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int l32 = lane & 31, h = lane >> 5;
+    const int64_t n0 = (int64_t)blockIdx.x * 32;
+    const int64_t n = n0 + l32;
+    const int64_t nc = n < g.N ? n : g.N - 1;                      // clamped: never stored
+    const int64_t mc = l32 < g.M ? l32 : g.M - 1;
+    const bool m_ok = l32 < g.M;
+    const int8_t *wrow = g.W + nc * g.ldw + h * 16;
+    const int8_t *arow = g.A + mc * g.lda + h * 16;
+    const int nstages = (int)(g.K / kStageK);
+    float acc[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    // row indices of this lane's 16 accumulators (clamped for the scale loads)
+    int64_t rowc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rowc[i] = (8 * i + 4 * h + 3 < g.M) ? (8 * i + 4 * h) : -1;
+
+    auto load_stage = [&](int s, bi8_v4i *wf, bi8_v4i *af) {
+        const int64_t k0 = (int64_t)s * kStageK;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            wf[ks] = __builtin_nontemporal_load((const bi8_v4i *)(wrow + k0 + ks * 32));
+            af[ks] = m_ok ? *(const bi8_v4i *)(arow + k0 + ks * 32) : bi8_v4i{0, 0, 0, 0};
+        }
+    };
+    bi8_v4i wf[2][4], af[2][4];
+    int s = wave;
+    if (s < nstages) load_stage(s, wf[0], af[0]);
+    int cur = 0;
+    for (; s < nstages; s += NW, cur ^= 1) {
+        if (s + NW < nstages) load_stage(s + NW, wf[cur ^ 1], af[cur ^ 1]);      // next stage of this wave in flight
+#pragma unroll
+        for (int blk = 0; blk < NBS; ++blk) {
+            const int64_t jb = (int64_t)s * NBS + blk;
+            const float sw = g.sW[jb * g.N + nc];
+            bi8_v16i p = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < KSB; ++ks)
+                p = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[cur][blk * KSB + ks], wf[cur][blk * KSB + ks], p, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int row = 8 * i + 4 * h + j;
+                    const float sx = (row < g.M) ? g.sA[jb * g.M + row] : 0.0f;
+                    acc[4 * i + j] = __builtin_fmaf((float)p[4 * i + j] * sx, sw, acc[4 * i + j]);
+                }
+            }
+        }
+    }
+    (void)rowc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
+    __syncthreads();
+    if (wave == 0) {
+        const float div = (float)(1.0 / (127.0 * 127.0));
+        const bool has_bias = g.bias != nullptr;
+        const float bias = (has_bias && n < g.N) ? load_bias(g, n) : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float v = red[0][r][lane];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) v += red[w][r][lane];
+            const int64_t m = 8 * (r >> 2) + 4 * h + (r & 3);
+            if (m < g.M && n < g.N) store_c<CDT>(g.C, m * g.ldc + n, v * div, has_bias, bias);
+        }
+    }
+}
+
 // Fallback for any K, block, alignment: 4 waves, each a 32x32 output subtile; every lane gathers its own
 // 16-byte MFMA operands with byte loads (zero outside the matrix and outside the current K-block).
 template <int CDT, bool PARTIALS>
@@ -628,9 +709,25 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
     return launch_tile<64, 128, 1, 2, 3, BLK, CDT, PARTIALS>(g, st);
 }
 
+template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {
+    const int64_t tn = (g.N + 31) / 32;
+    if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((gemm_skinny<BLK, CDT>), dim3((unsigned)tn), dim3(512), 0, st, g);
+    return bi8_launch_rc();
+}
+
 template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hipStream_t st) {
     const bool tile_ok = g.K % kStageK == 0 && g.lda % 16 == 0 && g.ldw % 16 == 0 && bi8_aligned(g.A, 16) && bi8_aligned(g.W, 16) &&
                          (PARTIALS || (bi8_aligned(g.sA, 4) && bi8_aligned(g.sW, 4)));
+    if constexpr (!PARTIALS) {
+        if (tile_ok && g.M <= 32) {
+            switch (block) {
+            case 32: return launch_skinny<32, CDT>(g, st);
+            case 64: return launch_skinny<64, CDT>(g, st);
+            case 128: return launch_skinny<128, CDT>(g, st);
+            }
+        }
+    }
     if (tile_ok) {
         switch (block) {
         case 32: return pick_tile<32, CDT, PARTIALS>(g, st);

@@ -24,6 +24,26 @@ def _stream(t: torch.Tensor) -> int:
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *a):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+_multi_device = None
+
+
+def _on_device(t: torch.Tensor):
+    """Context that makes t's device current for the launch; free on a one-GPU machine."""
+    global _multi_device
+    if _multi_device is None:
+        _multi_device = torch.cuda.device_count() > 1
+    return torch.cuda.device(t.device) if _multi_device else _NO_GUARD
+
+
 def _float_operand(x: torch.Tensor) -> torch.Tensor:
     if x.dtype not in _DT:
         raise TypeError(f"unsupported dtype {x.dtype}: expected float32, bfloat16 or float16")
@@ -60,7 +80,7 @@ def quantize_block_rowwise(x: torch.Tensor, fblock_size=None):
     output = torch.empty((m, k), device=x.device, dtype=torch.int8)
     # output_maxs is transposed: block-major, row-minor (:226-227)
     output_maxs = torch.empty((ceil_div(k, fblock_size), m), device=x.device, dtype=torch.float32)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         rc = _lib.load().bi8_quantize_rowwise(x.data_ptr(), _DT[x.dtype], output.data_ptr(), output_maxs.data_ptr(),
                                               m, k, _ld(x), max(k, 1), fblock_size, _stream(x))
     _lib.check(rc, "bi8_quantize_rowwise")
@@ -76,7 +96,7 @@ def quantize_block_transposed(x: torch.Tensor, fblock_size=None):
     x = _rows(_float_operand(x))
     output = torch.empty((c, r), device=x.device, dtype=torch.int8)
     output_maxs = torch.empty((ceil_div(r, fblock_size), c), device=x.device, dtype=torch.float32)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         rc = _lib.load().bi8_quantize_transposed(x.data_ptr(), _DT[x.dtype], output.data_ptr(), output_maxs.data_ptr(),
                                                  r, c, _ld(x), max(r, 1), fblock_size, _stream(x))
     _lib.check(rc, "bi8_quantize_transposed")
@@ -94,7 +114,7 @@ def dequantize_block_rowwise(x: torch.Tensor, state_x: torch.Tensor, fblock_size
     x = _rows(x)
     state_x = _scales_in(state_x)
     output = torch.empty((M, K), device=x.device, dtype=out_dtype)
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         rc = _lib.load().bi8_dequantize_rowwise(x.data_ptr(), state_x.data_ptr(), output.data_ptr(), _DT[out_dtype],
                                                 M, K, _ld(x), max(K, 1), fblock_size, _stream(x))
     _lib.check(rc, "bi8_dequantize_rowwise")
@@ -132,7 +152,7 @@ def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
             bias = bias.float()
         bias = bias.contiguous()
         bias_ptr, bias_dt = bias.data_ptr(), _DT[bias.dtype]
-    with torch.cuda.device(a.device):
+    with _on_device(a):
         rc = _lib.load().bi8_gemm_nt_dequant(a.data_ptr(), w.data_ptr(), state_x.data_ptr(), state_w.data_ptr(),
                                              bias_ptr, bias_dt, c.data_ptr(), _DT[out_dtype], M, N, K,
                                              _ld(a), _ld(w), max(N, 1), block, _stream(a))
@@ -148,7 +168,7 @@ def int8_matmul_block_partials(a, b, fblock_size=None):
     M, K = a.shape
     N = w.shape[0]
     p = torch.empty((ceil_div(K, block), M, N), device=a.device, dtype=torch.int32)
-    with torch.cuda.device(a.device):
+    with _on_device(a):
         rc = _lib.load().bi8_gemm_nt_partials(a.data_ptr(), w.data_ptr(), p.data_ptr(), M, N, K, _ld(a), _ld(w),
                                               block, _stream(a))
     _lib.check(rc, "bi8_gemm_nt_partials")
