@@ -1,13 +1,15 @@
 // Block dequantize (bi8_dequantize_rowwise): out = (scale * float(code)) * fp32(1/127), cast on store.
 // Replaces _dequantize_block_rowwise, triton_functions.py:468-490.  HBM-bound: one lane = one 128-bit store
 // of outputs (8 bf16/f16 or 4 fp32) per step, so every wave store covers 1 KiB of contiguous output.  Same
-// tiling as the quantizer: a workgroup owns 16 rows x 2 KiB of output row and first pulls its scales in
-// through LDS, so the block-major / row-minor scale array is read as runs of 16 consecutive rows.
+// tiling as the quantizer: a workgroup owns 8 rows x 2 KiB of output row and first pulls its scales in
+// through LDS, so the block-major / row-minor scale array is read as runs of 8 consecutive rows.
 #include "bi8_common.h"
 
 namespace {
 
-constexpr int kRows = 16;
+constexpr int kLoads = 4;          // wave-loads per lane per tile (8 and 16 measured slower)
+constexpr int kRpw = kLoads / 2;   // rows per wave
+constexpr int kRows = 4 * kRpw;    // rows per workgroup tile
 constexpr int kThreads = 256;
 
 // One lane = kOut outputs = one 16-byte store (8 bf16/f16 or 4 fp32), so every store instruction of a wave
@@ -38,9 +40,8 @@ template <int DT> __device__ __forceinline__ void store_vec(void *out, int64_t i
     }
 }
 
-constexpr int kLoads = 8;          // wave-loads per lane per tile
 
-// workgroup tile: 16 rows x (2 * 64 * kOut) codes; wave w owns rows 4w .. 4w+3, two chunks of 64 * kOut codes each
+// workgroup tile: 8 rows x (2 * 64 * kOut) codes; wave w owns rows 2w, 2w+1, two chunks of 64 * kOut codes each
 template <int DT>
 __global__ __launch_bounds__(kThreads) void dequantize_rows_vec(const int8_t *__restrict__ q, const float *__restrict__ scales,
                                                                 void *__restrict__ out, int64_t M, int64_t K, int64_t ldq,
@@ -61,7 +62,7 @@ __global__ __launch_bounds__(kThreads) void dequantize_rows_vec(const int8_t *__
     uint32_t raw[kLoads][VEC / 4];
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
-        const int64_t row = row0 + wave * 4 + (i >> 1);
+        const int64_t row = row0 + wave * kRpw + (i >> 1);
         const int64_t col = col0 + ((i & 1) * BI8_WAVE + lane) * VEC;
 #pragma unroll
         for (int e = 0; e < VEC / 4; ++e) raw[i][e] = 0u;
@@ -86,11 +87,11 @@ __global__ __launch_bounds__(kThreads) void dequantize_rows_vec(const int8_t *__
     const float inv127 = (float)(1.0 / 127.0);
 #pragma unroll
     for (int i = 0; i < kLoads; ++i) {
-        const int64_t row = row0 + wave * 4 + (i >> 1);
+        const int64_t row = row0 + wave * kRpw + (i >> 1);
         const int incol = ((i & 1) * BI8_WAVE + lane) * VEC;
         const int64_t col = col0 + incol;
         if (row < M && col < K) {
-            const float s = s_tile[incol >> log2b][wave * 4 + (i >> 1)];
+            const float s = s_tile[incol >> log2b][wave * kRpw + (i >> 1)];
             float v[VEC];
 #pragma unroll
             for (int e = 0; e < VEC / 4; ++e) {

@@ -4,14 +4,15 @@
 // runs of 16 consecutive rows (the scale array is block-major / row-minor).
 //
 // Replaces _quantize_block_rowwise, triton_functions.py:193-216 (one program per row, serial over the
-// row's blocks) with a 2-D tiling: one workgroup = 16 rows x 2 KiB of row, one lane = 16 input bytes,
+// row's blocks) with a 2-D tiling: one workgroup = 16 rows x 1 KiB of row, one lane = 16 input bytes,
 // one K-block = L adjacent lanes (L = block * sizeof(elem) / 16), absmax by DPP inside the lane group.
 #include "bi8_common.h"
 
 namespace {
 
-constexpr int kRows = 16;          // rows per workgroup tile
-constexpr int kChunks = 2;         // 1 KiB wave-loads per row per tile
+constexpr int kRowsPerWave = 4;            // = 16-byte loads in flight per lane; 2 and 8 both measured slower
+constexpr int kRows = 4 * kRowsPerWave;    // rows per workgroup tile
+constexpr int kChunks = 1;                 // 1 KiB wave-loads per row per tile (2 and 4 measured slower)
 constexpr int kThreads = 256;
 
 template <int DT> struct Vec {
@@ -59,10 +60,10 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_vec(const void *__rest
     const int64_t col0 = (int64_t)tile_k * TE;
     const char *xb = (const char *)x;
 
-    bi8_v4u raw[4][kChunks];
+    bi8_v4u raw[kRowsPerWave][kChunks];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t row = row0 + wave * 4 + i;
+    for (int i = 0; i < kRowsPerWave; ++i) {
+        const int64_t row = row0 + wave * kRowsPerWave + i;
 #pragma unroll
         for (int c = 0; c < kChunks; ++c) {
             const int64_t col = col0 + (c * BI8_WAVE + lane) * VEC;
@@ -74,8 +75,8 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_vec(const void *__rest
     }
 
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int64_t row = row0 + wave * 4 + i;
+    for (int i = 0; i < kRowsPerWave; ++i) {
+        const int64_t row = row0 + wave * kRowsPerWave + i;
 #pragma unroll
         for (int c = 0; c < kChunks; ++c) {
             const int64_t col = col0 + (c * BI8_WAVE + lane) * VEC;
@@ -89,7 +90,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_vec(const void *__rest
                 special |= (f[e] != f[e]);
             }
             m = bi8_group_max<L>(m);
-            if ((lane & (L - 1)) == 0) s_tile[(c * BI8_WAVE + lane) / L][wave * 4 + i] = m;
+            if ((lane & (L - 1)) == 0) s_tile[(c * BI8_WAVE + lane) / L][wave * kRowsPerWave + i] = m;
             special |= !bi8_scale_is_ordinary(m);
 
             uint32_t code[VEC];

@@ -155,6 +155,52 @@ def test_operand_layouts(ops):
             ops.int8_matmul_block64_rowwise_dequantize(A, W[:, :-1].t(), sa, sw)
 
 
+# decode-like shapes (few rows): (M, N, K); K a multiple of 128 selects the few-row kernel, 200 and 1000 do not
+FEW_ROWS = [(1, 32, 128), (1, 4096, 4096), (2, 33, 256), (7, 1000, 1152), (16, 4096, 1024), (31, 500, 2048),
+            (32, 96, 8192), (32, 2049, 384), (5, 300, 200), (32, 64, 1000)]
+
+
+@pytest.mark.parametrize("shape", FEW_ROWS)
+@pytest.mark.parametrize("block", [32, 64, 128])
+def test_few_rows_parity(ops, shape, block):
+    """M <= 32 (one token / a small decode batch): outputs against the checker for every output dtype, bias as an
+    exact identity, and row r of a batch equal to the same row computed alone (no cross-row leakage)"""
+    M, N, K = shape
+    g = torch.Generator().manual_seed(7 * M + N + K + block)
+    A, W = _codes(g, M, K), _codes(g, N, K)
+    nblk = -(-K // block)
+    sa = torch.rand(nblk, M, generator=g) * 4 + 0.01
+    sw = torch.rand(nblk, N, generator=g) * 0.1 + 1e-4
+    sa[nblk // 2, M // 2] = 0.0                                    # an all-zero block has scale 0
+    bias = torch.randn(N, generator=g)
+    Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
+    for out in ("f32", "bf16", "f16"):
+        _, ref, mag = _reference(A, W, sa, sw, block, None, DTYPES[out])
+        with cfg_as(ops, block, DTYPES[out]):
+            C = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sad, swd)
+            Cb = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sad, swd, bias.to(DEV))
+            r = M - 1
+            Cr = ops.int8_matmul_block64_rowwise_dequantize(Ad[r:r + 1], Wd.t(), sad[:, r:r + 1].contiguous(), swd)
+        assert C.dtype == DTYPES[out] and C.shape == (M, N)
+        _assert_close(C.cpu(), ref, mag, TOL[out])
+        assert torch.equal(Cb, C + bias.to(DEV).to(DTYPES[out]))
+        assert torch.equal(Cr[0], C[r])
+
+
+def test_few_rows_operand_views(ops):
+    """few-row kernel on operands that are column slices of wider buffers (leading dimension > K)"""
+    g = torch.Generator().manual_seed(11)
+    M, N, K, B = 8, 200, 512, 128
+    Abig, Wbig = _codes(g, M, K + 64).to(DEV), _codes(g, N, K + 48).to(DEV)
+    sa = torch.rand(K // B, M, generator=g).to(DEV); sw = torch.rand(K // B, N, generator=g).to(DEV)
+    with cfg_as(ops, B, torch.float32):
+        A, W = Abig[:, 16:16 + K], Wbig[:, 32:32 + K]
+        base = ops.int8_matmul_block64_rowwise_dequantize(A.contiguous(), W.contiguous().t(), sa, sw)
+        assert torch.equal(ops.int8_matmul_block64_rowwise_dequantize(A, W.t(), sa, sw), base)
+        _, ref, mag = _reference(A.cpu(), W.cpu(), sa.cpu(), sw.cpu(), B, None, torch.float32)
+        _assert_close(base.cpu(), ref, mag, TOL["f32"])
+
+
 def test_end_to_end_vs_dense_config1(ops):
     """X fp32 [256,1024] ~N(0,1); W fp32 [1024,1024] ~N(0,0.02); block 64; fp32 out, compared to the fp32
     matmul and to the checker's forward."""
