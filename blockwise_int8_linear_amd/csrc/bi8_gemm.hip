@@ -519,6 +519,228 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
     }
 }
 
+// ---- 256x256 tile, block 128 ------------------------------------------------------------------------------------
+// The large-problem kernel.  Twice the output per byte of operand moved from L2 to LDS compared to the 256x128
+// tile, which is what bounds gemm_tile at large sizes.  8 waves as 4 (rows) x 2 (columns); one wave owns 64 x 128
+// outputs as 4 x 8 subtiles of 16x16 (v_mfma_i32_16x16x64_i8: four accumulator registers per subtile, so the
+// int32 partials in flight cost 16 registers and the row scales of a stage 16), 128 fp32 accumulators per lane.
+// Per stage (128 bytes of K = one K-block) a wave keeps its 64 rows of A in registers and streams the eight
+// column subtiles of W through two register buffers, one column ahead.  Work is issued in "pairs" (two row
+// subtiles of one column = four MFMAs); each MFMA is followed by a quarter of the fold of the previous pair, so the
+// matrix pipe and the vector ALU overlap.  Two LDS stage buffers, ONE barrier per stage, placed where the last
+// operand of the stage has been read (top of the eighth column): it certifies that the next stage has landed
+// and releases this stage's buffer to the loads of the stage after next.
+struct WideLds {
+    static constexpr int kABuf = 256 * kStageK, kWBuf = 256 * kStageK;       // 32 KiB per operand per stage
+    static constexpr int kSBuf = 256 * 4;                                    // one scale row of the tile
+    static constexpr int kAReg = 0;
+    static constexpr int kWReg = kAReg + 2 * kABuf;
+    static constexpr int kSAReg = kWReg + 2 * kWBuf;
+    static constexpr int kSWReg = kSAReg + 2 * kSBuf;
+    static constexpr int kBytes = kSWReg + 2 * kSBuf;                        // 132 KiB of the CU's 160
+};
+
+template <int CDT>
+__global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
+    using L = WideLds;
+    constexpr int BM = 256, BN = 256, NW = 8;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int r16 = lane & 15, q = lane >> 4;
+
+    int tile_m, tile_n;
+    tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int nstages = (int)(g.K / kStageK);
+
+    // ---- loader (same scheme as gemm_tile): wave instruction i covers tile rows 8i .. 8i+7, lane -> row
+    // 8i + lane/8, LDS chunk lane%8, which holds source chunk (lane%8) ^ ((row >> 1) & 7); i = wave + 8*it.
+    const int ld_row = lane >> 3;
+    const int ld_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+    const int64_t a_rows = (g.M - m0 < BM) ? (g.M - m0) : BM, w_rows = (g.N - n0 < BN) ? (g.N - n0) : BN;
+    const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
+    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
+    const uint32_t a_off = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_off = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
+    const uint32_t a_wave = (uint32_t)(wave * 8 * g.lda), w_wave = (uint32_t)(wave * 8 * g.ldw);
+    const uint32_t a_step = (uint32_t)(NW * 8 * g.lda), w_step = (uint32_t)(NW * 8 * g.ldw);
+    // scale rows of the stage's K-block: waves 0-3 fetch 64 row scales each, waves 4-7 64 column scales each
+    const int64_t nblk = g.K / 128;
+    const bool s_is_a = wave < 4;
+    const int s_part = wave & 3;
+    const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
+    const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
+    const bi8_rsrc s_rsrc = s_is_a ? sa_rsrc : sw_rsrc;
+    const uint32_t s_off = (uint32_t)((s_part * 64 + lane) * 4);
+    const uint32_t s_dst = (uint32_t)((s_is_a ? L::kSAReg : L::kSWReg) + s_part * 256);
+    const uint32_t s_inc = (uint32_t)((s_is_a ? g.M : g.N) * 4);
+    uint32_t s_pos = 0, k_pos = 0;                 // scale-row and K position of the next stage to load
+    constexpr int kLoadsPerStage = 4 + 4 + 1;
+
+    const uint32_t lds_base = bi8_lds_address(lds);
+    auto issue_stage = [&](int buf) {
+#pragma unroll
+        for (int it = 0; it < 4; ++it) bi8_buffer_to_lds16(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024, a_off, k_pos + a_wave + it * a_step);
+#pragma unroll
+        for (int it = 0; it < 4; ++it) bi8_buffer_to_lds16(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + it * NW) * 1024, w_off, k_pos + w_wave + it * w_step);
+        bi8_buffer_to_lds4(s_rsrc, lds_base + s_dst + buf * L::kSBuf, s_off, s_pos);
+        k_pos += kStageK;
+        s_pos += s_inc;
+    };
+
+    // ---- operand fragments: lane -> row r16 of a 16-row subtile, 16-byte chunk 4*kb + q of the stage's eight;
+    // stored at chunk position (4*kb + q) ^ ((row >> 1) & 7) and (row >> 1) & 7 = r16 >> 1 for every subtile,
+    // so the address of kb = 1 is the address of kb = 0 with bit 6 flipped.
+    int a_base[2], w_base[2];
+    a_base[0] = L::kAReg + (wm * 64 + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
+    w_base[0] = L::kWReg + (wn * 128 + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
+    a_base[1] = a_base[0] ^ 64;
+    w_base[1] = w_base[0] ^ 64;
+    // a subtile's outputs: lane -> column r16, rows 4q .. 4q+3
+    const int sa_base = L::kSAReg + (wm * 64 + 4 * q) * 4;
+    const int sw_base = L::kSWReg + (wn * 128 + r16) * 4;
+
+    float acc[4][8][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+
+    constexpr int kMagicBits = 0x4B400000;        // bit pattern of 1.5 * 2^23
+    const bi8_v4i magic = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
+    bi8_v4i A[4][2], Bf[2][2];                     // [row subtile][kb], [column parity][kb]
+    bi8_v4i c[2][2];                               // int32 partials: [pair parity][row subtile of the pair]
+    bi8_v4f sx[4];                                 // row scales per row subtile
+    float swb[2] = {0.0f, 0.0f}, swc[2] = {0.0f, 0.0f}, swr[2] = {0.0f, 0.0f};   // per column parity: b, -(1.5*2^23)*b, raw
+    c[0][0] = c[0][1] = c[1][0] = c[1][1] = magic;  // "partial 0" for the fold that precedes the first pair
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sx[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto read_a = [&](bi8_v4i *dst, int i, int buf) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) dst[kb] = *(const bi8_v4i *)(lds + a_base[kb] + buf * L::kABuf + i * 16 * kStageK);
+    };
+    auto read_b = [&](bi8_v4i *dst, float &raw, int j, int buf) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) dst[kb] = *(const bi8_v4i *)(lds + w_base[kb] + buf * L::kWBuf + j * 16 * kStageK);
+        raw = *(const float *)(lds + sw_base + buf * L::kSBuf + j * 16 * 4);
+    };
+    auto read_sx = [&](bi8_v4f &dst, int i, int buf) { dst = *(const bi8_v4f *)(lds + sa_base + buf * L::kSBuf + i * 16 * 4); };
+    // two elements of a finished partial: fma(f, b, c) = fl(b * P) (the partial carries the 1.5*2^23 offset), then
+    // the row scale and the accumulation
+    auto fold2 = [&](const bi8_v4i &pt, int r0, const bi8_v4f &s, float b, float cm, float *dst) {
+#pragma unroll
+        for (int r = r0; r < r0 + 2; ++r) {
+            const float u = __builtin_fmaf(bi8_u2f((uint32_t)pt[r]), b, cm);
+            dst[r] = __builtin_fmaf(u, s[r], dst[r]);
+        }
+    };
+    // one pair = row subtiles (a0, a1) of one column: four MFMAs, each followed by a quarter of the previous pair's fold
+    auto pair = [&](bi8_v4i *cn, const bi8_v4i *a0, const bi8_v4i *a1, const bi8_v4i *b, const bi8_v4i *cp, const bi8_v4f &s0,
+                    const bi8_v4f &s1, float fb, float fc, float *d0, float *d1) {
+        cn[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b[0], magic, 0, 0, 0);
+        fold2(cp[0], 0, s0, fb, fc, d0);
+        __builtin_amdgcn_sched_barrier(0);
+        cn[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[0], b[0], magic, 0, 0, 0);
+        fold2(cp[0], 2, s0, fb, fc, d0);
+        __builtin_amdgcn_sched_barrier(0);
+        cn[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b[1], cn[0], 0, 0, 0);
+        fold2(cp[1], 0, s1, fb, fc, d1);
+        __builtin_amdgcn_sched_barrier(0);
+        cn[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[1], b[1], cn[1], 0, 0, 0);
+        fold2(cp[1], 2, s1, fb, fc, d1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto wait_vm = [&](auto pending_c) {
+        constexpr int kPending = decltype(pending_c)::value;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
+    };
+
+    // On entry to a stage (buffer F): A[0], A[1], Bf[0], swr[0] already hold this stage's row subtiles 0, 1 and
+    // column 0 (read during the previous stage's last column); c[1] is the previous stage's last pair (rows 2, 3
+    // of column 7), still to be folded with the OLD sx[2], sx[3], swb[1], swc[1].
+    auto stage = [&](auto buf_c) {
+        constexpr int F = decltype(buf_c)::value, G = 1 - F;
+        read_a(A[2], 2, F);
+        read_a(A[3], 3, F);
+        read_sx(sx[0], 0, F);
+        read_sx(sx[1], 1, F);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            constexpr int kPrevCol[8] = {7, 0, 1, 2, 3, 4, 5, 6};
+            const int jb = j & 1;
+            swb[jb] = bi8_u2f((bi8_f2u(swr[jb]) + 2u) & ~3u);      // column scale -> 22 significant bits
+            swc[jb] = -BI8_MAGIC * swb[jb];                        // exact
+            if (j < 7) {
+                read_b(Bf[jb ^ 1], swr[jb ^ 1], j + 1, F);
+            } else {
+                // every operand of this stage is in registers or on its way (lgkmcnt): synchronize
+                __builtin_amdgcn_s_waitcnt(0xC07F);                // lgkmcnt(0) only
+                wait_vm(std::integral_constant<int, 0>{});         // this wave's loads of the next stage have landed
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                issue_stage(F);                                    // the stage after next, into the buffer just released
+                read_b(Bf[0], swr[0], 0, G);                       // the next stage's column 0
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // rows 0, 1 of column j; meanwhile fold rows 2, 3 of the column before
+            pair(c[0], A[0], A[1], Bf[jb], c[1], sx[2], sx[3], swb[jb ^ 1], swc[jb ^ 1], acc[2][kPrevCol[j]], acc[3][kPrevCol[j]]);
+            if (j == 0) {
+                read_sx(sx[2], 2, F);
+                read_sx(sx[3], 3, F);
+            }
+            if (j == 7) {                                          // the next stage's row subtiles 0, 1
+                read_a(A[0], 0, G);
+                read_a(A[1], 1, G);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // rows 2, 3 of column j; meanwhile fold rows 0, 1 of column j
+            pair(c[1], A[2], A[3], Bf[jb], c[0], sx[0], sx[1], swb[jb], swc[jb], acc[0][j], acc[1][j]);
+        }
+    };
+
+    // prologue: two stages of loads, wait for the first, read the first pair's operands
+    issue_stage(0);
+    issue_stage(1);
+    wait_vm(std::integral_constant<int, kLoadsPerStage>{});
+    __syncthreads();
+    read_a(A[0], 0, 0);
+    read_a(A[1], 1, 0);
+    read_b(Bf[0], swr[0], 0, 0);
+    // The trip count is rounded up to even and loads run two stages ahead: stages past the end of K read their
+    // scales through the buffers' range check as zeros, so they add exactly 0 to the accumulators.
+    for (int s = 0; s < nstages; s += 2) {
+        stage(std::integral_constant<int, 0>{});
+        stage(std::integral_constant<int, 1>{});
+    }
+    wait_vm(std::integral_constant<int, 0>{});     // nothing may still be writing LDS when the wave ends
+    fold2(c[1][0], 0, sx[2], swb[1], swc[1], acc[2][7]);
+    fold2(c[1][0], 2, sx[2], swb[1], swc[1], acc[2][7]);
+    fold2(c[1][1], 0, sx[3], swb[1], swc[1], acc[3][7]);
+    fold2(c[1][1], 2, sx[3], swb[1], swc[1], acc[3][7]);
+
+    const float div = (float)(1.0 / (127.0 * 127.0));
+    const bool has_bias = g.bias != nullptr;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int64_t n = n0 + wn * 128 + j * 16 + r16;
+        const bool n_ok = n < g.N;
+        const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t m = m0 + wm * 64 + i * 16 + 4 * q + r;
+                if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[i][j][r] * div, has_bias, bias);
+            }
+    }
+}
+
 // Skinny GEMM (M <= 32), HBM-bound on W: the whole problem is one pass over the N*K bytes of weight codes.
 // One workgroup = 32 output columns, 8 waves that split K in interleaved 128-byte stages; every wave gathers its
 // MFMA operands straight from global memory in operand layout (16 bytes per lane; the four k-steps of a stage
@@ -682,6 +904,18 @@ int launch_tile(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
+template <int CDT> int launch_wide(GemmArgs g, hipStream_t st) {
+    const int64_t tm = (g.M + 255) / 256, tn = (g.N + 255) / 256;
+    if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+    g.tiles_m = (int)tm;
+    g.tiles_n = (int)tn;
+    auto kern = gemm_wide<CDT>;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, WideLds::kBytes);
+    if (e != hipSuccess) return bi8_hip_rc(e);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(512), WideLds::kBytes, st, g);
+    return bi8_launch_rc();
+}
+
 template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipStream_t st) {
     const int64_t tm = (g.M + 63) / 64, tn = (g.N + 63) / 64;
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
@@ -701,6 +935,11 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
     if (BI8_FORCE_TILE == 3) return launch_tile<128, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
     if constexpr (BLK == 128) if (BI8_FORCE_TILE == 4) return launch_tile<256, 256, 4, 2, 2, BLK, CDT, PARTIALS>(g, st);
 #endif
+#ifndef BI8_WIDE_MIN_TILES
+#define BI8_WIDE_MIN_TILES 512
+#endif
+    if constexpr (BLK == 128 && !PARTIALS)
+        if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= BI8_WIDE_MIN_TILES) return launch_wide<CDT>(g, st);
     if constexpr (kBigFits) {
         const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
         if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : 3, BLK, CDT, PARTIALS>(g, st);
