@@ -44,6 +44,15 @@ __device__ __forceinline__ void bi8_buffer_to_lds16(bi8_rsrc r, uint32_t lds_add
                  : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff)
                  : "memory", "m0");
 }
+// Same with the scalar offset given as a sum: the addition sits between the write of M0 and the load, where the
+// hardware needs one independent instruction anyway.
+__device__ __forceinline__ void bi8_buffer_to_lds16_sum(bi8_rsrc r, uint32_t lds_addr, uint32_t voff, uint32_t soff_a, uint32_t soff_b) {
+    uint32_t soff;
+    asm volatile("s_mov_b32 m0, %1\n\ts_add_u32 %0, %4, %5\n\tbuffer_load_dwordx4 %2, %3, %0 offen lds"
+                 : "=&s"(soff)
+                 : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff_a), "s"(soff_b)
+                 : "memory", "m0", "scc");
+}
 __device__ __forceinline__ void bi8_buffer_to_lds4(bi8_rsrc r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
@@ -530,6 +539,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
 // matrix pipe and the vector ALU overlap.  Two LDS stage buffers, ONE barrier per stage, placed where the last
 // operand of the stage has been read (top of the eighth column): it certifies that the next stage has landed
 // and releases this stage's buffer to the loads of the stage after next.
+// Measured on MI355X: a SIMD issues about one instruction of any kind per 4 cycles, so the kernel is bound by its
+// instruction count; two fold instructions per output per K-block are 2/3 of it.
 struct WideLds {
     static constexpr int kABuf = 256 * kStageK, kWBuf = 256 * kStageK;       // 32 KiB per operand per stage
     static constexpr int kSBuf = 256 * 4;                                    // one scale row of the tile
@@ -579,16 +590,23 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     const uint32_t s_inc = (uint32_t)((s_is_a ? g.M : g.N) * 4);
     uint32_t s_pos = 0, k_pos = 0;                 // scale-row and K position of the next stage to load
     constexpr int kLoadsPerStage = 4 + 4 + 1;
+    // A wave's nine load instructions of a stage are spread out so that the texture path never sees all 72 of the
+    // workgroup at once: the first kEarly right after the barrier that releases their buffer (eighth column of
+    // the stage two before), the other six two per column during the first columns of the stage before.
+    constexpr int kEarly = 3, kLateCols = (kLoadsPerStage - kEarly) / 2;
 
     const uint32_t lds_base = bi8_lds_address(lds);
-    auto issue_stage = [&](int buf) {
-#pragma unroll
-        for (int it = 0; it < 4; ++it) bi8_buffer_to_lds16(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024, a_off, k_pos + a_wave + it * a_step);
-#pragma unroll
-        for (int it = 0; it < 4; ++it) bi8_buffer_to_lds16(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + it * NW) * 1024, w_off, k_pos + w_wave + it * w_step);
-        bi8_buffer_to_lds4(s_rsrc, lds_base + s_dst + buf * L::kSBuf, s_off, s_pos);
-        k_pos += kStageK;
-        s_pos += s_inc;
+    // load instruction idx of a stage: 0-3 = A rows, 4-7 = W rows, 8 = scales; the K position advances after the last
+    auto issue_one = [&](int buf, int idx) {
+        if (idx < 4) {
+            bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + idx * NW) * 1024, a_off, k_pos, a_wave + idx * a_step);
+        } else if (idx < 8) {
+            bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + (idx - 4) * NW) * 1024, w_off, k_pos, w_wave + (idx - 4) * w_step);
+        } else {
+            bi8_buffer_to_lds4(s_rsrc, lds_base + s_dst + buf * L::kSBuf, s_off, s_pos);
+            k_pos += kStageK;
+            s_pos += s_inc;
+        }
     };
 
     // ---- operand fragments: lane -> row r16 of a 16-row subtile, 16-byte chunk 4*kb + q of the stage's eight;
@@ -676,6 +694,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             const int jb = j & 1;
             swb[jb] = bi8_u2f((bi8_f2u(swr[jb]) + 2u) & ~3u);      // column scale -> 22 significant bits
             swc[jb] = -BI8_MAGIC * swb[jb];                        // exact
+            // the rest of the NEXT stage's loads, two per column, into the other buffer (released one column ago)
+            if (j < kLateCols) issue_one(G, kEarly + 2 * j);
             if (j < 7) {
                 read_b(Bf[jb ^ 1], swr[jb ^ 1], j + 1, F);
             } else {
@@ -684,7 +704,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
                 wait_vm(std::integral_constant<int, 0>{});         // this wave's loads of the next stage have landed
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
-                issue_stage(F);                                    // the stage after next, into the buffer just released
+#pragma unroll
+                for (int idx = 0; idx < kEarly - 1; ++idx) issue_one(F, idx);   // the stage after next, into the buffer just released
                 read_b(Bf[0], swr[0], 0, G);                       // the next stage's column 0
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -694,7 +715,9 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
                 read_sx(sx[2], 2, F);
                 read_sx(sx[3], 3, F);
             }
+            if (j < kLateCols) issue_one(G, kEarly + 2 * j + 1);
             if (j == 7) {                                          // the next stage's row subtiles 0, 1
+                issue_one(F, kEarly - 1);
                 read_a(A[0], 0, G);
                 read_a(A[1], 1, G);
             }
@@ -704,10 +727,12 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         }
     };
 
-    // prologue: two stages of loads, wait for the first, read the first pair's operands
-    issue_stage(0);
-    issue_stage(1);
-    wait_vm(std::integral_constant<int, kLoadsPerStage>{});
+    // prologue: the first stage's loads and the early part of the second's; wait for the first stage
+#pragma unroll
+    for (int idx = 0; idx < kLoadsPerStage; ++idx) issue_one(0, idx);
+#pragma unroll
+    for (int idx = 0; idx < kEarly; ++idx) issue_one(1, idx);
+    wait_vm(std::integral_constant<int, kEarly>{});
     __syncthreads();
     read_a(A[0], 0, 0);
     read_a(A[1], 1, 0);
