@@ -960,8 +960,9 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
     if (BI8_FORCE_TILE == 3) return launch_tile<128, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
     if constexpr (BLK == 128) if (BI8_FORCE_TILE == 4) return launch_tile<256, 256, 4, 2, 2, BLK, CDT, PARTIALS>(g, st);
 #endif
+    // 256x256 tiles once they fill most of the 256 CUs (measured crossover against the 256x128 tile: ~160 tiles)
 #ifndef BI8_WIDE_MIN_TILES
-#define BI8_WIDE_MIN_TILES 512
+#define BI8_WIDE_MIN_TILES 160
 #endif
     if constexpr (BLK == 128 && !PARTIALS)
         if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= BI8_WIDE_MIN_TILES) return launch_wide<CDT>(g, st);
