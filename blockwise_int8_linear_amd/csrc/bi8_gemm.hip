@@ -4,17 +4,22 @@
 //
 //   C[m,n] = cast( (1/127^2) * sum_j sA[j,m] * sW[j,n] * P_j[m,n] ),   P_j = int32 dot over K-block j
 //
-// Main kernel (gemm_tile): NT GEMM, both operands K-contiguous.
-//   - v_mfma_i32_32x32x32_i8; one wave owns TM x TN subtiles of 32x32, int32 partial per K-block in
-//     registers, converted and folded into an fp32 accumulator as soon as the block's MFMAs are issued;
-//   - A and W tiles (128 bytes of K per row per stage) and the stage's scale rows go HBM -> LDS directly
-//     (global_load_lds, 16 bytes per lane), two stages in flight, one barrier per stage;
+// NT GEMM, both operands K-contiguous.  Four kernels, chosen by shape in dispatch():
+//   gemm_wide    block 128, problems of >= 160 tiles of 256x256: v_mfma_i32_16x16x64_i8, 64x128 per wave;
+//   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x128 / 64x128 tiles, 64x64 per wave; also
+//                the int32 block partials;
+//   gemm_skinny  M <= 32: one pass over W, K split over the waves of a workgroup;
+//   gemm_generic anything else (K not a multiple of 128, rows not 16-byte aligned, other block sizes): same
+//                MFMA, operands gathered straight from global memory with byte loads.
+// Common to the tiled kernels:
+//   - the int32 partial of a K-block stays in registers and is folded into an fp32 accumulator with two vector
+//     ops per output as soon as the block's MFMAs are issued;
+//   - A and W tiles (128 bytes of K per row per stage) and the stage's scale rows go L2 -> LDS directly
+//     (buffer_load ... lds, 16 bytes per lane), two LDS stage buffers, one barrier per stage;
 //   - LDS rows are 128 bytes with the 16-byte chunk index XOR-ed with ((row >> 1) & 7): 16 consecutive rows of
 //     one chunk column cover all 64 banks, so the MFMA operand reads (ds_read_b128) run at full LDS rate;
 //   - the workgroup index is remapped so that the 32 workgroups resident on one XCD (one L2) cover a
 //     compact patch of output tiles.
-// Shapes the main kernel cannot take (K not a multiple of 128, rows not 16-byte aligned, other block
-// sizes) go to gemm_generic: same MFMA, operands gathered straight from global memory with byte loads.
 #include <type_traits>
 
 #include "bi8_common.h"
@@ -63,19 +68,12 @@ __device__ __forceinline__ void bi8_buffer_to_lds4(bi8_rsrc r, uint32_t lds_addr
 // Workgroups are dealt round-robin to the 8 XCDs.  Give XCD x the x-th contiguous eighth of a
 // tile order in which consecutive indices form kGroupM-row bands walked column by column.
 constexpr int kXcds = 8;
-#ifndef BI8_GROUP_M
-#define BI8_GROUP_M 4
-#endif
-constexpr int kGroupM = BI8_GROUP_M;
+constexpr int kGroupM = 4;
 __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tiles_n, int &tm, int &tn) {
     const int total = tiles_m * tiles_n;
     const int per = total / kXcds;                 // full rounds
     int idx;
-#ifdef BI8_NO_XCD_REMAP
-    if (false) idx = 0;
-#else
     if (pid < per * kXcds) idx = (pid % kXcds) * per + pid / kXcds;
-#endif
     else idx = pid;                                // remainder keeps its place at the end
     const int band = kGroupM * tiles_n;
     const int b = idx / band;
@@ -780,20 +778,17 @@ __global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int l32 = lane & 31, h = lane >> 5;
     const int64_t n0 = (int64_t)blockIdx.x * 32;
+    const int64_t m0 = (int64_t)blockIdx.y * 32;      // row group of this workgroup
     const int64_t n = n0 + l32;
     const int64_t nc = n < g.N ? n : g.N - 1;                      // clamped: never stored
-    const int64_t mc = l32 < g.M ? l32 : g.M - 1;
-    const bool m_ok = l32 < g.M;
+    const int64_t mc = m0 + l32 < g.M ? m0 + l32 : g.M - 1;
+    const bool m_ok = m0 + l32 < g.M;
     const int8_t *wrow = g.W + nc * g.ldw + h * 16;
     const int8_t *arow = g.A + mc * g.lda + h * 16;
     const int nstages = (int)(g.K / kStageK);
     float acc[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
-    // row indices of this lane's 16 accumulators (clamped for the scale loads)
-    int64_t rowc[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) rowc[i] = (8 * i + 4 * h + 3 < g.M) ? (8 * i + 4 * h) : -1;
 
     auto load_stage = [&](int s, bi8_v4i *wf, bi8_v4i *af) {
         const int64_t k0 = (int64_t)s * kStageK;
@@ -821,14 +816,13 @@ __global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
             for (int i = 0; i < 4; ++i) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int row = 8 * i + 4 * h + j;
+                    const int64_t row = m0 + 8 * i + 4 * h + j;
                     const float sx = (row < g.M) ? g.sA[jb * g.M + row] : 0.0f;
                     acc[4 * i + j] = __builtin_fmaf((float)p[4 * i + j] * sx, sw, acc[4 * i + j]);
                 }
             }
         }
     }
-    (void)rowc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) red[wave][r][lane] = acc[r];
     __syncthreads();
@@ -841,7 +835,7 @@ __global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
             float v = red[0][r][lane];
 #pragma unroll
             for (int w = 1; w < NW; ++w) v += red[w][r][lane];
-            const int64_t m = 8 * (r >> 2) + 4 * h + (r & 3);
+            const int64_t m = m0 + 8 * (r >> 2) + 4 * h + (r & 3);
             if (m < g.M && n < g.N) store_c<CDT>(g.C, m * g.ldc + n, v * div, has_bias, bias);
         }
     }
@@ -951,21 +945,12 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
 }
 
 // tile shape by problem shape: the big tile when there is enough work to fill 256 CUs with it
+constexpr int64_t kWideMinTiles = 160;
 template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipStream_t st) {
     constexpr bool kBigFits = TileLds<256, 128, BLK, 3>::kFits;
-#ifdef BI8_FORCE_TILE
-    if constexpr (kBigFits) if (BI8_FORCE_TILE == 0) return launch_tile<256, 128, 4, 2, 3, BLK, CDT, PARTIALS>(g, st);
-    if (BI8_FORCE_TILE == 1) return launch_tile<128, 128, 2, 2, 2, BLK, CDT, PARTIALS>(g, st);
-    if (BI8_FORCE_TILE == 2) return launch_tile<64, 128, 1, 2, 3, BLK, CDT, PARTIALS>(g, st);
-    if (BI8_FORCE_TILE == 3) return launch_tile<128, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
-    if constexpr (BLK == 128) if (BI8_FORCE_TILE == 4) return launch_tile<256, 256, 4, 2, 2, BLK, CDT, PARTIALS>(g, st);
-#endif
     // 256x256 tiles once they fill most of the 256 CUs (measured crossover against the 256x128 tile: ~160 tiles)
-#ifndef BI8_WIDE_MIN_TILES
-#define BI8_WIDE_MIN_TILES 160
-#endif
     if constexpr (BLK == 128 && !PARTIALS)
-        if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= BI8_WIDE_MIN_TILES) return launch_wide<CDT>(g, st);
+        if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= kWideMinTiles) return launch_wide<CDT>(g, st);
     if constexpr (kBigFits) {
         const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
         if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : 3, BLK, CDT, PARTIALS>(g, st);
@@ -975,15 +960,18 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
 }
 
 template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {
-    const int64_t tn = (g.N + 31) / 32;
-    if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((gemm_skinny<BLK, CDT>), dim3((unsigned)tn), dim3(512), 0, st, g);
+    const int64_t tn = (g.N + 31) / 32, tm = (g.M + 31) / 32;
+    if (tn > 0x7fffffffLL || tm > 65535) return BI8_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((gemm_skinny<BLK, CDT>), dim3((unsigned)tn, (unsigned)tm), dim3(512), 0, st, g);
     return bi8_launch_rc();
 }
 
 template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hipStream_t st) {
+    // the tiled kernels address a tile's operand rows and the scale rows with 32-bit byte offsets
+    const int64_t max_ld = g.lda > g.ldw ? g.lda : g.ldw, max_mn = g.M > g.N ? g.M : g.N;
+    const bool offsets_ok = max_ld < (1 << 22) && (block <= 0 || (g.K / block + 1) * max_mn * 4 < 0x7fffffffLL);
     const bool tile_ok = g.K % kStageK == 0 && g.lda % 16 == 0 && g.ldw % 16 == 0 && bi8_aligned(g.A, 16) && bi8_aligned(g.W, 16) &&
-                         (PARTIALS || (bi8_aligned(g.sA, 4) && bi8_aligned(g.sW, 4)));
+                         (PARTIALS || (bi8_aligned(g.sA, 4) && bi8_aligned(g.sW, 4))) && offsets_ok;
     if constexpr (!PARTIALS) {
         if (tile_ok && g.M <= 32) {
             switch (block) {

@@ -15,8 +15,9 @@
  *   - return value 0 = success, BI8_ERR_* for rejected arguments (nothing was launched),
  *     BI8_ERR_HIP_BASE + hipError_t when the launch itself failed;
  *   - `block` is the quantization group size along the contraction dimension
- *     (block_linear_config.GROUP_SIZE, block_linear_config.py:3): a power of two, 16..1024 for the
- *     quantizers and 32..256 for the GEMM;
+ *     (block_linear_config.GROUP_SIZE, block_linear_config.py:3): any size from 1 to 2^20 is accepted;
+ *     the fast kernels take powers of two (quantizers 8..512, GEMM 32, 64 and 128 with K a multiple of
+ *     128 and 16-byte aligned rows), every other case runs slower general kernels with the same results;
  *   - scales use the reference's layout: fp32 [ceil(K/block), rows], block-major / row-minor
  *     (triton_functions.py:214-216, :227), and hold the block ABSMAX (not absmax/127).
  */
