@@ -546,7 +546,12 @@ struct WideLds {
     static constexpr int kWReg = kAReg + 2 * kABuf;
     static constexpr int kSAReg = kWReg + 2 * kWBuf;
     static constexpr int kSWReg = kSAReg + 2 * kSBuf;
-    static constexpr int kBytes = kSWReg + 2 * kSBuf;                        // 132 KiB of the CU's 160
+    // after the K loop the same memory holds each wave's 64x128 tile of 16-bit outputs, row-major; the pitch
+    // (256 + 16 bytes) puts the four row groups of one accumulator register into different banks
+    static constexpr int kOutPitch = 272;
+    static constexpr int kStages = kSWReg + 2 * kSBuf;                       // 132 KiB
+    static constexpr int kOut = 8 * 64 * kOutPitch;                          // 136 KiB
+    static constexpr int kBytes = kOut > kStages ? kOut : kStages;           // of the CU's 160 KiB
 };
 
 template <int CDT>
@@ -749,6 +754,45 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
 
     const float div = (float)(1.0 / (127.0 * 127.0));
     const bool has_bias = g.bias != nullptr;
+    if constexpr (CDT != BI8_F32) {
+        // 16-bit outputs leave through LDS: in the accumulator layout a store instruction would write 32-byte
+        // runs of four rows; from a row-major copy of the wave's 64x128 tile it writes 256-byte runs.
+        if (g.ldc % 8 == 0 && ((uintptr_t)g.C & 15) == 0) {
+            __syncthreads();                       // every wave is done with the stage buffers
+            uint8_t *tile = lds + wave * (64 * L::kOutPitch);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int64_t n = n0 + wn * 128 + j * 16 + r16;
+                const float bias = (has_bias && n < g.N) ? bi8_round_to<CDT>(load_bias(g, n)) : 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        float v = bi8_round_to<CDT>(acc[i][j][r] * div);      // acc.to(C.dtype), then + bias in C's dtype
+                        if (has_bias) v = v + bias;
+                        const uint32_t bits = (CDT == BI8_BF16) ? bi8_bf16_bits(v) : bi8_f16_bits(v);
+                        *(uint16_t *)(tile + (i * 16 + 4 * q + r) * L::kOutPitch + (j * 16 + r16) * 2) = (uint16_t)bits;
+                    }
+            }
+            // lane -> row 4p + lane/16 of the tile, 8 outputs (16 bytes) at column 8 * (lane % 16)
+            const int64_t n = n0 + wn * 128 + (lane & 15) * 8;
+#pragma unroll
+            for (int p = 0; p < 16; ++p) {
+                const int row = 4 * p + (lane >> 4);
+                const int64_t m = m0 + wm * 64 + row;
+                const bi8_v4u v = *(const bi8_v4u *)(tile + row * L::kOutPitch + (lane & 15) * 16);
+                if (m < g.M) {
+                    uint16_t *dst = (uint16_t *)g.C + m * g.ldc + n;
+                    if (n + 8 <= g.N) {
+                        *(bi8_v4u *)dst = v;
+                    } else {
+                        for (int e = 0; e < 8 && n + e < g.N; ++e) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+                    }
+                }
+            }
+            return;
+        }
+    }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int64_t n = n0 + wn * 128 + j * 16 + r16;
