@@ -885,6 +885,111 @@ __global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
     }
 }
 
+// Few-row GEMM (M <= 16, blocks 64 and 128): decode.  HBM-bound on W; everything is arranged to keep many bytes of
+// W in flight.  One workgroup = 16 output columns, 4 waves that split K in interleaved 128-byte stages; a wave
+// gathers its operands straight from global memory in the layout of v_mfma_i32_16x16x64_i8 (16 bytes per lane:
+// 16 rows x 64 contiguous bytes per load instruction) through a ring of kDepth stages of registers, i.e. up to
+// kDepth * 2 KiB of W outstanding per wave.  The row scales of the whole problem (at most 16 rows) sit in LDS,
+// zero for rows >= M; the four partial accumulators are summed through LDS in wave order (deterministic).
+// Stages past the end of K load nothing and fold with column scale 0.
+constexpr int kGemvDepth = 8;
+template <int BLK, int CDT>
+__global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
+    constexpr int NW = 4, D = kGemvDepth;
+    constexpr int NBS = kStageK / BLK;             // K-blocks per stage: one MFMA (64 bytes of K) each when BLK = 64
+    static_assert(BLK == 64 || BLK == 128, "one or two 64-byte MFMAs per K-block");
+    extern __shared__ __attribute__((aligned(16))) float gemv_lds[];
+    float(*red)[4][64] = (float(*)[4][64])gemv_lds;                 // [wave][register][lane]
+    float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][16 rows]
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, q = lane >> 4;
+    const int64_t n = (int64_t)blockIdx.x * 16 + r16;
+    const int64_t nc = n < g.N ? n : g.N - 1;                       // clamped: never stored
+    const bool m_ok = r16 < g.M;
+    const int8_t *wrow = g.W + nc * g.ldw + q * 16;
+    const int8_t *arow = g.A + (m_ok ? r16 : 0) * g.lda + q * 16;
+    const int nstages = (int)(g.K / kStageK);
+    const int nblk = nstages * NBS;
+
+    // stage t of this wave = global stage wave + NW * t; stages past the end are clamped and get column scale 0
+    bi8_v4i wf[D][2], af[D][2];
+    float swf[D][NBS];
+    auto load_stage = [&](int t, bi8_v4i *w, bi8_v4i *a, float *sw) {
+        const int s = wave + NW * t;
+        if (s < nstages) {                         // wave-uniform
+            const int64_t k0 = (int64_t)s * kStageK;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                w[kb] = __builtin_nontemporal_load((const bi8_v4i *)(wrow + k0 + kb * 64));
+                a[kb] = m_ok ? *(const bi8_v4i *)(arow + k0 + kb * 64) : bi8_v4i{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) sw[b] = g.sW[((int64_t)s * NBS + b) * g.N + nc];
+        } else {
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) sw[b] = 0.0f;
+        }
+    };
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int mine = (nstages - wave + NW - 1) / NW;                // stages of this wave (wave < NW <= nstages not required)
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        wf[d][0] = wf[d][1] = af[d][0] = af[d][1] = bi8_v4i{0, 0, 0, 0};
+        load_stage(d, wf[d], af[d], swf[d]);
+    }
+    // the row scales go to LDS while the first stages are on their way
+    for (int i = tid; i < nblk * 16; i += 256) {
+        const int jb = i >> 4, m = i & 15;
+        s_sx[i] = m < g.M ? g.sA[(int64_t)jb * g.M + m] : 0.0f;
+    }
+    __syncthreads();
+    for (int base = 0; base < mine; base += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int t = base + d;
+            const int s = wave + NW * t;
+            const int sb = (s < nstages ? s : nstages - 1) * NBS;
+            const bi8_v4i zero = {0, 0, 0, 0};
+            bi8_v4i p[NBS];
+            if constexpr (NBS == 1) {
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][0], wf[d][0], zero, 0, 0, 0);
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][1], wf[d][1], p[0], 0, 0, 0);
+            } else {
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][0], wf[d][0], zero, 0, 0, 0);
+                p[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][1], wf[d][1], zero, 0, 0, 0);
+            }
+            float swv[NBS];
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) swv[b] = swf[d][b];
+            load_stage(t + D, wf[d], af[d], swf[d]);                // refill the slot
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) {
+                const bi8_v4f sx = *(const bi8_v4f *)(s_sx + (sb + b) * 16 + 4 * q);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf((float)p[b][r] * sx[r], swv[b], acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
+    __syncthreads();
+    if (wave == 0) {
+        const float div = (float)(1.0 / (127.0 * 127.0));
+        const bool has_bias = g.bias != nullptr;
+        const float bias = (has_bias && n < g.N) ? load_bias(g, n) : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = red[0][r][lane];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) v += red[w][r][lane];
+            const int64_t m = 4 * q + r;
+            if (m < g.M && n < g.N) store_c<CDT>(g.C, m * g.ldc + n, v * div, has_bias, bias);
+        }
+    }
+}
+
 // Fallback for any K, block, alignment: 4 waves, each a 32x32 output subtile; every lane gathers its own
 // 16-byte MFMA operands with byte loads (zero outside the matrix and outside the current K-block).
 template <int CDT, bool PARTIALS>
@@ -1010,6 +1115,15 @@ template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
+constexpr int kGemvMaxBlocks = 512;                // row scales in LDS: 64 bytes per K-block, 32 KiB at most
+template <int BLK, int CDT> int launch_gemv(GemmArgs g, hipStream_t st) {
+    const int64_t tn = (g.N + 15) / 16;
+    if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+    const size_t lds = (4 * 4 * 64 + (size_t)(g.K / BLK) * 16) * sizeof(float);
+    hipLaunchKernelGGL((gemm_gemv<BLK, CDT>), dim3((unsigned)tn), dim3(256), lds, st, g);
+    return bi8_launch_rc();
+}
+
 template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hipStream_t st) {
     // the tiled kernels address a tile's operand rows and the scale rows with 32-bit byte offsets
     const int64_t max_ld = g.lda > g.ldw ? g.lda : g.ldw, max_mn = g.M > g.N ? g.M : g.N;
@@ -1017,6 +1131,12 @@ template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hip
     const bool tile_ok = g.K % kStageK == 0 && g.lda % 16 == 0 && g.ldw % 16 == 0 && bi8_aligned(g.A, 16) && bi8_aligned(g.W, 16) &&
                          (PARTIALS || (bi8_aligned(g.sA, 4) && bi8_aligned(g.sW, 4))) && offsets_ok;
     if constexpr (!PARTIALS) {
+#ifndef BI8_NO_GEMV
+        if (tile_ok && g.M <= 16 && g.K / block <= kGemvMaxBlocks) {
+            if (block == 64) return launch_gemv<64, CDT>(g, st);
+            if (block == 128) return launch_gemv<128, CDT>(g, st);
+        }
+#endif
         if (tile_ok && g.M <= 32) {
             switch (block) {
             case 32: return launch_skinny<32, CDT>(g, st);
