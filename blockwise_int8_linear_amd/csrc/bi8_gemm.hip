@@ -8,7 +8,9 @@
 //   gemm_wide    block 128, problems of >= 160 tiles of 256x256: v_mfma_i32_16x16x64_i8, 64x128 per wave;
 //   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x128 / 64x128 tiles, 64x64 per wave; also
 //                the int32 block partials;
-//   gemm_skinny  M <= 32: one pass over W, K split over the waves of a workgroup;
+//   gemm_gemv    M <= 16, blocks 64/128 (decode): one pass over W, 16 columns per workgroup, K split over 4 waves,
+//                operands gathered from global memory through an 8-stage register ring;
+//   gemm_skinny  M <= 32 otherwise: the same idea with 32x32x32 MFMAs and one stage of lookahead;
 //   gemm_generic anything else (K not a multiple of 128, rows not 16-byte aligned, other block sizes): same
 //                MFMA, operands gathered straight from global memory with byte loads.
 // Common to the tiled kernels:
