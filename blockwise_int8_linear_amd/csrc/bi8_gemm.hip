@@ -541,9 +541,10 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
 // and releases this stage's buffer to the loads of the stage after next.
 // Measured on MI355X: a SIMD issues about one instruction of any kind per 4 cycles, so the kernel is bound by its
 // instruction count; two fold instructions per output per K-block are 2/3 of it.
-struct WideLds {
+template <int NBS> struct WideLds {                 // NBS = K-blocks per stage
     static constexpr int kABuf = 256 * kStageK, kWBuf = 256 * kStageK;       // 32 KiB per operand per stage
-    static constexpr int kSBuf = 256 * 4;                                    // one scale row of the tile
+    static constexpr int kSRow = 256 * 4;                                    // one scale row of the tile
+    static constexpr int kSBuf = NBS * kSRow;                                // the stage's scale rows, one per K-block
     static constexpr int kAReg = 0;
     static constexpr int kWReg = kAReg + 2 * kABuf;
     static constexpr int kSAReg = kWReg + 2 * kWBuf;
@@ -556,9 +557,11 @@ struct WideLds {
     static constexpr int kBytes = kOut > kStages ? kOut : kStages;           // of the CU's 160 KiB
 };
 
-template <int CDT>
+template <int BLK, int CDT>
 __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
-    using L = WideLds;
+    static_assert(BLK == 128 || BLK == 64, "a K-block is one or two 64-byte MFMAs");
+    constexpr int NBS = kStageK / BLK;
+    using L = WideLds<NBS>;
     constexpr int BM = 256, BN = 256, NW = 8;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -583,8 +586,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     const uint32_t a_off = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_off = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
     const uint32_t a_wave = (uint32_t)(wave * 8 * g.lda), w_wave = (uint32_t)(wave * 8 * g.ldw);
     const uint32_t a_step = (uint32_t)(NW * 8 * g.lda), w_step = (uint32_t)(NW * 8 * g.ldw);
-    // scale rows of the stage's K-block: waves 0-3 fetch 64 row scales each, waves 4-7 64 column scales each
-    const int64_t nblk = g.K / 128;
+    // scale rows of the stage's K-blocks: waves 0-3 fetch 64 row scales each, waves 4-7 64 column scales each
+    const int64_t nblk = g.K / BLK;
     const bool s_is_a = wave < 4;
     const int s_part = wave & 3;
     const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
@@ -594,23 +597,23 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     const uint32_t s_dst = (uint32_t)((s_is_a ? L::kSAReg : L::kSWReg) + s_part * 256);
     const uint32_t s_inc = (uint32_t)((s_is_a ? g.M : g.N) * 4);
     uint32_t s_pos = 0, k_pos = 0;                 // scale-row and K position of the next stage to load
-    constexpr int kLoadsPerStage = 4 + 4 + 1;
-    // A wave's nine load instructions of a stage are spread out so that the texture path never sees all 72 of the
-    // workgroup at once: the first kEarly right after the barrier that releases their buffer (eighth column of
-    // the stage two before), the other six two per column during the first columns of the stage before.
-    constexpr int kEarly = 3, kLateCols = (kLoadsPerStage - kEarly) / 2;
+    constexpr int kLoadsPerStage = 4 + 4 + NBS;
+    // A wave's nine or ten load instructions of a stage are spread out so that the texture path never sees all of
+    // the workgroup's at once: the first kEarly right after the barrier that releases their buffer (last column
+    // step of the stage two before), the others two per step during the first steps of the stage before.
+    constexpr int kEarly = 3, kLateCols = (kLoadsPerStage - kEarly + 1) / 2;
 
     const uint32_t lds_base = bi8_lds_address(lds);
-    // load instruction idx of a stage: 0-3 = A rows, 4-7 = W rows, 8 = scales; the K position advances after the last
+    // load instruction idx of a stage: 0-3 = A rows, 4-7 = W rows, 8.. = scale rows; the K position advances after the last
     auto issue_one = [&](int buf, int idx) {
         if (idx < 4) {
             bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + idx * NW) * 1024, a_off, k_pos, a_wave + idx * a_step);
         } else if (idx < 8) {
             bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + (idx - 4) * NW) * 1024, w_off, k_pos, w_wave + (idx - 4) * w_step);
-        } else {
-            bi8_buffer_to_lds4(s_rsrc, lds_base + s_dst + buf * L::kSBuf, s_off, s_pos);
-            k_pos += kStageK;
+        } else if (idx < kLoadsPerStage) {
+            bi8_buffer_to_lds4(s_rsrc, lds_base + s_dst + buf * L::kSBuf + (idx - 8) * L::kSRow, s_off, s_pos);
             s_pos += s_inc;
+            if (idx == kLoadsPerStage - 1) k_pos += kStageK;
         }
     };
 
@@ -687,7 +690,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     // On entry to a stage (buffer F): A[0], A[1], Bf[0], swr[0] already hold this stage's row subtiles 0, 1 and
     // column 0 (read during the previous stage's last column); c[1] is the previous stage's last pair (rows 2, 3
     // of column 7), still to be folded with the OLD sx[2], sx[3], swb[1], swc[1].
-    auto stage = [&](auto buf_c) {
+    auto stage = [&](auto buf_c) {                  // BLK = 128
         constexpr int F = decltype(buf_c)::value, G = 1 - F;
         read_a(A[2], 2, F);
         read_a(A[3], 3, F);
@@ -732,6 +735,74 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         }
     };
 
+    // ---- BLK = 64: a stage is two K-blocks, each ONE MFMA per subtile.  The stage runs as 16 column steps (K-block
+    // kb = step / 8, column = step % 8); a pair is two MFMAs, each followed by the whole fold of one subtile of the
+    // previous pair (twice the vector work per MFMA of the block-128 schedule).  W fragments (one 16-byte chunk
+    // column) and column scales are read one step ahead, the row scales of K-block 1 at step 8.
+    bi8_v4i Bh[2];                                 // [step parity]
+    auto read_bh = [&](bi8_v4i &dst, float &raw, int step, int buf) {
+        const int kb = step >> 3, j = step & 7;
+        dst = *(const bi8_v4i *)(lds + w_base[kb] + buf * L::kWBuf + j * 16 * kStageK);
+        raw = *(const float *)(lds + sw_base + buf * L::kSBuf + kb * L::kSRow + j * 16 * 4);
+    };
+    auto read_sx64 = [&](bi8_v4f &dst, int i, int kb, int buf) {
+        dst = *(const bi8_v4f *)(lds + sa_base + buf * L::kSBuf + kb * L::kSRow + i * 16 * 4);
+    };
+    auto pair64 = [&](bi8_v4i *cn, const bi8_v4i &a0, const bi8_v4i &a1, const bi8_v4i &b, const bi8_v4i *cp, const bi8_v4f &s0,
+                      const bi8_v4f &s1, float fb, float fc, float *d0, float *d1) {
+        cn[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, magic, 0, 0, 0);
+        fold2(cp[0], 0, s0, fb, fc, d0);
+        fold2(cp[0], 2, s0, fb, fc, d0);
+        __builtin_amdgcn_sched_barrier(0);
+        cn[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b, magic, 0, 0, 0);
+        fold2(cp[1], 0, s1, fb, fc, d1);
+        fold2(cp[1], 2, s1, fb, fc, d1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto stage64 = [&](auto buf_c) {
+        constexpr int F = decltype(buf_c)::value, G = 1 - F;
+        read_a(A[2], 2, F);
+        read_a(A[3], 3, F);
+        read_sx64(sx[0], 0, 0, F);
+        read_sx64(sx[1], 1, 0, F);
+#pragma unroll
+        for (int h = 0; h < 16; ++h) {
+            const int kb = h >> 3, j = h & 7, hb = h & 1, jprev = (h + 15) & 7;
+            swb[hb] = bi8_u2f((bi8_f2u(swr[hb]) + 2u) & ~3u);      // column scale -> 22 significant bits
+            swc[hb] = -BI8_MAGIC * swb[hb];                        // exact
+            if (h < kLateCols) issue_one(G, kEarly + 2 * h);
+            if (h == 8) {                                          // K-block 1: row subtiles 0, 1 (2, 3 after the pending fold)
+                read_sx64(sx[0], 0, 1, F);
+                read_sx64(sx[1], 1, 1, F);
+            }
+            if (h < 15) {
+                read_bh(Bh[hb ^ 1], swr[hb ^ 1], h + 1, F);
+            } else {
+                __builtin_amdgcn_s_waitcnt(0xC07F);                // lgkmcnt(0) only
+                wait_vm(std::integral_constant<int, 0>{});
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int idx = 0; idx < kEarly - 1; ++idx) issue_one(F, idx);
+                read_bh(Bh[0], swr[0], 0, G);                      // the next stage's first step
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            pair64(c[0], A[0][kb], A[1][kb], Bh[hb], c[1], sx[2], sx[3], swb[hb ^ 1], swc[hb ^ 1], acc[2][jprev], acc[3][jprev]);
+            if (h == 0 || h == 8) {
+                read_sx64(sx[2], 2, kb, F);
+                read_sx64(sx[3], 3, kb, F);
+            }
+            if (h < kLateCols) issue_one(G, kEarly + 2 * h + 1);
+            if (h == 15) {
+                issue_one(F, kEarly - 1);
+                read_a(A[0], 0, G);
+                read_a(A[1], 1, G);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            pair64(c[1], A[2][kb], A[3][kb], Bh[hb], c[0], sx[0], sx[1], swb[hb], swc[hb], acc[0][j], acc[1][j]);
+        }
+    };
+
     // prologue: the first stage's loads and the early part of the second's; wait for the first stage
 #pragma unroll
     for (int idx = 0; idx < kLoadsPerStage; ++idx) issue_one(0, idx);
@@ -741,12 +812,18 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     __syncthreads();
     read_a(A[0], 0, 0);
     read_a(A[1], 1, 0);
-    read_b(Bf[0], swr[0], 0, 0);
+    if constexpr (BLK == 128) read_b(Bf[0], swr[0], 0, 0);
+    else read_bh(Bh[0], swr[0], 0, 0);
     // The trip count is rounded up to even and loads run two stages ahead: stages past the end of K read their
     // scales through the buffers' range check as zeros, so they add exactly 0 to the accumulators.
     for (int s = 0; s < nstages; s += 2) {
-        stage(std::integral_constant<int, 0>{});
-        stage(std::integral_constant<int, 1>{});
+        if constexpr (BLK == 128) {
+            stage(std::integral_constant<int, 0>{});
+            stage(std::integral_constant<int, 1>{});
+        } else {
+            stage64(std::integral_constant<int, 0>{});
+            stage64(std::integral_constant<int, 1>{});
+        }
     }
     wait_vm(std::integral_constant<int, 0>{});     // nothing may still be writing LDS when the wave ends
     fold2(c[1][0], 0, sx[2], swb[1], swc[1], acc[2][7]);
@@ -1074,15 +1151,16 @@ int launch_tile(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-template <int CDT> int launch_wide(GemmArgs g, hipStream_t st) {
+template <int BLK, int CDT> int launch_wide(GemmArgs g, hipStream_t st) {
+    using L = WideLds<kStageK / BLK>;
     const int64_t tm = (g.M + 255) / 256, tn = (g.N + 255) / 256;
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     g.tiles_m = (int)tm;
     g.tiles_n = (int)tn;
-    auto kern = gemm_wide<CDT>;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, WideLds::kBytes);
+    auto kern = gemm_wide<BLK, CDT>;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, L::kBytes);
     if (e != hipSuccess) return bi8_hip_rc(e);
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(512), WideLds::kBytes, st, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(512), L::kBytes, st, g);
     return bi8_launch_rc();
 }
 
@@ -1100,14 +1178,16 @@ constexpr int64_t kWideMinTiles = 160;
 template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipStream_t st) {
     constexpr bool kBigFits = TileLds<256, 128, BLK, 3>::kFits;
     // 256x256 tiles once they fill most of the 256 CUs (measured crossover against the 256x128 tile: ~160 tiles)
-    if constexpr (BLK == 128 && !PARTIALS)
-        if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= kWideMinTiles) return launch_wide<CDT>(g, st);
+    if constexpr ((BLK == 128 || BLK == 64) && !PARTIALS)
+        if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= kWideMinTiles) return launch_wide<BLK, CDT>(g, st);
     if constexpr (kBigFits) {
         const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
         if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : 3, BLK, CDT, PARTIALS>(g, st);
     }
-    if (g.M > 64) return launch_tile<128, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
-    return launch_tile<64, 128, 1, 2, 3, BLK, CDT, PARTIALS>(g, st);
+    // small grids: one workgroup per CU at best, so the tile is spread over as many waves as its shape allows
+    // (measured 25-37 % faster than 2x2 waves of 64x64 at M = 96 ... 1024)
+    if (g.M > 64) return launch_tile<128, 128, 4, 2, 3, BLK, CDT, PARTIALS>(g, st);
+    return launch_tile<64, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
 }
 
 template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {

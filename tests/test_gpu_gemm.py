@@ -77,7 +77,7 @@ def test_gemm_golden(ops):
 # tiles of 256x256) the 256x256-tile kernel of block 128 with an even, an odd and a longer run of K stages
 # and with a single stage
 SHAPES = [(253, 257, 234), (129, 266, 75), (389, 138, 45), (256, 512, 512), (1, 384, 256), (16, 1000, 1024),
-          (64, 128, 128), (100, 300, 384), (300, 500, 512), (1024, 512, 512), (3584, 3584, 256), (3500, 3700, 384),
+          (64, 128, 128), (48, 700, 640), (100, 300, 384), (300, 500, 512), (1024, 512, 512), (3584, 3584, 256), (3500, 3700, 384),
           (2304, 4500, 1152), (2560, 4096, 128)]
 
 
