@@ -1,7 +1,8 @@
 // Block quantize of the transpose (bi8_quantize_transposed): x [R,C] -> codes [C,R], scales [ceil(R/B), C],
 // blocks running down the columns of x.  The backward pass of the reference materializes x.t().contiguous()
 // and then calls the row quantizer (block_linear.py:93-94, :100-103): two extra full passes over HBM.
-// Here one workgroup reads a 128-row x 64-column tile once with 128-bit row loads, keeps it in LDS as
+// Here a workgroup reads a 128-row x 64-column tile once with 128-bit row loads (the next tile's loads already in
+// flight while this one is processed), keeps it in LDS as
 // fp32, reduces and quantizes down the columns, transposes the codes through LDS and writes them as
 // 128-byte runs of the output rows.  Results are identical to the two-step form.
 #include "bi8_common.h"
@@ -41,7 +42,7 @@ template <int DT> __device__ __forceinline__ void unpack(const bi8_v4u &raw, flo
 template <int DT, int B>
 __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__restrict__ x, int8_t *__restrict__ qT,
                                                                float *__restrict__ scalesT, int64_t R, int64_t C,
-                                                               int64_t ldx, int64_t ldq, int tiles_c) {
+                                                               int64_t ldx, int64_t ldq, int64_t tiles_c, int64_t ntiles) {
     constexpr int VEC = Vec<DT>::kElems;
     constexpr int64_t ES = 16 / VEC;
     constexpr int LPR = kTC / VEC;                 // lanes per tile row
@@ -53,82 +54,100 @@ __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__res
     __shared__ __attribute__((aligned(16))) uint8_t s_q[kTC * kQPitch];
 
     const int tid = threadIdx.x;
-    const int64_t tile_r = blockIdx.x / tiles_c;
-    const int tile_c = blockIdx.x % tiles_c;
-    const int64_t r0 = tile_r * kTR;
-    const int64_t c0 = (int64_t)tile_c * kTC;
     const char *xb = (const char *)x;
+    constexpr int NP = kTR / RPP;                  // 16-byte loads per thread per tile
 
-    // phase 1: rows of the tile -> fp32 in LDS
+    // A workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...; the loads of the next tile are issued before
+    // the current one is processed, so every workgroup has global loads in flight all the time.
+    auto load_tile = [&](int64_t tile, bi8_v4u *raw) {
+        const int64_t r0 = (tile / tiles_c) * kTR;
+        const int64_t c0 = (tile % tiles_c) * kTC;
 #pragma unroll
-    for (int p = 0; p < kTR / RPP; ++p) {
-        const int r = p * RPP + tid / LPR;
-        const int cc = (tid % LPR) * VEC;
-        bi8_v4u raw = {0u, 0u, 0u, 0u};
-        if (r0 + r < R && c0 + cc < C) raw = __builtin_nontemporal_load((const bi8_v4u *)(xb + ((r0 + r) * ldx + c0 + cc) * ES));
-        float f[VEC];
-        unpack<DT>(raw, f);
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) s_x[r * kPitch + cc + e] = f[e];
-    }
-    __syncthreads();
+        for (int p = 0; p < NP; ++p) {
+            const int r = p * RPP + tid / LPR;
+            const int cc = (tid % LPR) * VEC;
+            raw[p] = bi8_v4u{0u, 0u, 0u, 0u};
+            if (tile < ntiles && r0 + r < R && c0 + cc < C)
+                raw[p] = __builtin_nontemporal_load((const bi8_v4u *)(xb + ((r0 + r) * ldx + c0 + cc) * ES));
+        }
+    };
+    bi8_v4u raw[NP];
+    load_tile(blockIdx.x, raw);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t r0 = (tile / tiles_c) * kTR;
+        const int64_t c0 = (tile % tiles_c) * kTC;
 
-    // phase 2: column maxima over this thread's 32 rows, then over the block's row groups
-    const int c = tid & 63;
-    const int g = tid >> 6;
-    float v[32];
-    float m = 0.0f;
-    bool special = false;
+        // phase 1: rows of the tile -> fp32 in LDS; then start the next tile's loads
 #pragma unroll
-    for (int i = 0; i < 32; ++i) {
-        v[i] = s_x[(g * 32 + i) * kPitch + c];
-        m = __builtin_fmaxf(m, __builtin_fabsf(v[i]));
-        special |= (v[i] != v[i]);
-    }
-    if constexpr (GPB > 1) {
-        s_max[g][c] = m;
+        for (int p = 0; p < NP; ++p) {
+            const int r = p * RPP + tid / LPR;
+            const int cc = (tid % LPR) * VEC;
+            float f[VEC];
+            unpack<DT>(raw[p], f);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) s_x[r * kPitch + cc + e] = f[e];
+        }
+        load_tile(tile + gridDim.x, raw);
         __syncthreads();
-        const int gb = g & ~(GPB - 1);
-#pragma unroll
-        for (int k = 0; k < GPB; ++k) m = __builtin_fmaxf(m, s_max[gb + k][c]);
-    }
-    if ((g & (GPB - 1)) == 0) {
-        const int64_t jb = (r0 + g * 32) / B;
-        if (r0 + g * 32 < R && c0 + c < C) scalesT[jb * C + c0 + c] = m;
-    }
 
-    // phase 3: codes of this thread's 32 rows -> byte tile [column][row]
-    special |= !bi8_scale_is_ordinary(m);
-    uint32_t code[32];
-    if (__builtin_expect(special, 0)) {
+        // phase 2: column maxima over this thread's 32 rows, then over the block's row groups
+        const int c = tid & 63;
+        const int g = tid >> 6;
+        float v[32];
+        float m = 0.0f;
+        bool special = false;
 #pragma unroll
-        for (int i = 0; i < 32; ++i) code[i] = bi8_code_slow(v[i], m);
-    } else {
-        const float y = 1.0f / m;
+        for (int i = 0; i < 32; ++i) {
+            v[i] = s_x[(g * 32 + i) * kPitch + c];
+            m = __builtin_fmaxf(m, __builtin_fabsf(v[i]));
+            special |= (v[i] != v[i]);
+        }
+        if constexpr (GPB > 1) {
+            s_max[g][c] = m;
+            __syncthreads();
+            const int gb = g & ~(GPB - 1);
 #pragma unroll
-        for (int i = 0; i < 32; ++i) code[i] = bi8_code_fast<NCORR>(v[i], m, y);
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-        *(uint32_t *)&s_q[c * kQPitch + g * 32 + 4 * i] = bi8_pack4(code[4 * i], code[4 * i + 1], code[4 * i + 2], code[4 * i + 3]);
-    __syncthreads();
+            for (int k = 0; k < GPB; ++k) m = __builtin_fmaxf(m, s_max[gb + k][c]);
+        }
+        if ((g & (GPB - 1)) == 0) {
+            const int64_t jb = (r0 + g * 32) / B;
+            if (r0 + g * 32 < R && c0 + c < C) scalesT[jb * C + c0 + c] = m;
+        }
 
-    // phase 4: 16 codes per lane, 8 lanes per output row
+        // phase 3: codes of this thread's 32 rows -> byte tile [column][row]
+        special |= !bi8_scale_is_ordinary(m);
+        uint32_t code[32];
+        if (__builtin_expect(special, 0)) {
 #pragma unroll
-    for (int p = 0; p < (kTC * kTR / 16) / kThreads; ++p) {
-        const int idx = p * kThreads + tid;
-        const int oc = idx / (kTR / 16);           // output row inside the tile = source column
-        const int seg = idx % (kTR / 16);
-        const int64_t orow = c0 + oc;
-        const int64_t ocol = r0 + seg * 16;
-        if (orow < C && ocol < R) {
-            const uint32_t *src = (const uint32_t *)&s_q[oc * kQPitch + seg * 16];
-            bi8_v4u w = {src[0], src[1], src[2], src[3]};
-            int8_t *dst = qT + orow * ldq + ocol;
-            if (ocol + 16 <= R) {
-                __builtin_nontemporal_store(w, (bi8_v4u *)dst);
-            } else {
-                for (int e = 0; e < (int)(R - ocol); ++e) dst[e] = (int8_t)((w[e >> 2] >> (8 * (e & 3))) & 0xffu);
+            for (int i = 0; i < 32; ++i) code[i] = bi8_code_slow(v[i], m);
+        } else {
+            const float y = 1.0f / m;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) code[i] = bi8_code_fast<NCORR>(v[i], m, y);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            *(uint32_t *)&s_q[c * kQPitch + g * 32 + 4 * i] = bi8_pack4(code[4 * i], code[4 * i + 1], code[4 * i + 2], code[4 * i + 3]);
+        __syncthreads();
+
+        // phase 4: 16 codes per lane, 8 lanes per output row.  The next iteration's writes to s_x come after this
+        // barrier (all column reads are done), its writes to s_q after its own first barrier (all reads below are done).
+#pragma unroll
+        for (int p = 0; p < (kTC * kTR / 16) / kThreads; ++p) {
+            const int idx = p * kThreads + tid;
+            const int oc = idx / (kTR / 16);       // output row inside the tile = source column
+            const int seg = idx % (kTR / 16);
+            const int64_t orow = c0 + oc;
+            const int64_t ocol = r0 + seg * 16;
+            if (orow < C && ocol < R) {
+                const uint32_t *src = (const uint32_t *)&s_q[oc * kQPitch + seg * 16];
+                bi8_v4u w = {src[0], src[1], src[2], src[3]};
+                int8_t *dst = qT + orow * ldq + ocol;
+                if (ocol + 16 <= R) {
+                    __builtin_nontemporal_store(w, (bi8_v4u *)dst);
+                } else {
+                    for (int e = 0; e < (int)(R - ocol); ++e) dst[e] = (int8_t)((w[e >> 2] >> (8 * (e & 3))) & 0xffu);
+                }
             }
         }
     }
@@ -157,9 +176,12 @@ template <int DT, int B>
 int launch_tile(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq, hipStream_t st) {
     const int64_t tiles_c = (C + kTC - 1) / kTC;
     const int64_t tiles_r = (R + kTR - 1) / kTR;
-    if (tiles_c * tiles_r > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((quantize_cols_tile<DT, B>), dim3((unsigned)(tiles_c * tiles_r)), dim3(kThreads), 0, st, x, qT, scalesT, R, C,
-                       ldx, ldq, (int)tiles_c);
+    const int64_t ntiles = tiles_c * tiles_r;
+    // three workgroups fit a CU (42 KiB of LDS each); more tiles than that are walked by resident workgroups
+    const int64_t resident = 3 * 256;
+    const int64_t grid = ntiles < resident ? ntiles : resident;
+    hipLaunchKernelGGL((quantize_cols_tile<DT, B>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, qT, scalesT, R, C, ldx, ldq,
+                       tiles_c, ntiles);
     return bi8_launch_rc();
 }
 
