@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0          # HBM3E, 8 TB/s
 # Bytes that cross the L2 <-> fabric boundary in one 8192^3 block-128 launch of the headline kernel: FETCH_SIZE and
 # WRITE_SIZE of rocprofv3 --pmc runs of this file, scaled by what the same counters read for a 256 MiB copy
 # (x2.0 and x1.0); the runs and figures are in profiles/gemm_wide_8192x8192x8192_block128.md.  Not measured live.
-GEMM_8192_TRAFFIC_BYTES = 1008031044
+GEMM_8192_TRAFFIC_BYTES = 980842510
 
 
 def event_ms(fn, iters: int) -> float:
@@ -190,7 +190,7 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": round(achieved / INT8_PEAK_TOPS, 4),
                      "traffic": GEMM_8192_TRAFFIC_BYTES if (S == 8192 and B == 128) else None,
-                     "kernel": "gemm_wide<bf16> (256x256 tile, 8 waves of 64x128, 2 LDS stage buffers, v_mfma_i32_16x16x64_i8)", "ops_per_launch": ops_per_launch,
+                     "kernel": "gemm_wide<128,bf16> (256x256 tile, 8 waves of 64x128, 2 LDS stage buffers, v_mfma_i32_16x16x64_i8)", "ops_per_launch": ops_per_launch,
                      "avg_launch_ms": round(kern_ms, 4)},
     }
     if not args.no_quantize:
