@@ -145,3 +145,39 @@ def test_recip_division_is_exact():
     res = subprocess.run([exe, "50000000"], capture_output=True, text=True)
     assert res.returncode == 0, res.stdout
     assert res.stdout.count(" 0 mismatches") == 3, res.stdout
+
+
+def test_reference_module_names_can_be_aliased():
+    """code written against the reference's flat layout: `import block_linear_config`, `from triton_functions import ...`,
+    `from block_linear import BlockInt8Linear` (block_linear.py:8-12) resolve to this package after compat.install()"""
+    import importlib
+    import sys
+
+    import blockwise_int8_linear_amd as pkg
+    from blockwise_int8_linear_amd import compat
+    for name in ("block_linear_config", "triton_functions", "block_linear"):
+        assert name not in sys.modules
+    compat.install()
+    try:
+        cfg = importlib.import_module("block_linear_config")
+        tf = importlib.import_module("triton_functions")
+        bl = importlib.import_module("block_linear")
+        assert cfg is pkg.block_linear_config
+        assert tf.quantize_block_rowwise is pkg.quantize_block_rowwise
+        assert tf.int8_matmul_block64_rowwise_dequantize is pkg.int8_matmul_block64_rowwise_dequantize
+        assert tf.dequantize_block_rowwise is pkg.dequantize_block_rowwise and tf.ceil_div(7, 2) == 4
+        assert bl.BlockInt8Linear is pkg.BlockInt8Linear and bl.replace_linear_with_blockwise_int8 is pkg.replace_linear_with_blockwise_int8
+        old = cfg.GROUP_SIZE
+        cfg.GROUP_SIZE = 64                      # one config object under both names
+        assert pkg.block_linear_config.GROUP_SIZE == 64
+        cfg.GROUP_SIZE = old
+        compat.install()                         # idempotent
+    finally:
+        compat.uninstall()
+    assert "triton_functions" not in sys.modules
+    sys.modules["triton_functions"] = sys                      # somebody else's module of that name is not shadowed silently
+    try:
+        with pytest.raises(RuntimeError, match="already imported"):
+            compat.install()
+    finally:
+        del sys.modules["triton_functions"]
