@@ -34,7 +34,7 @@ constexpr int kStageK = 128;       // bytes of K per LDS stage
 typedef bi8_v4i bi8_rsrc;
 __device__ __forceinline__ bi8_rsrc bi8_make_rsrc(const void *base, int64_t bytes) {
     const uint64_t a = (uint64_t)base;
-    const int n = bytes > 0x7fffffffLL ? 0x7fffffff : (int)bytes;
+    const int n = bytes > 0x7fffffffLL ? 0x7fffffff : (bytes < 0 ? 0 : (int)bytes);    // never a wrapped (huge) range
     // dword0-1: 48-bit base, stride 0; dword2: size in bytes; dword3: raw 32-bit-format buffer (gfx9 family)
     return bi8_rsrc{(int)(uint32_t)a, (int)(uint32_t)((a >> 32) & 0xffffu), n, 0x00020000};
 }
@@ -1210,7 +1210,7 @@ template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hip
     // the tiled kernels address a tile's operand rows and the scale rows with 32-bit byte offsets
     const int64_t max_ld = g.lda > g.ldw ? g.lda : g.ldw, max_mn = g.M > g.N ? g.M : g.N;
     const bool offsets_ok = max_ld < (1 << 22) && (block <= 0 || (g.K / block + 1) * max_mn * 4 < 0x7fffffffLL);
-    const bool tile_ok = g.K % kStageK == 0 && g.lda % 16 == 0 && g.ldw % 16 == 0 && bi8_aligned(g.A, 16) && bi8_aligned(g.W, 16) &&
+    const bool tile_ok = g.K > 0 && g.K % kStageK == 0 && g.lda % 16 == 0 && g.ldw % 16 == 0 && bi8_aligned(g.A, 16) && bi8_aligned(g.W, 16) &&
                          (PARTIALS || (bi8_aligned(g.sA, 4) && bi8_aligned(g.sW, 4))) && offsets_ok;
     if constexpr (!PARTIALS) {
 #ifndef BI8_NO_GEMV

@@ -206,6 +206,27 @@ def test_few_rows_operand_views(ops):
         _assert_close(base.cpu(), ref, mag, TOL["f32"])
 
 
+def test_empty_dimensions(ops):
+    """M = 0 and N = 0 give empty outputs; K = 0 gives zeros (plus bias), for few and for many rows"""
+    with cfg_as(ops, 128, torch.float32):
+        for M, N in ((0, 256), (300, 0), (0, 0)):
+            a = torch.empty(M, 256, device=DEV, dtype=torch.int8)
+            w = torch.empty(N, 256, device=DEV, dtype=torch.int8)
+            c = ops.int8_matmul_block64_rowwise_dequantize(a, w.t(), torch.empty(2, M, device=DEV), torch.empty(2, N, device=DEV))
+            assert c.shape == (M, N)
+            assert ops.int8_matmul_block_partials(a, w.t()).shape == (2, M, N)
+        for M, N in ((3, 40), (200, 300), (4096, 4096)):
+            a = torch.empty(M, 0, device=DEV, dtype=torch.int8)
+            w = torch.empty(N, 0, device=DEV, dtype=torch.int8)
+            sa, sw = torch.empty(0, M, device=DEV), torch.empty(0, N, device=DEV)
+            bias = torch.randn(N, device=DEV)
+            c = ops.int8_matmul_block64_rowwise_dequantize(a, w.t(), sa, sw)
+            assert c.shape == (M, N) and (c == 0).all()
+            cb = ops.int8_matmul_block64_rowwise_dequantize(a, w.t(), sa, sw, bias)
+            assert torch.equal(cb, bias.expand(M, N))
+            assert ops.int8_matmul_block_partials(a, w.t()).shape == (0, M, N)
+
+
 def test_end_to_end_vs_dense_config1(ops):
     """X fp32 [256,1024] ~N(0,1); W fp32 [1024,1024] ~N(0,0.02); block 64; fp32 out, compared to the fp32
     matmul and to the checker's forward."""
