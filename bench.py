@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0          # HBM3E, 8 TB/s
 # Bytes that cross the L2 <-> fabric boundary in one 8192^3 block-128 launch of the headline kernel: FETCH_SIZE and
 # WRITE_SIZE of rocprofv3 --pmc runs of this file, scaled by what the same counters read for a 256 MiB copy
 # (x2.0 and x1.0); the runs and figures are in profiles/gemm_wide_8192x8192x8192_block128.md.  Not measured live.
-GEMM_8192_TRAFFIC_BYTES = 980842510
+GEMM_8192_TRAFFIC_BYTES = 980817527
 
 
 def event_ms(fn, iters: int) -> float:
