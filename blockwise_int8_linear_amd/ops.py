@@ -133,6 +133,31 @@ def _gemm_operands(a: torch.Tensor, b: torch.Tensor):
     return a, w
 
 
+_FAST_BLOCKS = (32, 64, 128)
+_PAD_MIN_WORK = 1 << 22            # M*N*K below which the general kernel is as quick as two padded copies
+
+
+def _pad_contraction(a, w, state_x, state_w, block):
+    """The tiled GEMM kernels want K to be a multiple of 128 and 16-byte aligned operand rows; a contraction like
+    the GPT-2 vocabulary (50257, the grad-input GEMM of the output layer) would fall to the general kernel, which is
+    ~40x slower.  Zero codes add nothing to any block partial, so such operands are copied once into buffers
+    padded with zero codes up to the next multiple of 128 (and the scales with zero rows if that adds K-blocks):
+    the results are the same numbers."""
+    M, K = a.shape
+    N = w.shape[0]
+    ragged = K % 128 != 0 or _ld(a) % 16 != 0 or _ld(w) % 16 != 0 or a.data_ptr() % 16 != 0 or w.data_ptr() % 16 != 0
+    if not ragged or block not in _FAST_BLOCKS or K == 0 or M * N * K < _PAD_MIN_WORK:
+        return a, w, state_x, state_w, K
+    k_pad = ceil_div(K, 128) * 128
+    a = torch.nn.functional.pad(a, (0, k_pad - K))
+    w = torch.nn.functional.pad(w, (0, k_pad - K))
+    extra = k_pad // block - state_x.shape[0]
+    if extra > 0:
+        state_x = torch.nn.functional.pad(state_x, (0, 0, 0, extra))
+        state_w = torch.nn.functional.pad(state_w, (0, 0, 0, extra))
+    return a, w, state_x, state_w, k_pad
+
+
 def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
     """a int8 [M,K], b int8 [K,N] (any strides), state_x [K/B, M], state_w [K/B, N], bias [N] or None
     -> [M,N] of INPUT_OUTPUT_TORCH_TYPE; triton_functions.py:142-168.  B = GROUP_SIZE at call time."""
@@ -144,6 +169,7 @@ def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
     nblk = ceil_div(K, block)
     assert tuple(state_x.shape) == (nblk, M) and tuple(state_w.shape) == (nblk, N), "scale shapes must be [ceil(K/block), rows]"
     state_x, state_w = _scales_in(state_x), _scales_in(state_w)
+    a, w, state_x, state_w, K = _pad_contraction(a, w, state_x, state_w, block)
     c = torch.empty((M, N), device=a.device, dtype=out_dtype)
     bias_ptr, bias_dt = None, 0
     if bias is not None:

@@ -206,6 +206,46 @@ def test_few_rows_operand_views(ops):
         _assert_close(base.cpu(), ref, mag, TOL["f32"])
 
 
+@pytest.mark.parametrize("block", [32, 64, 128])
+def test_vocabulary_sized_contraction(ops, block):
+    """K not a multiple of 128 with an odd leading dimension (the GPT-2 vocabulary 50257 as contraction, scaled
+    down): the operator pads the codes with zeros and runs the tiled kernels; same numbers as the checker, and the
+    same as the general kernel on a problem small enough to stay there"""
+    g = torch.Generator().manual_seed(block)
+    M, N, K = 300, 200, 5027
+    A, W = _codes(g, M, K), _codes(g, N, K)
+    nblk = -(-K // block)
+    sa = torch.rand(nblk, M, generator=g) + 0.1
+    sw = torch.rand(nblk, N, generator=g) * 0.05 + 1e-3
+    bias = torch.randn(N, generator=g)
+    _, ref, mag = _reference(A, W, sa, sw, block, None, torch.float32)
+    with cfg_as(ops, block, torch.float32):
+        Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
+        C = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sad, swd)
+        Cb = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sad, swd, bias.to(DEV))
+        small = ops.int8_matmul_block64_rowwise_dequantize(Ad[:8], Wd[:16].t(), sad[:, :8].contiguous(), swd[:, :16].contiguous())
+    _assert_close(C.cpu(), ref, mag, TOL["f32"])
+    assert torch.equal(Cb, C + bias.to(DEV))
+    _assert_close(small.cpu(), ref[:8, :16], mag[:8, :16], TOL["f32"])
+    assert ((small - C[:8, :16]).abs().cpu().double() <= 8e-6 * mag[:8, :16] + 2e-3 * ref[:8, :16].abs().double()).all()
+
+
+@pytest.mark.parametrize("block", [16, 48, 256])
+def test_other_block_sizes_run_the_general_kernel(ops, block):
+    g = torch.Generator().manual_seed(block)
+    M, N, K = 70, 90, 480
+    A, W = _codes(g, M, K), _codes(g, N, K)
+    nblk = -(-K // block)
+    sa = torch.rand(nblk, M, generator=g) + 0.1
+    sw = torch.rand(nblk, N, generator=g) * 0.05 + 1e-3
+    P_ref, ref, mag = _reference(A, W, sa, sw, block, None, torch.float32)
+    with cfg_as(ops, block, torch.float32):
+        C = ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa.to(DEV), sw.to(DEV))
+        P = ops.int8_matmul_block_partials(A.to(DEV), W.to(DEV).t())
+    _assert_close(C.cpu(), ref, mag, TOL["f32"])
+    assert torch.equal(P.cpu(), P_ref)
+
+
 def test_empty_dimensions(ops):
     """M = 0 and N = 0 give empty outputs; K = 0 gives zeros (plus bias), for few and for many rows"""
     with cfg_as(ops, 128, torch.float32):
