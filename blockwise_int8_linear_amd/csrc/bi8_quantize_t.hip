@@ -39,7 +39,10 @@ template <int DT> __device__ __forceinline__ void unpack(const bi8_v4u &raw, flo
 }
 
 // B in {32, 64, 128}: thread (c = tid % 64, g = tid / 64) owns source rows 32g .. 32g+31 of column c.
-template <int DT, int B>
+// VLOAD / VSTORE: the source rows / the output rows are 16-byte aligned, so a lane moves 16 bytes at a time; without
+// them the same tile is read element by element (64 consecutive elements per wave instruction) and written byte by
+// byte (64 consecutive bytes per wave instruction): odd leading dimensions such as the GPT-2 vocabulary, 50257.
+template <int DT, int B, bool VLOAD, bool VSTORE>
 __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__restrict__ x, int8_t *__restrict__ qT,
                                                                float *__restrict__ scalesT, int64_t R, int64_t C,
                                                                int64_t ldx, int64_t ldq, int64_t tiles_c, int64_t ntiles) {
@@ -55,20 +58,34 @@ __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__res
 
     const int tid = threadIdx.x;
     const char *xb = (const char *)x;
-    constexpr int NP = kTR / RPP;                  // 16-byte loads per thread per tile
+    constexpr int NP = VLOAD ? kTR / RPP : (kTR * kTC) / kThreads / 4;   // 16-byte loads (or groups of 4 elements) per thread per tile
 
     // A workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...; the loads of the next tile are issued before
     // the current one is processed, so every workgroup has global loads in flight all the time.
     auto load_tile = [&](int64_t tile, bi8_v4u *raw) {
         const int64_t r0 = (tile / tiles_c) * kTR;
         const int64_t c0 = (tile % tiles_c) * kTC;
+        if constexpr (VLOAD) {
 #pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            const int r = p * RPP + tid / LPR;
-            const int cc = (tid % LPR) * VEC;
-            raw[p] = bi8_v4u{0u, 0u, 0u, 0u};
-            if (tile < ntiles && r0 + r < R && c0 + cc < C)
-                raw[p] = __builtin_nontemporal_load((const bi8_v4u *)(xb + ((r0 + r) * ldx + c0 + cc) * ES));
+            for (int p = 0; p < NP; ++p) {
+                const int r = p * RPP + tid / LPR;
+                const int cc = (tid % LPR) * VEC;
+                raw[p] = bi8_v4u{0u, 0u, 0u, 0u};
+                if (tile < ntiles && r0 + r < R && c0 + cc < C)
+                    raw[p] = __builtin_nontemporal_load((const bi8_v4u *)(xb + ((r0 + r) * ldx + c0 + cc) * ES));
+            }
+        } else {
+            // element e = tid + 256 * k of the tile in row-major order, as fp32 bits: raw[p][i] is k = 4p + i
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e = tid + kThreads * (4 * p + i);
+                    const int r = e / kTC, cc = e % kTC;
+                    float f = 0.0f;
+                    if (tile < ntiles && r0 + r < R && c0 + cc < C) f = bi8_load_elem<DT>(x, (r0 + r) * ldx + c0 + cc);
+                    raw[p][i] = bi8_f2u(f);
+                }
         }
     };
     bi8_v4u raw[NP];
@@ -78,14 +95,24 @@ __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__res
         const int64_t c0 = (tile % tiles_c) * kTC;
 
         // phase 1: rows of the tile -> fp32 in LDS; then start the next tile's loads
+        if constexpr (VLOAD) {
 #pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            const int r = p * RPP + tid / LPR;
-            const int cc = (tid % LPR) * VEC;
-            float f[VEC];
-            unpack<DT>(raw[p], f);
+            for (int p = 0; p < NP; ++p) {
+                const int r = p * RPP + tid / LPR;
+                const int cc = (tid % LPR) * VEC;
+                float f[VEC];
+                unpack<DT>(raw[p], f);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) s_x[r * kPitch + cc + e] = f[e];
+                for (int e = 0; e < VEC; ++e) s_x[r * kPitch + cc + e] = f[e];
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < NP; ++p)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e = tid + kThreads * (4 * p + i);
+                    s_x[(e / kTC) * kPitch + e % kTC] = bi8_u2f(raw[p][i]);
+                }
         }
         load_tile(tile + gridDim.x, raw);
         __syncthreads();
@@ -132,6 +159,16 @@ __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__res
 
         // phase 4: 16 codes per lane, 8 lanes per output row.  The next iteration's writes to s_x come after this
         // barrier (all column reads are done), its writes to s_q after its own first barrier (all reads below are done).
+        if constexpr (!VSTORE) {
+            // byte e = tid + 256 * k of the code tile [64 output rows][128]: 64 consecutive bytes per wave instruction
+#pragma unroll 4
+            for (int k = 0; k < (kTC * kTR) / kThreads; ++k) {
+                const int e = tid + kThreads * k;
+                const int oc = e / kTR, ob = e % kTR;
+                const int64_t orow = c0 + oc, ocol = r0 + ob;
+                if (orow < C && ocol < R) qT[orow * ldq + ocol] = (int8_t)s_q[oc * kQPitch + ob];
+            }
+        } else
 #pragma unroll
         for (int p = 0; p < (kTC * kTR / 16) / kThreads; ++p) {
             const int idx = p * kThreads + tid;
@@ -172,7 +209,7 @@ __global__ __launch_bounds__(kThreads) void quantize_cols_generic(const void *__
     }
 }
 
-template <int DT, int B>
+template <int DT, int B, bool VLOAD, bool VSTORE>
 int launch_tile(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq, hipStream_t st) {
     const int64_t tiles_c = (C + kTC - 1) / kTC;
     const int64_t tiles_r = (R + kTR - 1) / kTR;
@@ -180,21 +217,28 @@ int launch_tile(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C,
     // three workgroups fit a CU (42 KiB of LDS each); more tiles than that are walked by resident workgroups
     const int64_t resident = 3 * 256;
     const int64_t grid = ntiles < resident ? ntiles : resident;
-    hipLaunchKernelGGL((quantize_cols_tile<DT, B>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, qT, scalesT, R, C, ldx, ldq,
-                       tiles_c, ntiles);
+    hipLaunchKernelGGL((quantize_cols_tile<DT, B, VLOAD, VSTORE>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, qT, scalesT, R, C,
+                       ldx, ldq, tiles_c, ntiles);
     return bi8_launch_rc();
+}
+
+template <int DT, int B>
+int launch_tile_any(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq, hipStream_t st) {
+    constexpr int VEC = Vec<DT>::kElems;
+    const bool vload = C % VEC == 0 && ldx % VEC == 0 && bi8_aligned(x, 16);
+    const bool vstore = ldq % 16 == 0 && bi8_aligned(qT, 16);
+    if (vload && vstore) return launch_tile<DT, B, true, true>(x, qT, scalesT, R, C, ldx, ldq, st);
+    if (vload) return launch_tile<DT, B, true, false>(x, qT, scalesT, R, C, ldx, ldq, st);
+    if (vstore) return launch_tile<DT, B, false, true>(x, qT, scalesT, R, C, ldx, ldq, st);
+    return launch_tile<DT, B, false, false>(x, qT, scalesT, R, C, ldx, ldq, st);
 }
 
 template <int DT>
 int dispatch(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq, int block, hipStream_t st) {
-    constexpr int VEC = Vec<DT>::kElems;
-    const bool tile_ok = C % VEC == 0 && ldx % VEC == 0 && ldq % 16 == 0 && bi8_aligned(x, 16) && bi8_aligned(qT, 16);
-    if (tile_ok) {
-        switch (block) {
-        case 32: return launch_tile<DT, 32>(x, qT, scalesT, R, C, ldx, ldq, st);
-        case 64: return launch_tile<DT, 64>(x, qT, scalesT, R, C, ldx, ldq, st);
-        case 128: return launch_tile<DT, 128>(x, qT, scalesT, R, C, ldx, ldq, st);
-        }
+    switch (block) {
+    case 32: return launch_tile_any<DT, 32>(x, qT, scalesT, R, C, ldx, ldq, st);
+    case 64: return launch_tile_any<DT, 64>(x, qT, scalesT, R, C, ldx, ldq, st);
+    case 128: return launch_tile_any<DT, 128>(x, qT, scalesT, R, C, ldx, ldq, st);
     }
     const int64_t nblk = (R + block - 1) / block;
     int64_t grid = (C * nblk + kThreads - 1) / kThreads;

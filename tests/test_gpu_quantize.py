@@ -143,7 +143,10 @@ def test_dequantize_parity(ops, out):
 @pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("block", [32, 64, 128])
 def test_quantize_transposed_equals_two_step(ops, dtype, block):
-    for (R, C) in [(256, 512), (8192, 768), (300, 1000), (1000, 72), (129, 64), (64, 50257 // 8 * 8)]:
+    # the last four: odd row lengths of the source and/or of the output (unaligned loads / byte stores in the tile
+    # kernel), among them the GPT-2 vocabulary as either dimension
+    for (R, C) in [(256, 512), (8192, 768), (300, 1000), (1000, 72), (129, 64), (64, 50257 // 8 * 8),
+                   (300, 517), (517, 304), (333, 77), (64, 50257), (50257, 64)]:
         x_cpu = outlier_tensor(R, C, DTYPES[dtype], seed=R + C)
         q, s = _check_quant(ops, x_cpu, block, transposed=True)
         x = x_cpu.to(DEV)
