@@ -110,13 +110,20 @@ template <int DT>
 __global__ __launch_bounds__(kThreads) void dequantize_rows_generic(const int8_t *__restrict__ q, const float *__restrict__ scales,
                                                                     void *__restrict__ out, int64_t M, int64_t K, int64_t ldq,
                                                                     int64_t ldo, int block) {
+    // one workgroup per (row, run of 2048 columns): consecutive lanes take consecutive elements, no 64-bit division
     const float inv127 = (float)(1.0 / 127.0);
-    const int64_t total = M * K;
-    const int64_t stride = (int64_t)gridDim.x * kThreads;
-    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
-        const int64_t row = i / K, k = i % K;
-        const float s = scales[(k / block) * M + row];
-        bi8_store_elem<DT>(out, row * ldo + k, (s * (float)q[row * ldq + k]) * inv127);
+    const int64_t runs = (K + 2047) / 2048;
+    const int64_t units = M * runs;
+    for (int64_t u = blockIdx.x; u < units; u += gridDim.x) {
+        const int64_t row = u / runs, k0 = (u % runs) * 2048;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int64_t k = k0 + t * kThreads + threadIdx.x;
+            if (k < K) {
+                const float s = scales[(k / block) * M + row];
+                bi8_store_elem<DT>(out, row * ldo + k, (s * (float)q[row * ldq + k]) * inv127);
+            }
+        }
     }
 }
 
@@ -136,8 +143,8 @@ int dispatch(const int8_t *q, const float *scales, void *out, int64_t M, int64_t
                            K, ldq, ldo, nblk, __builtin_ctz((unsigned)block), (int)tiles_k);
         return bi8_launch_rc();
     }
-    int64_t grid = (M * K + kThreads - 1) / kThreads;
-    if (grid > 65536) grid = 65536;
+    int64_t grid = M * ((K + 2047) / 2048);
+    if (grid > (1 << 20)) grid = 1 << 20;
     hipLaunchKernelGGL((dequantize_rows_generic<DT>), dim3((unsigned)grid), dim3(kThreads), 0, st, q, scales, out, M, K, ldq, ldo,
                        block);
     return bi8_launch_rc();

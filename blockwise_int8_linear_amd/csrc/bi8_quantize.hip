@@ -146,6 +146,57 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_generic(const void *__
     }
 }
 
+// Rows that are not 16-byte aligned (odd row length or leading dimension, e.g. 50257), blocks 32 / 64 / 128: one
+// wave per 512 consecutive elements of a row, lane l holds elements 64k + l (k = 0..7), so every load instruction
+// reads 64 consecutive elements and every store 64 consecutive code bytes; a K-block is 32 or 64 adjacent lanes
+// of one k, or (B = 128) the whole wave over two k.
+template <int DT, int B>
+__global__ __launch_bounds__(kThreads) void quantize_rows_loose(const void *__restrict__ x, int8_t *__restrict__ q,
+                                                                float *__restrict__ scales, int64_t M, int64_t K, int64_t ldx,
+                                                                int64_t ldq, int64_t chunks_per_row) {
+    constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
+    constexpr int U = 8;
+    const int lane = threadIdx.x & 63;
+    const int64_t unit = (int64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
+    const int64_t row = unit / chunks_per_row;
+    if (row >= M) return;
+    const int64_t k0 = (unit % chunks_per_row) * (64 * U);
+    float v[U], m[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        const int64_t idx = k0 + 64 * k + lane;
+        v[k] = idx < K ? bi8_load_elem<DT>(x, row * ldx + idx) : 0.0f;
+        m[k] = __builtin_fmaxf(0.0f, __builtin_fabsf(v[k]));        // ignores NaN
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        if constexpr (B == 128) {
+            if ((k & 1) == 0) m[k] = m[k + 1] = bi8_group_max<64>(__builtin_fmaxf(m[k], m[k + 1]));
+        } else {
+            m[k] = bi8_group_max<B>(m[k]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+        const int64_t idx = k0 + 64 * k + lane;
+        if (idx < K) {
+            const bool special = (v[k] != v[k]) || !bi8_scale_is_ordinary(m[k]);
+            const uint32_t code = special ? bi8_code_slow(v[k], m[k]) : bi8_code_fast<NCORR>(v[k], m[k], 1.0f / m[k]);
+            q[row * ldq + idx] = (int8_t)(code & 0xffu);
+            if (idx % B == 0) scales[(idx / B) * M + row] = m[k];
+        }
+    }
+}
+
+template <int DT, int B>
+int launch_loose(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int64_t ldx, int64_t ldq, hipStream_t st) {
+    const int64_t chunks = (K + 511) / 512;
+    const int64_t grid = (M * chunks + 3) / 4;
+    if (grid > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((quantize_rows_loose<DT, B>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, M, K, ldx, ldq, chunks);
+    return bi8_launch_rc();
+}
+
 template <int DT, int L>
 int launch_vec(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int64_t ldx, int64_t ldq, hipStream_t st) {
     constexpr int VEC = Vec<DT>::kElems;
@@ -175,6 +226,11 @@ int dispatch(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int6
         case 32: return launch_vec<DT, 32>(x, q, scales, M, K, ldx, ldq, st);
         case 64: return launch_vec<DT, 64>(x, q, scales, M, K, ldx, ldq, st);
         }
+    }
+    switch (block) {
+    case 32: return launch_loose<DT, 32>(x, q, scales, M, K, ldx, ldq, st);
+    case 64: return launch_loose<DT, 64>(x, q, scales, M, K, ldx, ldq, st);
+    case 128: return launch_loose<DT, 128>(x, q, scales, M, K, ldx, ldq, st);
     }
     const int64_t nblk = (K + block - 1) / block;
     const int64_t units = M * nblk;

@@ -56,7 +56,7 @@ def test_quantize_golden(ops):
 @pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("block", [16, 32, 64, 128, 256])
 def test_quantize_parity_seeded(ops, dtype, block):
-    for (M, K) in [(256, 1024), (37, 4096), (1, 11008), (130, 2048 + 8 * 5), (5, 1000), (19, 333)]:
+    for (M, K) in [(256, 1024), (37, 4096), (1, 11008), (130, 2048 + 8 * 5), (5, 1000), (19, 333), (9, 5027)]:
         x = outlier_tensor(M, K, DTYPES[dtype], seed=M + K + block)
         _check_quant(ops, x, block)
 
@@ -129,7 +129,7 @@ def test_dequantize_parity(ops, out):
             for got, e in zip(d.tolist(), exp):
                 assert (e is None and got in (float("inf"), float("-inf"))) or got == e
         g = torch.Generator().manual_seed(3)
-        for (M, K, B) in [(64, 2048, 128), (33, 1040, 16), (7, 999, 64), (16, 4096, 1024), (3, 70, 24)]:
+        for (M, K, B) in [(64, 2048, 128), (33, 1040, 16), (7, 999, 64), (16, 4096, 1024), (3, 70, 24), (5, 5027, 128)]:
             q = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
             s = torch.rand(-(-K // B), M, generator=g) * 3
             d = ops.dequantize_block_rowwise(q.to(DEV), s.to(DEV), B)
