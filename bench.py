@@ -5,8 +5,8 @@
 Workload (the configuration the headline metric is quoted on): int8 block GEMM with fused dequantize at
 M = N = K = 8192, block 128, bf16 out, operands = block-quantized bf16 N(0,1) activations and 0.02*N(0,1)
 weights (seed 0), already resident in HBM; next to it the block quantize -> dequantize round trip of a bf16
-[8192,8192] tensor with 0.1% x50 outliers at blocks 32/64/128.  A "step" is one GEMM launch through the
-drop-in operator.  Prints ONE JSON line.
+[8192,8192] tensor with 0.1% x50 outliers at blocks 32/64/128, and ("extras") the block-64 GEMM, the decode GEMM
+and the transposed quantizer.  A "step" is one GEMM launch through the drop-in operator.  Prints ONE JSON line.
 
 Kernel durations are measured with HIP events recorded on the stream the kernels are launched on (torch's
 current stream), around runs of back-to-back launches.
@@ -96,6 +96,70 @@ def bench_quantize(pkg, torch, iters: int):
             "roundtrip_mse": mse,
         }
         del qs, ss, ds
+    return out
+
+
+def bench_extras(pkg, torch):
+    """secondary figures of the same path, all through the C ABI with preallocated outputs: the block-64 GEMM at
+    8192^3, the few-row (decode) GEMM at Llama-7B shapes with the weights rotated through ~600 MB so that they come
+    from HBM, and the transposed quantizer of the backward pass"""
+    from blockwise_int8_linear_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    out = {}
+    S, B = 8192, 64
+    a = torch.randint(-127, 128, (S, S), device="cuda", dtype=torch.int8)
+    w = torch.randint(-127, 128, (S, S), device="cuda", dtype=torch.int8)
+    sa = torch.rand(S // B, S, device="cuda") + 0.5
+    sw = torch.rand(S // B, S, device="cuda") * 0.02
+    c = torch.empty(S, S, device="cuda", dtype=torch.bfloat16)
+
+    def g64():
+        assert lib.bi8_gemm_nt_dequant(a.data_ptr(), w.data_ptr(), sa.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
+                                       S, S, S, S, S, S, B, st) == 0
+    g64()
+    t = min(event_ms(g64, 10) for _ in range(2))
+    out["gemm_block64_8192"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1)}
+    del a, w, sa, sw, c
+
+    B = 128
+    for (K, N) in ((4096, 11008), (11008, 4096)):
+        nset = max(2, int(600e6 // (N * K)))
+        ws = [torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8) for _ in range(nset)]
+        sw = torch.rand(K // B, N, device="cuda") * 0.02
+        for M in (1, 16):
+            x = torch.randint(-127, 128, (M, K), device="cuda", dtype=torch.int8)
+            sx = torch.rand(K // B, M, device="cuda") + 0.5
+            c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+            turn = [0]
+
+            def gv():
+                i = turn[0] = (turn[0] + 1) % nset
+                assert lib.bi8_gemm_nt_dequant(x.data_ptr(), ws[i].data_ptr(), sx.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
+                                               M, N, K, K, K, N, B, st) == 0
+            for _ in range(5):
+                gv()
+            t = min(event_ms(gv, 50) for _ in range(2))
+            nbytes = N * K + 4 * (K // B) * (N + M) + M * K + 2 * M * N
+            out[f"decode_gemm_M{M}_K{K}_N{N}"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
+                                                  "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
+        del ws
+
+    M = K = 8192
+    xs = [torch.randn(M, K, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3)]
+    qs = [torch.empty(K, M, device="cuda", dtype=torch.int8) for _ in range(3)]
+    ss = [torch.empty(M // 128, K, device="cuda", dtype=torch.float32) for _ in range(3)]
+    turn = [0]
+
+    def qt():
+        i = turn[0] = (turn[0] + 1) % 3
+        assert lib.bi8_quantize_transposed(xs[i].data_ptr(), 1, qs[i].data_ptr(), ss[i].data_ptr(), M, K, K, M, 128, st) == 0
+    for _ in range(6):
+        qt()
+    t = min(event_ms(qt, 30) for _ in range(2))
+    nbytes = M * K * 3 + 4 * M * K // 128
+    out["quantize_transposed_bf16_8192"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
+                                            "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
     return out
 
 
@@ -195,6 +259,7 @@ def main():
     }
     if not args.no_quantize:
         res["quantize_roundtrip"] = bench_quantize(pkg, torch, 50)
+        res["extras"] = bench_extras(pkg, torch)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(torch, xq.cpu(), wq.cpu(), sx.cpu(), sw.cpu(), B)
     print(json.dumps(res))
