@@ -20,7 +20,13 @@ def ceil_div(n: int, d: int) -> int:
     return -(n // -d)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """hipStream_t of torch's current stream on t's device (the raw getter is ~2 us cheaper than the Stream object)"""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
@@ -52,6 +58,8 @@ def _float_operand(x: torch.Tensor) -> torch.Tensor:
 
 def _rows(x: torch.Tensor) -> torch.Tensor:
     """2-D tensor whose rows are contiguous (leading dimension = stride(0))."""
+    if x.is_contiguous():
+        return x
     if x.numel() and (x.stride(1) != 1 or (x.shape[0] > 1 and x.stride(0) < x.shape[1])):
         return x.contiguous()
     return x
