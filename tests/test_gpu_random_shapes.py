@@ -99,3 +99,39 @@ def test_quantize_dequantize_random(ops, seed):
     do = oracle.dequantize_block_rowwise(qo, so, block, DTYPES[dtype])
     view = torch.int32 if dtype == "f32" else torch.int16
     assert torch.equal(d.cpu().view(view), do.view(view)), (M, K, pad, block, dtype)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_gemm_random_large(ops, seed):
+    """shapes of at least 160 output tiles of 256x256 (the large-problem kernel for blocks 64 and 128), ragged edges"""
+    rng = random.Random(3000 + seed)
+    block = rng.choice([64, 128])
+    out = rng.choice(["f32", "bf16", "f16"])
+    M, N = rng.randint(3300, 4400), rng.randint(3300, 4400)
+    K = 128 * rng.randint(1, 5)
+    g = torch.Generator().manual_seed(seed)
+    A = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+    W = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    nblk = K // block
+    sa = torch.rand(nblk, M, generator=g) * 3 + 0.01
+    sw = torch.rand(nblk, N, generator=g) * 0.1 + 1e-4
+    bias = torch.randn(N, generator=g)
+    P = oracle_torch.gemm_nt_partials(A, W, block)
+    ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw, block, None, DTYPES[out])
+    mag = torch.zeros(M, N, dtype=torch.float64)
+    for j in range(nblk):
+        mag += P[j].abs().double() * sa[j].double()[:, None] * sw[j].double()[None, :]
+    mag /= 127.0 * 127.0
+    cfg = ops.block_linear_config
+    old = (cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE)
+    cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = block, DTYPES[out]
+    try:
+        Ad, Wd = A.to(DEV), W.to(DEV)
+        C = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sa.to(DEV), sw.to(DEV))
+        Cb = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sa.to(DEV), sw.to(DEV), bias.to(DEV))
+    finally:
+        cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = old
+    assert torch.equal(Cb, C + bias.to(DEV).to(DTYPES[out]))
+    err = (C.cpu().double() - ref.double()).abs()
+    bound = TOL[out] * ref.double().abs() + 4e-6 * mag + 1e-30
+    assert (err <= bound).all(), f"M={M} N={N} K={K} block={block} out={out}: max excess {(err - bound).max().item():.3e}"
