@@ -49,7 +49,7 @@ __device__ __forceinline__ void bi8_buffer_to_lds16(bi8_rsrc r, uint32_t lds_add
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff)
-                 : "memory", "m0");
+                 : "memory", "m0", "vcc");      // vcc listed so that no operand is allocated to it (not encodable as soffset)
 }
 // Same with the scalar offset given as a sum: the addition sits between the write of M0 and the load, where the
 // hardware needs one independent instruction anyway.
@@ -58,13 +58,13 @@ __device__ __forceinline__ void bi8_buffer_to_lds16_sum(bi8_rsrc r, uint32_t lds
     asm volatile("s_mov_b32 m0, %1\n\ts_add_u32 %0, %4, %5\n\tbuffer_load_dwordx4 %2, %3, %0 offen lds"
                  : "=&s"(soff)
                  : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff_a), "s"(soff_b)
-                 : "memory", "m0", "scc");
+                 : "memory", "m0", "scc", "vcc");
 }
 __device__ __forceinline__ void bi8_buffer_to_lds4(bi8_rsrc r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff)
-                 : "memory", "m0");
+                 : "memory", "m0", "vcc");      // vcc listed so that no operand is allocated to it (not encodable as soffset)
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs.  Give XCD x the x-th contiguous eighth of a
