@@ -196,6 +196,22 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
 
     constexpr int kLoadsPerStage = kAIter + kWIter + kSIter;     // VMEM instructions one wave issues per stage
     const uint32_t lds_base = bi8_lds_address(lds);
+    // the same in two halves (A rows; W rows + scales + advance), so that a stage's loads need not all be issued at once
+    auto issue_half = [&](int buf, int half) {
+        if (half == 0) {
+#pragma unroll
+            for (int it = 0; it < kAIter; ++it) bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024, a_off, k_pos, a_wave + it * a_step);
+        } else {
+#pragma unroll
+            for (int it = 0; it < kWIter; ++it) bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + it * NW) * 1024, w_off, k_pos, w_wave + it * w_step);
+            k_pos += kStageK;
+#pragma unroll
+            for (int it = 0; it < kSIter; ++it) {
+                bi8_buffer_to_lds4(s_rsrc[it], lds_base + s_dst[it] + buf * s_bufstep[it], s_off[it], s_pos[it]);
+                s_pos[it] += s_inc[it];
+            }
+        }
+    };
     auto issue_stage = [&](int buf) {             // buf is wave-uniform: LDS destinations and K position are scalars
 #pragma unroll
         for (int it = 0; it < kAIter; ++it) bi8_buffer_to_lds16(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + it * NW) * 1024, a_off, k_pos + a_wave + it * a_step);
@@ -445,11 +461,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
             wait_vm(Drained{});                    // this wave's loads of stage s+1 have landed
             __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
-            issue_stage(F);                        // stage s+2 into the buffer just released
+            issue_half(F, 0);                      // stage s+2 into the buffer just released: A rows now, the rest one subtile later
             // subtile (1,G), meanwhile the next stage's row subtile 0
             read_a(A0, 0, G);
             __builtin_amdgcn_sched_barrier(0);
             item(p[0], A1, Bq[G], p[1], sx0, sw2[G], swc2[G], acc[0][G], false);
+            issue_half(F, 1);
             // subtile (1,F), meanwhile the next stage's column subtile G (its first)
             read_w(Bq[G], G, G);
             __builtin_amdgcn_sched_barrier(0);
