@@ -102,7 +102,8 @@ def bench_quantize(pkg, torch, iters: int):
 def bench_extras(pkg, torch):
     """secondary figures of the same path, all through the C ABI with preallocated outputs: the block-64 GEMM at
     8192^3, the few-row (decode) GEMM at Llama-7B shapes with the weights rotated through ~600 MB so that they come
-    from HBM, and the transposed quantizer of the backward pass"""
+    from HBM (and the one-token eval-path linear, quantize included, as two launches and as one kernel), and the
+    transposed quantizer of the backward pass"""
     from blockwise_int8_linear_amd import _lib
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
@@ -143,6 +144,26 @@ def bench_extras(pkg, torch):
             nbytes = N * K + 4 * (K // B) * (N + M) + M * K + 2 * M * N
             out[f"decode_gemm_M{M}_K{K}_N{N}"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
                                                   "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
+            if M == 1:
+                # the whole eval-path linear for one token: row quantizer + GEMM as two launches, and as the one kernel
+                xf = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+                xq = torch.empty(M, K, device="cuda", dtype=torch.int8)
+
+                def two():
+                    i = turn[0] = (turn[0] + 1) % nset
+                    assert lib.bi8_quantize_rowwise(xf.data_ptr(), 1, xq.data_ptr(), sx.data_ptr(), M, K, K, K, B, st) == 0
+                    assert lib.bi8_gemm_nt_dequant(xq.data_ptr(), ws[i].data_ptr(), sx.data_ptr(), sw.data_ptr(), None, 0,
+                                                   c.data_ptr(), 1, M, N, K, K, K, N, B, st) == 0
+
+                def one():
+                    i = turn[0] = (turn[0] + 1) % nset
+                    assert lib.bi8_linear_few_rows(xf.data_ptr(), 1, ws[i].data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(),
+                                                   M, N, K, K, K, N, B, st) == 0
+                for _ in range(5):
+                    two(), one()
+                t2 = min(event_ms(two, 50) for _ in range(2))
+                t1 = min(event_ms(one, 50) for _ in range(2))
+                out[f"decode_linear_M1_K{K}_N{N}"] = {"one_kernel_us": round(t1 * 1e3, 2), "two_launches_us": round(t2 * 1e3, 2)}
         del ws
 
     M = K = 8192

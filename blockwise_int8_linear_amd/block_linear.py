@@ -7,7 +7,9 @@ Differences from the reference that do not change results:
     ``.t().contiguous()`` followed by the row quantizer (block_linear.py:93-94, :100-103);
   * ``ctx.save_for_backward`` is called, not assigned over (block_linear.py:73);
   * switching the module back to training mode drops the cached int8 weights, so a later ``eval()``
-    re-quantizes the current weights (the reference keeps serving the first cache, block_linear.py:138-139).
+    re-quantizes the current weights (the reference keeps serving the first cache, block_linear.py:138-139);
+  * the eval path with at most 4 rows (token-by-token decode) quantizes and multiplies in one kernel
+    (block_linear.py:141-144 are two launches).
 """
 from __future__ import annotations
 
@@ -17,6 +19,7 @@ import torch.nn as nn
 from .ops import (
     dequantize_block_rowwise,
     int8_matmul_block64_rowwise_dequantize,
+    linear_few_rows,
     quantize_block_rowwise,
     quantize_block_transposed,
 )
@@ -96,10 +99,18 @@ class BlockInt8Linear(nn.Linear):
         if getattr(self, "W_int8", None) is None:
             self.prepare_for_eval()
         X = x.reshape(-1, x.size(-1))
-        X_int8, state_X = quantize_block_rowwise(X)
-        return int8_matmul_block64_rowwise_dequantize(
-            X_int8, self.W_int8.t(), state_X, self.state_W, self.bias
-        ).view(*x.size()[:-1], -1)
+        out = None
+        if X.shape[0] <= 2:
+            # token-by-token decode: quantize and multiply in one kernel.  Every workgroup of that kernel quantizes
+            # x for itself, which pays off (measured) for one row at block 128, for two up to a medium output
+            # width, and at block 64 up to 4096 outputs
+            wide_block = self.state_W.shape[0] * 128 == X.shape[1]
+            if (wide_block and (X.shape[0] == 1 or self.out_features <= 16384)) or self.out_features <= 4096:
+                out = linear_few_rows(X, self.W_int8, self.state_W, self.bias)
+        if out is None:
+            X_int8, state_X = quantize_block_rowwise(X)
+            out = int8_matmul_block64_rowwise_dequantize(X_int8, self.W_int8.t(), state_X, self.state_W, self.bias)
+        return out.view(*x.size()[:-1], -1)
 
     def forward(self, x):
         if not self.training:

@@ -58,6 +58,31 @@ template <int DT> __device__ __forceinline__ void bi8_store_elem(void *p, int64_
     else ((uint16_t *)p)[i] = (uint16_t)bi8_f16_bits(v);
 }
 
+// ---- 16-byte loads of floating-point elements -----------------------------------------------------
+template <int DT> struct Bi8Vec {
+    static constexpr int kElems = (DT == BI8_F32) ? 4 : 8;     // elements per 16-byte load
+};
+
+// 16 raw bytes -> kElems floats
+template <int DT> __device__ __forceinline__ void bi8_unpack(const bi8_v4u &raw, float *f) {
+    if constexpr (DT == BI8_F32) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) f[e] = bi8_u2f(raw[e]);
+    } else if constexpr (DT == BI8_BF16) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f[2 * e] = bi8_u2f(raw[e] << 16);
+            f[2 * e + 1] = bi8_u2f(raw[e] & 0xffff0000u);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            f[2 * e] = bi8_from_f16_bits(raw[e] & 0xffffu);
+            f[2 * e + 1] = bi8_from_f16_bits(raw[e] >> 16);
+        }
+    }
+}
+
 // ---- cross-lane maximum over aligned groups of L lanes (L a power of two, 1..64) ---------------
 // DPP moves for the steps inside a row of 16 lanes, ds_bpermute beyond.  max is idempotent, so the
 // mirror patterns (lane i <-> 7-i, i <-> 15-i) finish the 8- and 16-lane reductions.

@@ -1086,6 +1086,175 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
     }
 }
 
+// Quantize + few-row GEMM in one launch (M <= 4: single-token decode).  The eval path of the reference quantizes the
+// activations and then multiplies (block_linear.py:141-144): two launches of which the first moves a few KiB.  Here
+// every workgroup first starts its W loads exactly as gemm_gemv does, then quantizes the whole of x [M,K] (read
+// through L2) into LDS -- int8 codes [M][K] and row scales [K-block][4] -- with the arithmetic of the row quantizer
+// (same helpers, same results), and runs the gemm_gemv loop with its A operands read from LDS.  The output is bit for
+// bit that of bi8_quantize_rowwise followed by bi8_gemm_nt_dequant.
+constexpr int kFewRowsMax = 4;
+constexpr size_t kFewRowsLdsMax = 64 * 1024;
+template <int BLK, int DT>
+__global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const void *__restrict__ x, int64_t ldx) {
+    constexpr int NW = 4, D = kGemvDepth;
+    constexpr int NBS = kStageK / BLK;
+    constexpr int VEC = Bi8Vec<DT>::kElems;
+    constexpr int L = BLK / VEC;                   // lanes that hold one K-block of one row
+    constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
+    constexpr int64_t ES = 16 / VEC;
+    constexpr int U = 4;                           // 16-byte loads of x in flight per lane
+    static_assert(BLK == 64 || BLK == 128, "one or two 64-byte MFMAs per K-block");
+    extern __shared__ __attribute__((aligned(16))) float gemv_lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, q = lane >> 4;
+    const int K = (int)g.K, M = (int)g.M;
+    const int nstages = K / kStageK;
+    const int nblk = nstages * NBS;
+    float(*red)[4][64] = (float(*)[4][64])gemv_lds;                 // [wave][register][lane]
+    float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][4 rows]
+    int8_t *s_a = (int8_t *)(s_sx + (size_t)nblk * 4);               // [M][K], 16-byte aligned
+    const int64_t n = (int64_t)blockIdx.x * 16 + r16;
+    const int64_t nc = n < g.N ? n : g.N - 1;                       // clamped: never stored
+    const int8_t *wrow = g.W + nc * g.ldw + q * 16;
+
+    bi8_v4i wf[D][2];
+    float swf[D][NBS];
+    auto load_stage = [&](int t, bi8_v4i *w, float *sw) {
+        const int s = wave + NW * t;
+        if (s < nstages) {                         // wave-uniform
+            const int64_t k0 = (int64_t)s * kStageK;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) w[kb] = __builtin_nontemporal_load((const bi8_v4i *)(wrow + k0 + kb * 64));
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) sw[b] = g.sW[((int64_t)s * NBS + b) * g.N + nc];
+        } else {
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) sw[b] = 0.0f;
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+        wf[d][0] = wf[d][1] = bi8_v4i{0, 0, 0, 0};
+        load_stage(d, wf[d], swf[d]);
+    }
+
+    // x -> codes and scales in LDS.  Chunk c = 16 bytes of x; K % 128 == 0 makes every aligned group of L chunks one
+    // K-block of one row, and a group is either all inside x or all past its end.
+    const char *xb = (const char *)x;
+    const int cpr = K / VEC;                       // chunks per row
+    const int total = M * cpr;
+    for (int c0 = 0; c0 < total; c0 += 256 * U) {
+        bi8_v4u raw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * 256 + tid;
+            raw[u] = bi8_v4u{0u, 0u, 0u, 0u};
+            if (c < total) raw[u] = *(const bi8_v4u *)(xb + ((int64_t)(c / cpr) * ldx + (int64_t)(c % cpr) * VEC) * ES);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * 256 + tid;
+            if (c0 + u * 256 + (tid & ~63) >= total) break;        // wave-uniform: nothing left for this wave
+            const int row = c / cpr, col = (c % cpr) * VEC;
+            float f[VEC];
+            bi8_unpack<DT>(raw[u], f);
+            float m = 0.0f;
+            bool special = false;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                m = __builtin_fmaxf(m, __builtin_fabsf(f[e]));
+                special |= (f[e] != f[e]);
+            }
+            m = bi8_group_max<L>(m);
+            special |= !bi8_scale_is_ordinary(m);
+            uint32_t code[VEC];
+            if (__builtin_expect(special, 0)) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) code[e] = bi8_code_slow(f[e], m);
+            } else {
+                const float y = 1.0f / m;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) code[e] = bi8_code_fast<NCORR>(f[e], m, y);
+            }
+            if (c < total) {
+                if ((lane & (L - 1)) == 0) s_sx[(col / BLK) * 4 + row] = m;
+                int8_t *dst = s_a + row * K + col;
+                if constexpr (VEC == 4) {
+                    *(uint32_t *)dst = bi8_pack4(code[0], code[1], code[2], code[3]);
+                } else {
+                    *(bi8_v2u *)dst = bi8_v2u{bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
+                }
+            }
+        }
+    }
+    for (int i = tid; i < nblk * 4; i += 256)
+        if ((i & 3) >= M) s_sx[i] = 0.0f;
+    __syncthreads();
+
+    // the A operands follow the W ring one slot behind its refill: read from LDS a whole ring ahead of their use
+    const bool m_ok = r16 < M;
+    const int8_t *arow = s_a + (m_ok ? r16 : 0) * K + q * 16;
+    bi8_v4i af[D][2];
+    auto read_a = [&](int t, bi8_v4i *a) {
+        const int s = wave + NW * t;
+        const int sc = s < nstages ? s : nstages - 1;              // stages past the end fold with column scale 0
+        a[0] = a[1] = bi8_v4i{0, 0, 0, 0};
+        if (m_ok) {
+            a[0] = *(const bi8_v4i *)(arow + sc * kStageK);
+            a[1] = *(const bi8_v4i *)(arow + sc * kStageK + 64);
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) read_a(d, af[d]);
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int mine = (nstages - wave + NW - 1) / NW;
+    for (int base = 0; base < mine; base += D) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) {
+            const int t = base + d;
+            const int s = wave + NW * t;
+            const int sb = (s < nstages ? s : nstages - 1) * NBS;
+            const bi8_v4i zero = {0, 0, 0, 0};
+            bi8_v4i p[NBS];
+            if constexpr (NBS == 1) {
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][0], wf[d][0], zero, 0, 0, 0);
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][1], wf[d][1], p[0], 0, 0, 0);
+            } else {
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][0], wf[d][0], zero, 0, 0, 0);
+                p[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][1], wf[d][1], zero, 0, 0, 0);
+            }
+            float swv[NBS];
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) swv[b] = swf[d][b];
+            load_stage(t + D, wf[d], swf[d]);                       // refill the slot
+            read_a(t + D, af[d]);
+#pragma unroll
+            for (int b = 0; b < NBS; ++b) {
+                const bi8_v4f sx = *(const bi8_v4f *)(s_sx + (sb + b) * 4);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf((float)p[b][r] * sx[r], swv[b], acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
+    __syncthreads();
+    if (wave == 0 && q == 0) {                     // rows 0..3 live in lanes 0..15
+        const float div = (float)(1.0 / (127.0 * 127.0));
+        const bool has_bias = g.bias != nullptr;
+        const float bias = (has_bias && n < g.N) ? load_bias(g, n) : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float v = red[0][r][lane];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) v += red[w][r][lane];
+            if (r < M && n < g.N) store_c<DT>(g.C, (int64_t)r * g.ldc + n, v * div, has_bias, bias);
+        }
+    }
+}
+
 // Fallback for any K, block, alignment: 4 waves, each a 32x32 output subtile; every lane gathers its own
 // 16-byte MFMA operands with byte loads (zero outside the matrix and outside the current K-block).
 template <int CDT, bool PARTIALS>
@@ -1270,6 +1439,35 @@ extern "C" int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float
     case BI8_F32: return dispatch<BI8_F32, false>(g, block, st);
     case BI8_BF16: return dispatch<BI8_BF16, false>(g, block, st);
     default: return dispatch<BI8_F16, false>(g, block, st);
+    }
+}
+
+template <int DT> int launch_few_rows(const GemmArgs &g, const void *x, int64_t ldx, int block, size_t lds, hipStream_t st) {
+    const unsigned tn = (unsigned)((g.N + 15) / 16);
+    if (block == 64) hipLaunchKernelGGL((linear_few_rows<64, DT>), dim3(tn), dim3(256), lds, st, g, x, ldx);
+    else hipLaunchKernelGGL((linear_few_rows<128, DT>), dim3(tn), dim3(256), lds, st, g, x, ldx);
+    return bi8_launch_rc();
+}
+
+extern "C" int bi8_linear_few_rows(const void *x, int dtype, const int8_t *W, const float *sW, const void *bias, int bias_dtype,
+                                   void *C, int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldc, int block,
+                                   void *stream) {
+    if (dtype < 0 || dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return BI8_ERR_BAD_DTYPE;
+    if (block < 1 || block > (1 << 20)) return BI8_ERR_BAD_BLOCK;
+    if (M < 0 || N < 0 || K < 0 || ldx < K || ldw < K || ldc < N) return BI8_ERR_BAD_SHAPE;
+    if (!x || !W || !sW || !C) return BI8_ERR_NULL_POINTER;
+    const int64_t vec = dtype == BI8_F32 ? 4 : 8;
+    if (M < 1 || M > kFewRowsMax || N < 1 || (block != 64 && block != 128) || K < kStageK || K % kStageK != 0 || ldx % vec != 0 ||
+        ldw % 16 != 0 || !bi8_aligned(x, 16) || !bi8_aligned(W, 16) || !bi8_aligned(sW, 4) || (N + 15) / 16 > 0x7fffffffLL)
+        return BI8_ERR_UNSUPPORTED;
+    const size_t lds = (4 * 4 * 64 + (size_t)(K / block) * 4) * sizeof(float) + (size_t)M * (size_t)K;
+    if (lds > kFewRowsLdsMax) return BI8_ERR_UNSUPPORTED;
+    GemmArgs g{nullptr, W, nullptr, sW, bias, C, nullptr, M, N, K, 0, ldw, ldc, 0, 0, bias_dtype};
+    hipStream_t st = (hipStream_t)stream;
+    switch (dtype) {
+    case BI8_F32: return launch_few_rows<BI8_F32>(g, x, ldx, block, lds, st);
+    case BI8_BF16: return launch_few_rows<BI8_BF16>(g, x, ldx, block, lds, st);
+    default: return launch_few_rows<BI8_F16>(g, x, ldx, block, lds, st);
     }
 }
 

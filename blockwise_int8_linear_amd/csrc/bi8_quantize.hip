@@ -15,35 +15,11 @@ constexpr int kRows = 4 * kRowsPerWave;    // rows per workgroup tile
 constexpr int kChunks = 1;                 // 1 KiB wave-loads per row per tile (2 and 4 measured slower)
 constexpr int kThreads = 256;
 
-template <int DT> struct Vec {
-    static constexpr int kElems = (DT == BI8_F32) ? 4 : 8;     // elements per 16-byte load
-};
-
-// 16 raw bytes -> kElems floats
-template <int DT> __device__ __forceinline__ void unpack(const bi8_v4u &raw, float *f) {
-    if constexpr (DT == BI8_F32) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) f[e] = bi8_u2f(raw[e]);
-    } else if constexpr (DT == BI8_BF16) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f[2 * e] = bi8_u2f(raw[e] << 16);
-            f[2 * e + 1] = bi8_u2f(raw[e] & 0xffff0000u);
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f[2 * e] = bi8_from_f16_bits(raw[e] & 0xffffu);
-            f[2 * e + 1] = bi8_from_f16_bits(raw[e] >> 16);
-        }
-    }
-}
-
 template <int DT, int L>
 __global__ __launch_bounds__(kThreads) void quantize_rows_vec(const void *__restrict__ x, int8_t *__restrict__ q,
                                                               float *__restrict__ scales, int64_t M, int64_t K,
                                                               int64_t ldx, int64_t ldq, int64_t nblk, int tiles_k) {
-    constexpr int VEC = Vec<DT>::kElems;
+    constexpr int VEC = Bi8Vec<DT>::kElems;
     constexpr int B = L * VEC;                       // block size in elements
     constexpr int TE = kChunks * BI8_WAVE * VEC;     // elements of one row covered by a tile
     constexpr int NB = TE / B;                       // K-blocks per tile row
@@ -81,7 +57,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_vec(const void *__rest
         for (int c = 0; c < kChunks; ++c) {
             const int64_t col = col0 + (c * BI8_WAVE + lane) * VEC;
             float f[VEC];
-            unpack<DT>(raw[i][c], f);
+            bi8_unpack<DT>(raw[i][c], f);
             float m = 0.0f;
             bool special = false;
 #pragma unroll
@@ -199,7 +175,7 @@ int launch_loose(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, 
 
 template <int DT, int L>
 int launch_vec(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int64_t ldx, int64_t ldq, hipStream_t st) {
-    constexpr int VEC = Vec<DT>::kElems;
+    constexpr int VEC = Bi8Vec<DT>::kElems;
     constexpr int B = L * VEC;
     constexpr int TE = kChunks * BI8_WAVE * VEC;
     const int64_t tiles_k = (K + TE - 1) / TE;
@@ -213,7 +189,7 @@ int launch_vec(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, in
 
 template <int DT>
 int dispatch(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int64_t ldx, int64_t ldq, int block, hipStream_t st) {
-    constexpr int VEC = Vec<DT>::kElems;
+    constexpr int VEC = Bi8Vec<DT>::kElems;
     const bool vec_ok = bi8_pow2(block) && block >= VEC && block <= 64 * VEC && K % VEC == 0 && ldx % VEC == 0 &&
                         ldq % VEC == 0 && bi8_aligned(x, 16) && bi8_aligned(q, VEC);
     if (vec_ok) {

@@ -15,29 +15,6 @@ constexpr int kThreads = 256;
 constexpr int kPitch = kTC + 1;    // fp32 tile pitch: column walks hit distinct banks
 constexpr int kQPitch = kTR + 4;   // code tile pitch in bytes (33 dwords)
 
-template <int DT> struct Vec {
-    static constexpr int kElems = (DT == BI8_F32) ? 4 : 8;
-};
-
-template <int DT> __device__ __forceinline__ void unpack(const bi8_v4u &raw, float *f) {
-    if constexpr (DT == BI8_F32) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) f[e] = bi8_u2f(raw[e]);
-    } else if constexpr (DT == BI8_BF16) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f[2 * e] = bi8_u2f(raw[e] << 16);
-            f[2 * e + 1] = bi8_u2f(raw[e] & 0xffff0000u);
-        }
-    } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            f[2 * e] = bi8_from_f16_bits(raw[e] & 0xffffu);
-            f[2 * e + 1] = bi8_from_f16_bits(raw[e] >> 16);
-        }
-    }
-}
-
 // B in {32, 64, 128}: thread (c = tid % 64, g = tid / 64) owns source rows 32g .. 32g+31 of column c.
 // VLOAD / VSTORE: the source rows / the output rows are 16-byte aligned, so a lane moves 16 bytes at a time; without
 // them the same tile is read element by element (64 consecutive elements per wave instruction) and written byte by
@@ -46,7 +23,7 @@ template <int DT, int B, bool VLOAD, bool VSTORE>
 __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__restrict__ x, int8_t *__restrict__ qT,
                                                                float *__restrict__ scalesT, int64_t R, int64_t C,
                                                                int64_t ldx, int64_t ldq, int64_t tiles_c, int64_t ntiles) {
-    constexpr int VEC = Vec<DT>::kElems;
+    constexpr int VEC = Bi8Vec<DT>::kElems;
     constexpr int64_t ES = 16 / VEC;
     constexpr int LPR = kTC / VEC;                 // lanes per tile row
     constexpr int RPP = kThreads / LPR;            // rows per load pass
@@ -101,7 +78,7 @@ __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__res
                 const int r = p * RPP + tid / LPR;
                 const int cc = (tid % LPR) * VEC;
                 float f[VEC];
-                unpack<DT>(raw[p], f);
+                bi8_unpack<DT>(raw[p], f);
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) s_x[r * kPitch + cc + e] = f[e];
             }
@@ -224,7 +201,7 @@ int launch_tile(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C,
 
 template <int DT, int B>
 int launch_tile_any(const void *x, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq, hipStream_t st) {
-    constexpr int VEC = Vec<DT>::kElems;
+    constexpr int VEC = Bi8Vec<DT>::kElems;
     const bool vload = C % VEC == 0 && ldx % VEC == 0 && bi8_aligned(x, 16);
     const bool vstore = ldq % 16 == 0 && bi8_aligned(qT, 16);
     if (vload && vstore) return launch_tile<DT, B, true, true>(x, qT, scalesT, R, C, ldx, ldq, st);

@@ -194,6 +194,45 @@ def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
     return c
 
 
+_FEW_ROWS = 4
+_FEW_ROWS_LDS = 64 * 1024
+
+
+def linear_few_rows(x, W_int8, state_W, bias=None):
+    """``quantize_block_rowwise(x)`` followed by ``int8_matmul_block64_rowwise_dequantize(x_int8, W_int8.t(),
+    state_x, state_W, bias)`` (BlockInt8Linear.infer, block_linear.py:141-144) as ONE kernel, for the few-row case of
+    token-by-token decode: x [M,K] float with 1 <= M <= 4, W_int8 [N,K] and state_W [K/B, N] the cached weights.
+    Returns the same bits as the two launchers, or None when the operands are outside what the fused kernel covers
+    (the caller then runs the two launchers)."""
+    block = block_linear_config.GROUP_SIZE
+    dtype = block_linear_config.INPUT_OUTPUT_TORCH_TYPE
+    M, K = x.shape
+    N = W_int8.shape[0]
+    if not (1 <= M <= _FEW_ROWS and block in (64, 128) and K > 0 and K % 128 == 0 and N > 0 and x.dtype == dtype
+            and x.dtype in _DT and W_int8.dtype == torch.int8 and state_W.dtype == torch.float32
+            and 4096 + 16 * (K // block) + M * K <= _FEW_ROWS_LDS):
+        return None
+    assert x.is_cuda and W_int8.is_cuda
+    assert W_int8.shape[1] == K and tuple(state_W.shape) == (K // block, N), "incompatible dimensions"
+    x, w = _rows(x), _rows(W_int8)
+    state_W = state_W if state_W.is_contiguous() else state_W.contiguous()
+    bias_ptr, bias_dt = None, 0
+    if bias is not None:
+        assert bias.is_cuda and bias.numel() == N
+        if bias.dtype not in _DT:
+            bias = bias.float()
+        bias = bias.contiguous()
+        bias_ptr, bias_dt = bias.data_ptr(), _DT[bias.dtype]
+    c = torch.empty((M, N), device=x.device, dtype=dtype)
+    with _on_device(x):
+        rc = _lib.load().bi8_linear_few_rows(x.data_ptr(), _DT[dtype], w.data_ptr(), state_W.data_ptr(), bias_ptr, bias_dt,
+                                             c.data_ptr(), M, N, K, _ld(x), _ld(w), N, block, _stream(x))
+    if rc == _lib.ERR_UNSUPPORTED:          # alignment of a view, for instance
+        return None
+    _lib.check(rc, "bi8_linear_few_rows")
+    return c
+
+
 def int8_matmul_block_partials(a, b, fblock_size=None):
     """The GEMM kernel's int32 block partials, before any scaling: int32 [ceil(K/B), M, N]
     (what ``tl.dot`` yields at triton_functions.py:115).  Parity/debug operator."""

@@ -41,6 +41,7 @@ extern "C" {
 #define BI8_ERR_BAD_BLOCK 3
 #define BI8_ERR_BAD_SHAPE 4   /* negative size, or a leading dimension smaller than the row length */
 #define BI8_ERR_TOO_LARGE 5   /* a dimension exceeds what one launch can index */
+#define BI8_ERR_UNSUPPORTED 6 /* valid arguments outside what this entry point covers; nothing was launched */
 #define BI8_ERR_HIP_BASE 1000 /* BI8_ERR_HIP_BASE + hipError_t */
 
 /* ABI version of this header (bumped on any signature change). */
@@ -103,6 +104,23 @@ int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float *sA, const
 int bi8_gemm_nt_partials(const int8_t *A, const int8_t *W, int32_t *P,
                          int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw,
                          int block, void *stream);
+
+/*
+ * Quantize + GEMM of the eval path in ONE launch for at most 4 rows (single-token decode).  Replaces the pair
+ * `quantize_block_rowwise(X)` + `int8_matmul_block64_rowwise_dequantize(X_int8, W_int8.t(), state_X, state_W, bias)`
+ * of BlockInt8Linear.infer (block_linear.py:141-144) when X has 1..4 rows.
+ *   x     [M,K] of `dtype`, leading dimension ldx   (activations, not yet quantized)
+ *   W     int8 [N,K], leading dimension ldw;  sW fp32 [K/block, N]   (the cached weights, block_linear.py:127-128)
+ *   C     [M,N] of the same `dtype`, leading dimension ldc;  bias [N] of bias_dtype or NULL
+ * The result is bit for bit that of bi8_quantize_rowwise followed by bi8_gemm_nt_dequant on the same operands.
+ * Covers 1 <= M <= 4, block 64 or 128, K a positive multiple of 128 with 4096 + 16*K/block + M*K <= 65536 (the
+ * quantized rows sit in LDS), x and W 16-byte aligned with ldx*sizeof(elem) and ldw multiples of 16; anything else
+ * returns BI8_ERR_UNSUPPORTED and the caller uses the two separate entry points.
+ */
+int bi8_linear_few_rows(const void *x, int dtype, const int8_t *W, const float *sW,
+                        const void *bias, int bias_dtype, void *C,
+                        int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldc,
+                        int block, void *stream);
 
 #ifdef __cplusplus
 }

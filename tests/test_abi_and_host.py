@@ -30,7 +30,8 @@ def _header_decls():
 def test_library_exports_every_declared_symbol():
     decls = _header_decls()
     assert set(decls) == {"bi8_version", "bi8_strerror", "bi8_quantize_rowwise", "bi8_quantize_transposed",
-                          "bi8_dequantize_rowwise", "bi8_gemm_nt_dequant", "bi8_gemm_nt_partials"}
+                          "bi8_dequantize_rowwise", "bi8_gemm_nt_dequant", "bi8_gemm_nt_partials",
+                          "bi8_linear_few_rows"}
     lib = _lib.load()
     for name in decls:
         assert hasattr(lib, name), f"{name} not exported"
@@ -57,7 +58,7 @@ def test_ctypes_signatures_match_header():
 
 def test_version_and_error_strings():
     lib = _lib.load()
-    assert lib.bi8_version() == _lib.ABI_VERSION == 1
+    assert lib.bi8_version() == _lib.ABI_VERSION == 2
     assert lib.bi8_strerror(0) == b"success"
     assert b"block" in lib.bi8_strerror(3)
     with pytest.raises(_lib.Bi8Error, match="leading dimension"):
@@ -80,6 +81,14 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.bi8_gemm_nt_dequant(p, p, p, p, p, 9, p, 1, 4, 4, 128, 128, 128, 4, 128, None) == 2
     assert lib.bi8_gemm_nt_dequant(None, None, None, None, None, 0, None, 1, 0, 4, 128, 128, 128, 4, 128, None) == 0
     assert lib.bi8_gemm_nt_partials(p, p, None, 4, 4, 128, 128, 128, 128, None) == 1
+    # x, dtype, W, sW, bias, bias_dtype, C, M, N, K, ldx, ldw, ldc, block, stream
+    assert lib.bi8_linear_few_rows(p, 1, p, p, None, 0, p, 1, 64, 256, 128, 256, 64, 128, None) == 4    # ldx < K
+    assert lib.bi8_linear_few_rows(p, 1, p, None, None, 0, p, 1, 64, 256, 256, 256, 64, 128, None) == 1  # null scales
+    assert lib.bi8_linear_few_rows(p, 1, p, p, None, 0, p, 5, 64, 256, 256, 256, 64, 128, None) == 6    # five rows
+    assert lib.bi8_linear_few_rows(p, 1, p, p, None, 0, p, 1, 64, 256, 256, 256, 64, 32, None) == 6     # block 32
+    assert lib.bi8_linear_few_rows(p, 1, p, p, None, 0, p, 1, 64, 192, 192, 192, 64, 64, None) == 6     # K % 128
+    assert lib.bi8_linear_few_rows(p, 1, p, p, None, 0, p, 4, 64, 32768, 32768, 32768, 64, 128, None) == 6  # LDS budget
+    assert b"covers" in lib.bi8_strerror(6)
 
 
 def test_python_api_mirrors_reference_names_and_defaults():
