@@ -167,3 +167,22 @@ def test_eval_path_in_a_hip_graph(pkg):
                 torch.cuda.synchronize()
                 assert torch.equal(static_y, eager)
                 assert torch.isfinite(static_y.float()).all()
+
+
+def test_reference_benchmark_sweep_and_accuracy_demo(pkg):
+    """the sweep of triton_functions.py:521-566 at two small sizes (every provider returns positive rates) and the
+    demo scenario of block_linear.py:161-224 (errors of a few percent at most, smaller for smaller blocks)"""
+    from blockwise_int8_linear_amd import triton_functions as tf
+    from blockwise_int8_linear_amd.examples import accuracy
+    rows = tf.benchmark(sizes=[256, 512], print_data=False)
+    assert set(rows) == {"dense", "blockwise_int8", "blockwise_int8_quantise", "dense+copy"}
+    assert all(len(v) == 2 and all(r[1] > 0 for r in v) for v in rows.values())
+    a = torch.randn(70, 256, device=DEV).bfloat16()
+    b = torch.randn(90, 256, device=DEV).bfloat16()
+    assert ((tf.fast_matmulT(a, b).float() - a.float() @ b.float().t()).norm() / (a.float() @ b.float().t()).norm()).item() < 0.03
+    err = {blk: accuracy.demo_case(blk) for blk in (32, 128)}
+    for blk in err:
+        for what in ("output", "grad_weight", "grad_input"):
+            assert err[blk][what]["rel"] < 0.03
+    assert err[32]["output"]["rel"] < err[128]["output"]["rel"]
+    assert accuracy.forward_case()["rel"] < 0.03
