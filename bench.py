@@ -102,8 +102,8 @@ def bench_quantize(pkg, torch, iters: int):
 def bench_extras(pkg, torch):
     """secondary figures of the same path, all through the C ABI with preallocated outputs: the block-64 GEMM at
     8192^3, the few-row (decode) GEMM at Llama-7B shapes with the weights rotated through ~600 MB so that they come
-    from HBM (and the one-token eval-path linear, quantize included, as two launches and as one kernel), and the
-    transposed quantizer of the backward pass"""
+    from HBM (and the one-token eval-path linear, quantize included, as two launches and as one kernel), the
+    transposed quantizer of the backward pass and the quantizer that writes both directions from one read"""
     from blockwise_int8_linear_amd import _lib
     lib = _lib.load()
     st = torch.cuda.current_stream().cuda_stream
@@ -181,6 +181,21 @@ def bench_extras(pkg, torch):
     nbytes = M * K * 3 + 4 * M * K // 128
     out["quantize_transposed_bf16_8192"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
                                             "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
+
+    # both directions from one read (three buffer sets again)
+    qr = [torch.empty(M, K, device="cuda", dtype=torch.int8) for _ in range(3)]
+    sr = [torch.empty(K // 128, M, device="cuda", dtype=torch.float32) for _ in range(3)]
+
+    def qd():
+        i = turn[0] = (turn[0] + 1) % 3
+        assert lib.bi8_quantize_dual(xs[i].data_ptr(), 1, qr[i].data_ptr(), sr[i].data_ptr(), qs[i].data_ptr(), ss[i].data_ptr(),
+                                     M, K, K, K, M, 128, st) == 0
+    for _ in range(6):
+        qd()
+    t = min(event_ms(qd, 30) for _ in range(2))
+    nbytes = M * K * 4 + 8 * M * K // 128
+    out["quantize_dual_bf16_8192"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
+                                      "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
     return out
 
 

@@ -12,6 +12,7 @@ from .ops import (
     int8_matmul_block64_rowwise_dequantize,
     int8_matmul_block_partials,
     linear_few_rows,
+    quantize_block_dual,
     quantize_block_rowwise,
     quantize_block_transposed,
 )
@@ -20,5 +21,5 @@ __all__ = [
     "block_linear_config", "BlockInt8Linear", "BlockLinear", "blockwise_int8_linear",
     "replace_linear_with_blockwise_int8", "quantize_block_rowwise", "quantize_block_transposed",
     "dequantize_block_rowwise", "int8_matmul_block64_rowwise_dequantize", "int8_matmul_block_partials",
-    "linear_few_rows",
+    "linear_few_rows", "quantize_block_dual",
 ]

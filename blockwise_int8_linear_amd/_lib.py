@@ -22,6 +22,7 @@ SIGNATURES = {
     "bi8_strerror": (ctypes.c_char_p, [_ci]),
     "bi8_quantize_rowwise": (_ci, [_vp, _ci, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_quantize_transposed": (_ci, [_vp, _ci, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp]),
+    "bi8_quantize_dual": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_dequantize_rowwise": (_ci, [_vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_gemm_nt_dequant": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_gemm_nt_partials": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),

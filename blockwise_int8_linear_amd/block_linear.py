@@ -3,8 +3,9 @@ backward run blockwise-int8 GEMMs), its autograd function and the model-surgery 
 HIP operators of ``ops.py``.
 
 Differences from the reference that do not change results:
-  * the backward pass quantizes the transposes of W, X and G with one fused kernel each instead of
-    ``.t().contiguous()`` followed by the row quantizer (block_linear.py:93-94, :100-103);
+  * the transposes of W, X and G that the backward pass quantizes (``.t().contiguous()`` followed by the row
+    quantizer, block_linear.py:93-94, :100-103) are never materialized, and each of X, W and G is read once for both
+    of its quantization directions (X and W in the forward pass, whose transposed codes are what is saved for backward);
   * ``ctx.save_for_backward`` is called, not assigned over (block_linear.py:73);
   * switching the module back to training mode drops the cached int8 weights, so a later ``eval()``
     re-quantizes the current weights (the reference keeps serving the first cache, block_linear.py:138-139);
@@ -20,6 +21,7 @@ from .ops import (
     dequantize_block_rowwise,
     int8_matmul_block64_rowwise_dequantize,
     linear_few_rows,
+    quantize_block_dual,
     quantize_block_rowwise,
     quantize_block_transposed,
 )
@@ -43,14 +45,28 @@ def replace_linear_with_blockwise_int8(model):
 
 
 class blockwise_int8_linear(torch.autograd.Function):
-    """y = x @ W.T + bias with both operands block-quantized on the fly (block_linear.py:69-112)."""
+    """y = x @ W.T + bias with both operands block-quantized on the fly (block_linear.py:69-112).
+
+    The backward pass needs X and W quantized along the other direction (blocks over the tokens for grad_W, over the
+    output features for grad_X; block_linear.py:93-94, :100-103).  Those codes are produced in the forward pass by the
+    same read of X and W (``quantize_block_dual``) and saved in place of X and W; the numbers are the ones the
+    reference computes from the saved X and W in its backward."""
 
     @staticmethod
     def forward(ctx, X_3D, W, bias):
         X = X_3D.reshape(-1, X_3D.size(-1))
-        ctx.save_for_backward(X, W)
-        X_int8, state_X = quantize_block_rowwise(X)
-        W_int8, state_W = quantize_block_rowwise(W)
+        need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if need_gw:
+            X_int8, state_X, Xt_int8, Xt_state = quantize_block_dual(X)         # [M,K] and [K,M], [M/B,K]
+        else:
+            X_int8, state_X = quantize_block_rowwise(X)
+            Xt_int8 = Xt_state = None
+        if need_gx:
+            W_int8, state_W, Wt_int8, Wt_state = quantize_block_dual(W)         # [N,K] and [K,N], [N/B,K]
+        else:
+            W_int8, state_W = quantize_block_rowwise(W)
+            Wt_int8 = Wt_state = None
+        ctx.save_for_backward(Xt_int8, Xt_state, Wt_int8, Wt_state)
         out = int8_matmul_block64_rowwise_dequantize(X_int8, W_int8.t(), state_X, state_W, bias)
         return out.view(*X_3D.size()[:-1], -1)
 
@@ -58,18 +74,21 @@ class blockwise_int8_linear(torch.autograd.Function):
     def backward(ctx, G_3D):
         G = G_3D.reshape(-1, G_3D.size(-1))
         grad_X = grad_W = grad_bias = None
-        X, W = ctx.saved_tensors
-        if ctx.needs_input_grad[0]:
-            # grad_X [M,K] = G [M,N] @ W [N,K]: contraction over N, so W is requantized along N
+        Xt_int8, Xt_state, Wt_int8, Wt_state = ctx.saved_tensors
+        need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if need_gx and need_gw:
+            g_int8, g_state, gt_int8, gt_state = quantize_block_dual(G)         # one read of G for both GEMMs
+        elif need_gx:
             g_int8, g_state = quantize_block_rowwise(G)
-            Wt_int8, w_state = quantize_block_transposed(W)                 # [K,N], [N/B,K]
-            grad_X = int8_matmul_block64_rowwise_dequantize(g_int8, Wt_int8.t(), g_state, w_state)
+        elif need_gw:
+            gt_int8, gt_state = quantize_block_transposed(G)                    # [N,M], [M/B,N]
+        if need_gx:
+            # grad_X [M,K] = G [M,N] @ W [N,K]: contraction over N, W quantized along N
+            grad_X = int8_matmul_block64_rowwise_dequantize(g_int8, Wt_int8.t(), g_state, Wt_state)
             grad_X = grad_X.view(*G_3D.size()[:-1], -1)
-        if ctx.needs_input_grad[1]:
-            # grad_W [N,K] = G.T [N,M] @ X [M,K]: contraction over the tokens, both requantized along M
-            x_int8, x_state = quantize_block_transposed(X)                  # [K,M], [M/B,K]
-            gt_int8, gt_state = quantize_block_transposed(G)                # [N,M], [M/B,N]
-            grad_W = int8_matmul_block64_rowwise_dequantize(gt_int8, x_int8.t(), gt_state, x_state)
+        if need_gw:
+            # grad_W [N,K] = G.T [N,M] @ X [M,K]: contraction over the tokens, both quantized along M
+            grad_W = int8_matmul_block64_rowwise_dequantize(gt_int8, Xt_int8.t(), gt_state, Xt_state)
         if ctx.needs_input_grad[2]:
             grad_bias = G.sum(dim=0)
         return grad_X, grad_W, grad_bias

@@ -1,0 +1,242 @@
+// Block quantize in both directions at once (bi8_quantize_dual): x [R,C] -> codes [R,C] with scales [ceil(C/B), R]
+// (blocks along the rows, what bi8_quantize_rowwise writes) AND codes [C,R] with scales [ceil(R/B), C] (blocks down
+// the columns, what bi8_quantize_transposed writes), from one pass over x.  A training step of the reference
+// quantizes each of X, W and G twice, once per direction (block_linear.py:77-78, :92-94, :100-103): with this kernel
+// every one of them is read from HBM once.
+//
+// A workgroup owns a 128 x 128 tile, held in registers as two 64-column halves (16 bytes per lane per row pass; the
+// next tile's loads are issued while this one is processed).  The row direction is finished straight from the
+// registers: the lanes of one row reduce their absmax with DPP, quantize and store their codes.  The column direction
+// runs half by half through LDS exactly as in bi8_quantize_transposed.  Both outputs are bit for bit those of the
+// two separate entry points.
+#include "bi8_common.h"
+
+namespace {
+
+constexpr int kTR = 128;           // tile rows
+constexpr int kTC = 64;            // columns of one half
+constexpr int kThreads = 256;
+constexpr int kPitch = kTC + 1;    // fp32 half-tile pitch: column walks hit distinct banks
+constexpr int kQPitch = kTR + 4;   // code tile pitch in bytes (33 dwords)
+
+template <int DT, int B>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == BI8_F32 ? 2 : 3))) void quantize_dual_tile(const void *__restrict__ x, int8_t *__restrict__ q,
+                                                               float *__restrict__ scales, int8_t *__restrict__ qT,
+                                                               float *__restrict__ scalesT, int64_t R, int64_t C, int64_t ldx,
+                                                               int64_t ldq, int64_t ldqt, int64_t tiles_c, int64_t ntiles) {
+    constexpr int VEC = Bi8Vec<DT>::kElems;
+    constexpr int64_t ES = 16 / VEC;
+    constexpr int LPR = kTC / VEC;                 // lanes per half row: 8 (16-bit) or 16 (fp32)
+    constexpr int RPP = kThreads / LPR;            // rows per load pass
+    constexpr int NP = kTR / RPP;                  // load passes per half
+    constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
+    constexpr int GPB = B / 32;                    // 32-row groups per column block
+    constexpr int LB = (B < kTC ? B : kTC) / VEC;  // lanes of one half row that share a row block
+    static_assert(B == 32 || B == 64 || B == 128, "tile = one or more whole blocks in both directions");
+    __shared__ float s_x[kTR * kPitch];
+    __shared__ float s_max[4][kTC];
+    __shared__ __attribute__((aligned(16))) uint8_t s_q[kTC * kQPitch];
+
+    const int tid = threadIdx.x;
+    const char *xb = (const char *)x;
+    const int lr = tid / LPR;                      // row inside a pass
+    const int cc = (tid % LPR) * VEC;              // first column of this lane inside a half
+
+    auto load_half = [&](int64_t tile, int h, bi8_v4u *raw) {
+        const int64_t r0 = (tile / tiles_c) * kTR;
+        const int64_t c0 = (tile % tiles_c) * (2 * kTC) + h * kTC;
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int r = p * RPP + lr;
+            raw[p] = bi8_v4u{0u, 0u, 0u, 0u};
+            if (tile < ntiles && r0 + r < R && c0 + cc < C)
+                raw[p] = __builtin_nontemporal_load((const bi8_v4u *)(xb + ((r0 + r) * ldx + c0 + cc) * ES));
+        }
+    };
+
+    bi8_v4u raw[2][NP];
+    load_half(blockIdx.x, 0, raw[0]);
+    load_half(blockIdx.x, 1, raw[1]);
+    for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
+        const int64_t r0 = (tile / tiles_c) * kTR;
+        const int64_t cbase = (tile % tiles_c) * (2 * kTC);
+
+        // ---- along the rows, from the registers ----------------------------------------------------------------
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int64_t row = r0 + p * RPP + lr;
+            float f[2][VEC];
+            float m[2];
+            bool special[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                bi8_unpack<DT>(raw[h][p], f[h]);
+                m[h] = 0.0f;
+                special[h] = false;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    m[h] = __builtin_fmaxf(m[h], __builtin_fabsf(f[h][e]));
+                    special[h] |= (f[h][e] != f[h][e]);
+                }
+            }
+            if constexpr (B == 2 * kTC) {
+                m[0] = m[1] = bi8_group_max<LPR>(__builtin_fmaxf(m[0], m[1]));
+            } else {
+                m[0] = bi8_group_max<LB>(m[0]);
+                m[1] = bi8_group_max<LB>(m[1]);
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int64_t col = cbase + h * kTC + cc;
+                const bool live = row < R && col < C;
+                if (live && (tid % LB) == 0 && (B != 2 * kTC || h == 0)) scales[(col / B) * R + row] = m[h];
+                const bool slow = special[h] | !bi8_scale_is_ordinary(m[h]);
+                uint32_t code[VEC];
+                if (__builtin_expect(slow, 0)) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) code[e] = bi8_code_slow(f[h][e], m[h]);
+                } else {
+                    const float y = 1.0f / m[h];
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) code[e] = bi8_code_fast<NCORR>(f[h][e], m[h], y);
+                }
+                if (live) {
+                    int8_t *dst = q + row * ldq + col;
+                    if constexpr (VEC == 4) {
+                        __builtin_nontemporal_store(bi8_pack4(code[0], code[1], code[2], code[3]), (uint32_t *)dst);
+                    } else {
+                        bi8_v2u w = {bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
+                        __builtin_nontemporal_store(w, (bi8_v2u *)dst);
+                    }
+                }
+            }
+        }
+
+        // ---- down the columns, one half at a time through LDS --------------------------------------------------
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int64_t c0 = cbase + h * kTC;
+            // phase 1: this half -> fp32 in LDS (the previous half's column reads ended before the barrier that
+            // precedes its phase 4); then start the next tile's loads of this half
+#pragma unroll
+            for (int p = 0; p < NP; ++p) {
+                float f[VEC];
+                bi8_unpack<DT>(raw[h][p], f);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) s_x[(p * RPP + lr) * kPitch + cc + e] = f[e];
+            }
+            load_half(tile + gridDim.x, h, raw[h]);
+            __syncthreads();
+
+            // phase 2: column maxima over this thread's 32 rows, then over the block's row groups
+            const int c = tid & 63;
+            const int g = tid >> 6;
+            float v[32];
+            float m = 0.0f;
+            bool special = false;
+#pragma unroll
+            for (int i = 0; i < 32; ++i) {
+                v[i] = s_x[(g * 32 + i) * kPitch + c];
+                m = __builtin_fmaxf(m, __builtin_fabsf(v[i]));
+                special |= (v[i] != v[i]);
+            }
+            if constexpr (GPB > 1) {
+                s_max[g][c] = m;
+                __syncthreads();
+                const int gb = g & ~(GPB - 1);
+#pragma unroll
+                for (int k = 0; k < GPB; ++k) m = __builtin_fmaxf(m, s_max[gb + k][c]);
+            }
+            if ((g & (GPB - 1)) == 0) {
+                const int64_t jb = (r0 + g * 32) / B;
+                if (r0 + g * 32 < R && c0 + c < C) scalesT[jb * C + c0 + c] = m;
+            }
+
+            // phase 3: codes of this thread's 32 rows -> byte tile [column][row]
+            special |= !bi8_scale_is_ordinary(m);
+            uint32_t code[32];
+            if (__builtin_expect(special, 0)) {
+#pragma unroll
+                for (int i = 0; i < 32; ++i) code[i] = bi8_code_slow(v[i], m);
+            } else {
+                const float y = 1.0f / m;
+#pragma unroll
+                for (int i = 0; i < 32; ++i) code[i] = bi8_code_fast<NCORR>(v[i], m, y);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                *(uint32_t *)&s_q[c * kQPitch + g * 32 + 4 * i] = bi8_pack4(code[4 * i], code[4 * i + 1], code[4 * i + 2], code[4 * i + 3]);
+            __syncthreads();
+
+            // phase 4: 16 codes per lane, 8 lanes per output row.  The next writes to s_x come after this barrier, the
+            // next writes to s_q after the next phase-1 barrier.
+#pragma unroll
+            for (int p = 0; p < (kTC * kTR / 16) / kThreads; ++p) {
+                const int idx = p * kThreads + tid;
+                const int oc = idx / (kTR / 16);       // output row inside the half = source column
+                const int seg = idx % (kTR / 16);
+                const int64_t orow = c0 + oc;
+                const int64_t ocol = r0 + seg * 16;
+                if (orow < C && ocol < R) {
+                    const uint32_t *src = (const uint32_t *)&s_q[oc * kQPitch + seg * 16];
+                    bi8_v4u w = {src[0], src[1], src[2], src[3]};
+                    int8_t *dst = qT + orow * ldqt + ocol;
+                    if (ocol + 16 <= R) {
+                        __builtin_nontemporal_store(w, (bi8_v4u *)dst);
+                    } else {
+                        for (int e = 0; e < (int)(R - ocol); ++e) dst[e] = (int8_t)((w[e >> 2] >> (8 * (e & 3))) & 0xffu);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int DT, int B>
+int launch_dual(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq,
+                int64_t ldqt, hipStream_t st) {
+    const int64_t tiles_c = (C + 2 * kTC - 1) / (2 * kTC);
+    const int64_t tiles_r = (R + kTR - 1) / kTR;
+    const int64_t ntiles = tiles_c * tiles_r;
+    const int64_t resident = 3 * 256;              // at most three workgroups fit a CU (42 KiB of LDS each)
+    const int64_t grid = ntiles < resident ? ntiles : resident;
+    hipLaunchKernelGGL((quantize_dual_tile<DT, B>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT, R, C, ldx, ldq,
+                       ldqt, tiles_c, ntiles);
+    return bi8_launch_rc();
+}
+
+template <int DT>
+int dispatch(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq,
+             int64_t ldqt, int block, hipStream_t st) {
+    switch (block) {
+    case 32: return launch_dual<DT, 32>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
+    case 64: return launch_dual<DT, 64>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
+    default: return launch_dual<DT, 128>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
+    }
+}
+
+}  // namespace
+
+extern "C" int bi8_quantize_dual(const void *x, int x_dtype, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C,
+                                 int64_t ldx, int64_t ldq, int64_t ldqt, int block, void *stream) {
+    if (x_dtype < 0 || x_dtype > 2) return BI8_ERR_BAD_DTYPE;
+    if (block < 1 || block > (1 << 20)) return BI8_ERR_BAD_BLOCK;
+    if (R < 0 || C < 0 || ldx < C || ldq < C || ldqt < R) return BI8_ERR_BAD_SHAPE;
+    if (R == 0 || C == 0) return BI8_OK;
+    if (!x || !q || !scales || !qT || !scalesT) return BI8_ERR_NULL_POINTER;
+    const int64_t vec = x_dtype == BI8_F32 ? 4 : 8;
+    const bool one_pass = (block == 32 || block == 64 || block == 128) && C % vec == 0 && ldx % vec == 0 && bi8_aligned(x, 16) &&
+                          ldq % 8 == 0 && bi8_aligned(q, 8) && ldqt % 16 == 0 && bi8_aligned(qT, 16);
+    if (!one_pass) {
+        // other block sizes, odd row lengths, misaligned views: the two single-direction entry points, same results
+        const int rc = bi8_quantize_rowwise(x, x_dtype, q, scales, R, C, ldx, ldq, block, stream);
+        if (rc != BI8_OK) return rc;
+        return bi8_quantize_transposed(x, x_dtype, qT, scalesT, R, C, ldx, ldqt, block, stream);
+    }
+    hipStream_t st = (hipStream_t)stream;
+    switch (x_dtype) {
+    case BI8_F32: return dispatch<BI8_F32>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+    case BI8_BF16: return dispatch<BI8_BF16>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+    default: return dispatch<BI8_F16>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+    }
+}

@@ -111,6 +111,25 @@ def quantize_block_transposed(x: torch.Tensor, fblock_size=None):
     return output, _scales_out(output_maxs)
 
 
+def quantize_block_dual(x: torch.Tensor, fblock_size=None):
+    """``quantize_block_rowwise(x)`` and ``quantize_block_transposed(x)`` from one pass over x:
+    x [R,C] -> (int8 [R,C], scales [ceil(C/B), R], int8 [C,R], scales [ceil(R/B), C]), the same bits as the two calls.
+    A training step needs both directions of X, W and G (block_linear.py:77-78, :92-94, :100-103)."""
+    fblock_size = fblock_size or block_linear_config.GROUP_SIZE
+    r, c = x.shape
+    assert x.is_cuda
+    x = _rows(_float_operand(x))
+    q = torch.empty((r, c), device=x.device, dtype=torch.int8)
+    s = torch.empty((ceil_div(c, fblock_size), r), device=x.device, dtype=torch.float32)
+    qt = torch.empty((c, r), device=x.device, dtype=torch.int8)
+    st = torch.empty((ceil_div(r, fblock_size), c), device=x.device, dtype=torch.float32)
+    with _on_device(x):
+        rc = _lib.load().bi8_quantize_dual(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), qt.data_ptr(), st.data_ptr(),
+                                           r, c, _ld(x), max(c, 1), max(r, 1), fblock_size, _stream(x))
+    _lib.check(rc, "bi8_quantize_dual")
+    return q, _scales_out(s), qt, _scales_out(st)
+
+
 def dequantize_block_rowwise(x: torch.Tensor, state_x: torch.Tensor, fblock_size=None):
     """int8 [M,K] + scales [ceil(K/B), M] -> [M,K] of INPUT_OUTPUT_TORCH_TYPE; triton_functions.py:492-500."""
     fblock_size = fblock_size or block_linear_config.GROUP_SIZE

@@ -73,6 +73,19 @@ int bi8_quantize_transposed(const void *x, int x_dtype, int8_t *qT, float *scale
                             int64_t R, int64_t C, int64_t ldx, int64_t ldq, int block, void *stream);
 
 /*
+ * Both of the above from ONE pass over x: q / scales as bi8_quantize_rowwise writes them, qT / scalesT as
+ * bi8_quantize_transposed writes them (bit for bit).  A training step of the reference quantizes each of X, W and
+ * G once per direction (block_linear.py:77-78 forward, :92-94 and :100-103 backward); this entry point serves both
+ * uses of a tensor with one read of it.
+ *   x [R,C] leading dimension ldx;  q int8 [R,C] ld ldq, scales fp32 [ceil(C/block), R];
+ *   qT int8 [C,R] ld ldqt, scalesT fp32 [ceil(R/block), C]
+ * One kernel for block 32 / 64 / 128 with 16-byte aligned rows (ldq a multiple of 8, ldqt of 16); every other case
+ * runs the two single-direction kernels one after the other.
+ */
+int bi8_quantize_dual(const void *x, int x_dtype, int8_t *q, float *scales, int8_t *qT, float *scalesT,
+                      int64_t R, int64_t C, int64_t ldx, int64_t ldq, int64_t ldqt, int block, void *stream);
+
+/*
  * Block dequantize.  Replaces dequantize_block_rowwise / _dequantize_block_rowwise
  * (triton_functions.py:492-500 / :468-490):  out = (scale * float(q)) * fp32(1/127), cast to out_dtype.
  */

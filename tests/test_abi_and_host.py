@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
     decls = _header_decls()
     assert set(decls) == {"bi8_version", "bi8_strerror", "bi8_quantize_rowwise", "bi8_quantize_transposed",
                           "bi8_dequantize_rowwise", "bi8_gemm_nt_dequant", "bi8_gemm_nt_partials",
-                          "bi8_linear_few_rows"}
+                          "bi8_linear_few_rows", "bi8_quantize_dual"}
     lib = _lib.load()
     for name in decls:
         assert hasattr(lib, name), f"{name} not exported"
@@ -81,6 +81,8 @@ def test_argument_validation_happens_before_any_launch():
     assert lib.bi8_gemm_nt_dequant(p, p, p, p, p, 9, p, 1, 4, 4, 128, 128, 128, 4, 128, None) == 2
     assert lib.bi8_gemm_nt_dequant(None, None, None, None, None, 0, None, 1, 0, 4, 128, 128, 128, 4, 128, None) == 0
     assert lib.bi8_gemm_nt_partials(p, p, None, 4, 4, 128, 128, 128, 128, None) == 1
+    assert lib.bi8_quantize_dual(p, 1, p, p, p, p, 4, 128, 128, 128, 2, 128, None) == 4           # ldqt < R
+    assert lib.bi8_quantize_dual(p, 1, p, p, None, p, 4, 128, 128, 128, 4, 128, None) == 1        # null qT
     # x, dtype, W, sW, bias, bias_dtype, C, M, N, K, ldx, ldw, ldc, block, stream
     assert lib.bi8_linear_few_rows(p, 1, p, p, None, 0, p, 1, 64, 256, 128, 256, 64, 128, None) == 4    # ldx < K
     assert lib.bi8_linear_few_rows(p, 1, p, None, None, 0, p, 1, 64, 256, 256, 256, 64, 128, None) == 1  # null scales

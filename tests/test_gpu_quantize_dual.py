@@ -1,0 +1,87 @@
+"""bi8_quantize_dual (both quantization directions from one pass) against the CPU checker and against the two
+single-direction entry points: int8 codes and fp32 scales bit-exact in both outputs."""
+import pytest
+import torch
+
+import oracle
+from util import DTYPES, outlier_tensor
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import blockwise_int8_linear_amd as pkg
+    from blockwise_int8_linear_amd import _lib
+    _lib.load()
+    return pkg
+
+
+def _same(a, b):
+    return torch.equal(a.view(torch.int32) if a.dtype == torch.float32 else a, b.view(torch.int32) if b.dtype == torch.float32 else b)
+
+
+def _check(ops, x_cpu, block, x_dev=None):
+    x = x_cpu.to(DEV) if x_dev is None else x_dev
+    q, s, qt, st = ops.quantize_block_dual(x, block)
+    qo, so = oracle.quantize_block_rowwise(x_cpu, block, threads=True)
+    qto, sto = oracle.quantize_block_transposed(x_cpu, block, threads=True)
+    assert q.shape == qo.shape and s.shape == so.shape and qt.shape == qto.shape and st.shape == sto.shape
+    assert _same(s.cpu(), so), "row scales differ"
+    assert _same(st.cpu(), sto), "column scales differ"
+    assert torch.equal(q.cpu(), qo), f"{(q.cpu() != qo).sum().item()} row codes differ"
+    assert torch.equal(qt.cpu(), qto), f"{(qt.cpu() != qto).sum().item()} column codes differ"
+    q1, s1 = ops.quantize_block_rowwise(x, block)
+    q2, s2 = ops.quantize_block_transposed(x, block)
+    assert torch.equal(q, q1) and _same(s, s1) and torch.equal(qt, q2) and _same(st, s2)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("block", [32, 64, 128])
+def test_dual_parity(ops, dtype, block):
+    # whole tiles, ragged tiles in either direction, a single partial tile, one row, one 16-byte column group, many
+    # tiles per workgroup (more than 768 tiles), and shapes of the training configurations
+    for (R, C) in [(256, 256), (128, 128), (300, 1000), (1000, 72), (129, 64), (5, 8), (1, 4096), (4096, 8),
+                   (8192, 768), (768, 3072), (2176, 2304), (77, 1048)]:
+        _check(ops, outlier_tensor(R, C, DTYPES[dtype], seed=R * 3 + C + block), block)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_dual_cases_the_one_pass_kernel_does_not_take(ops, dtype):
+    """other block sizes, odd row lengths and misaligned views run the two single-direction kernels: same results"""
+    for (R, C, block) in [(200, 264, 16), (96, 520, 256), (90, 77, 64), (64, 517, 128), (300, 50257 // 50, 32)]:
+        _check(ops, outlier_tensor(R, C, DTYPES[dtype], seed=R + C), block)
+    big = outlier_tensor(130, 700, DTYPES[dtype], seed=9)
+    _check(ops, big[:, 3:3 + 512].contiguous(), 128, x_dev=big.to(DEV)[:, 3:3 + 512])        # misaligned start
+    _check(ops, big[:, 8:8 + 512].contiguous(), 128, x_dev=big.to(DEV)[:, 8:8 + 512])        # aligned view, ld 700
+
+
+def test_dual_special_values(ops):
+    x = torch.randn(256, 256, generator=torch.Generator().manual_seed(1))
+    x[0, :128] = 0.0                       # zero row block
+    x[:128, 5] = 0.0                       # zero column block
+    x[3, 130] = float("nan")
+    x[140, 7] = float("inf")
+    x[200, 128:256] *= 1e-42               # subnormal block
+    x[128:256, 200] *= 1e36                # huge column block
+    for block in (64, 128):
+        _check(ops, x, block)
+
+
+def test_dual_full_size(ops):
+    """[8192, 8192] bf16, block 128: against the two single-direction kernels (themselves checked against the CPU at
+    this size), and a 256 x 8192 slab against the CPU checker"""
+    x = outlier_tensor(8192, 8192, torch.bfloat16, seed=0).to(DEV)
+    q, s, qt, st = ops.quantize_block_dual(x, 128)
+    q1, s1 = ops.quantize_block_rowwise(x, 128)
+    q2, s2 = ops.quantize_block_transposed(x, 128)
+    assert torch.equal(q, q1) and _same(s, s1) and torch.equal(qt, q2) and _same(st, s2)
+    qo, so = oracle.quantize_block_rowwise(x[4096:4352].cpu(), 128, threads=True)
+    assert torch.equal(q[4096:4352].cpu(), qo) and _same(s[:, 4096:4352].cpu().contiguous(), so)
+
+
+def test_dual_empty(ops):
+    e = torch.empty(0, 128, device=DEV, dtype=torch.bfloat16)
+    q, s, qt, st = ops.quantize_block_dual(e, 128)
+    assert q.shape == (0, 128) and s.shape == (1, 0) and qt.shape == (128, 0) and st.shape == (0, 128)
