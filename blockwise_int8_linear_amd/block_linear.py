@@ -120,12 +120,9 @@ class BlockInt8Linear(nn.Linear):
         X = x.reshape(-1, x.size(-1))
         out = None
         if X.shape[0] <= 2:
-            # token-by-token decode: quantize and multiply in one kernel.  Every workgroup of that kernel quantizes
-            # x for itself, which pays off (measured) for one row at block 128, for two up to a medium output
-            # width, and at block 64 up to 4096 outputs
-            wide_block = self.state_W.shape[0] * 128 == X.shape[1]
-            if (wide_block and (X.shape[0] == 1 or self.out_features <= 16384)) or self.out_features <= 4096:
-                out = linear_few_rows(X, self.W_int8, self.state_W, self.bias)
+            # token-by-token decode: quantize and multiply in one kernel.  Every workgroup of that kernel quantizes x
+            # for itself, which pays off for one or two rows (measured; from four rows on the two launches are as fast)
+            out = linear_few_rows(X, self.W_int8, self.state_W, self.bias)
         if out is None:
             X_int8, state_X = quantize_block_rowwise(X)
             out = int8_matmul_block64_rowwise_dequantize(X_int8, self.W_int8.t(), state_X, self.state_W, self.bias)

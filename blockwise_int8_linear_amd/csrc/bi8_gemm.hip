@@ -38,6 +38,22 @@ __device__ __forceinline__ bi8_rsrc bi8_make_rsrc(const void *base, int64_t byte
     // dword0-1: 48-bit base, stride 0; dword2: size in bytes; dword3: raw 32-bit-format buffer (gfx9 family)
     return bi8_rsrc{(int)(uint32_t)a, (int)(uint32_t)((a >> 32) & 0xffffu), n, 0x00020000};
 }
+// The same resource as the compiler's buffer type, for loads into registers (the compiler tracks their completion):
+// the address is one VGPR offset plus one SGPR offset plus an immediate, instead of a 64-bit VGPR pointer per load.
+typedef __amdgpu_buffer_rsrc_t bi8_brsrc;
+__device__ __forceinline__ bi8_brsrc bi8_make_brsrc(const void *base, int64_t bytes) {
+    const int n = bytes > 0x7fffffffLL ? 0x7fffffff : (bytes < 0 ? 0 : (int)bytes);
+    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, n, 0x00020000);
+}
+constexpr int kBufNT = 2;          // cache policy bit "nt": streamed once
+constexpr int kBufOut = 0x40000000;  // added to a VGPR offset: beyond any range this file gives a buffer (< 2^31 bytes)
+__device__ __forceinline__ bi8_v4i bi8_buffer_load16(bi8_brsrc r, int voff, int soff, bool nt) {
+    return nt ? (bi8_v4i)__builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, kBufNT)
+              : (bi8_v4i)__builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0);
+}
+__device__ __forceinline__ float bi8_buffer_load_f32(bi8_brsrc r, int voff, int soff) {
+    return bi8_u2f(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
 __device__ __forceinline__ uint32_t bi8_lds_address(const void *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
 }
@@ -1001,47 +1017,57 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, q = lane >> 4;
-    const int64_t n = (int64_t)blockIdx.x * 16 + r16;
-    const int64_t nc = n < g.N ? n : g.N - 1;                       // clamped: never stored
-    const bool m_ok = r16 < g.M;
-    const int8_t *wrow = g.W + nc * g.ldw + q * 16;
-    const int8_t *arow = g.A + (m_ok ? r16 : 0) * g.lda + q * 16;
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int64_t n = n0 + r16;
     const int nstages = (int)(g.K / kStageK);
     const int nblk = nstages * NBS;
+    // Buffer addressing: one VGPR offset per operand (this lane's row and 16-byte chunk), the stage's K offset in an
+    // SGPR, the half-stage as an immediate.  Rows past N and past M lie beyond the range and read as zeros.
+    const int64_t wrows = g.N - n0 < 16 ? g.N - n0 : 16;
+    const bi8_brsrc rw = bi8_make_brsrc(g.W + n0 * g.ldw, (wrows - 1) * g.ldw + g.K);
+    const bi8_brsrc ra = bi8_make_brsrc(g.A, (g.M - 1) * g.lda + g.K);
+    const bi8_brsrc rs = bi8_make_brsrc(g.sW, (int64_t)nblk * g.N * 4);
+    const int voff_w = r16 * (int)g.ldw + q * 16;
+    const int voff_a = r16 * (int)g.lda + q * 16;
+    const int voff_s = (int)(n < g.N ? n : g.N - 1) * 4;           // clamped: never stored
+    const int srow = (int)g.N * 4;
 
     // stage t of this wave = global stage wave + NW * t; stages past the end are clamped and get column scale 0
     bi8_v4i wf[D][2], af[D][2];
     float swf[D][NBS];
-    auto load_stage = [&](int t, bi8_v4i *w, bi8_v4i *a, float *sw) {
+    // CHECKED loads give a stage past the end of K an offset beyond every buffer's range instead of a branch around
+    // them: they return zeros without touching memory (codes 0, column scale 0).
+    auto load_stage = [&](int t, bi8_v4i *w, bi8_v4i *a, float *sw, auto checked) {
         const int s = wave + NW * t;
-        if (s < nstages) {                         // wave-uniform
-            const int64_t k0 = (int64_t)s * kStageK;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                w[kb] = __builtin_nontemporal_load((const bi8_v4i *)(wrow + k0 + kb * 64));
-                a[kb] = m_ok ? *(const bi8_v4i *)(arow + k0 + kb * 64) : bi8_v4i{0, 0, 0, 0};
-            }
-#pragma unroll
-            for (int b = 0; b < NBS; ++b) sw[b] = g.sW[((int64_t)s * NBS + b) * g.N + nc];
-        } else {
-#pragma unroll
-            for (int b = 0; b < NBS; ++b) sw[b] = 0.0f;
+        int kill = 0, sc = s;
+        if constexpr (decltype(checked)::value) {
+            kill = s < nstages ? 0 : kBufOut;                       // wave-uniform
+            sc = s < nstages ? s : nstages - 1;
         }
+        const int k0 = sc * kStageK;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            w[kb] = bi8_buffer_load16(rw, voff_w + kill + kb * 64, k0, true);
+            a[kb] = bi8_buffer_load16(ra, voff_a + kill + kb * 64, k0, false);
+        }
+#pragma unroll
+        for (int b = 0; b < NBS; ++b) sw[b] = bi8_buffer_load_f32(rs, voff_s + kill, (sc * NBS + b) * srow);
     };
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const int mine = (nstages - wave + NW - 1) / NW;                // stages of this wave (wave < NW <= nstages not required)
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-        wf[d][0] = wf[d][1] = af[d][0] = af[d][1] = bi8_v4i{0, 0, 0, 0};
-        load_stage(d, wf[d], af[d], swf[d]);
-    }
+    for (int d = 0; d < D; ++d) load_stage(d, wf[d], af[d], swf[d], std::true_type{});
     // the row scales go to LDS while the first stages are on their way
     for (int i = tid; i < nblk * 16; i += 256) {
         const int jb = i >> 4, m = i & 15;
         s_sx[i] = m < g.M ? g.sA[(int64_t)jb * g.M + m] : 0.0f;
     }
     __syncthreads();
-    for (int base = 0; base < mine; base += D) {
+    // D stages from the ring; REFILL 2: every slot is refilled (all of those stages exist), 1: refilled with checked
+    // loads, 0: not refilled (the last group).  Straight-line code in each form: a branch around single loads costs
+    // the register allocator dozens of copies.
+    auto group = [&](int base, auto refill) {
+        constexpr int REFILL = decltype(refill)::value;
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             const int t = base + d;
@@ -1059,7 +1085,8 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
             float swv[NBS];
 #pragma unroll
             for (int b = 0; b < NBS; ++b) swv[b] = swf[d][b];
-            load_stage(t + D, wf[d], af[d], swf[d]);                // refill the slot
+            if constexpr (REFILL == 2) load_stage(t + D, wf[d], af[d], swf[d], std::false_type{});
+            if constexpr (REFILL == 1) load_stage(t + D, wf[d], af[d], swf[d], std::true_type{});
 #pragma unroll
             for (int b = 0; b < NBS; ++b) {
                 const bi8_v4f sx = *(const bi8_v4f *)(s_sx + (sb + b) * 16 + 4 * q);
@@ -1067,7 +1094,14 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
                 for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf((float)p[b][r] * sx[r], swv[b], acc[r]);
             }
         }
+    };
+    int base = 0;
+    for (; base + 2 * D <= mine; base += D) group(base, std::integral_constant<int, 2>{});
+    if (base + D < mine) {
+        group(base, std::integral_constant<int, 1>{});
+        base += D;
     }
+    group(base, std::integral_constant<int, 0>{});
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
     __syncthreads();
@@ -1115,30 +1149,34 @@ __global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const v
     float(*red)[4][64] = (float(*)[4][64])gemv_lds;                 // [wave][register][lane]
     float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][4 rows]
     int8_t *s_a = (int8_t *)(s_sx + (size_t)nblk * 4);               // [M][K], 16-byte aligned
-    const int64_t n = (int64_t)blockIdx.x * 16 + r16;
-    const int64_t nc = n < g.N ? n : g.N - 1;                       // clamped: never stored
-    const int8_t *wrow = g.W + nc * g.ldw + q * 16;
+    const int64_t n0 = (int64_t)blockIdx.x * 16;
+    const int64_t n = n0 + r16;
+    const int64_t wrows = g.N - n0 < 16 ? g.N - n0 : 16;
+    const bi8_brsrc rw = bi8_make_brsrc(g.W + n0 * g.ldw, (wrows - 1) * g.ldw + g.K);   // rows past N read as zeros
+    const bi8_brsrc rs = bi8_make_brsrc(g.sW, (int64_t)nblk * g.N * 4);
+    const int voff_w = r16 * (int)g.ldw + q * 16;
+    const int voff_s = (int)(n < g.N ? n : g.N - 1) * 4;           // clamped: never stored
+    const int srow = (int)g.N * 4;
 
     bi8_v4i wf[D][2];
     float swf[D][NBS];
-    auto load_stage = [&](int t, bi8_v4i *w, float *sw) {
+    // CHECKED loads: a stage past the end of K gets an offset beyond the buffers' ranges and returns zeros without
+    // touching memory
+    auto load_stage = [&](int t, bi8_v4i *w, float *sw, auto checked) {
         const int s = wave + NW * t;
-        if (s < nstages) {                         // wave-uniform
-            const int64_t k0 = (int64_t)s * kStageK;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) w[kb] = __builtin_nontemporal_load((const bi8_v4i *)(wrow + k0 + kb * 64));
-#pragma unroll
-            for (int b = 0; b < NBS; ++b) sw[b] = g.sW[((int64_t)s * NBS + b) * g.N + nc];
-        } else {
-#pragma unroll
-            for (int b = 0; b < NBS; ++b) sw[b] = 0.0f;
+        int kill = 0, sc = s;
+        if constexpr (decltype(checked)::value) {
+            kill = s < nstages ? 0 : kBufOut;                       // wave-uniform
+            sc = s < nstages ? s : nstages - 1;
         }
+        const int k0 = sc * kStageK;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) w[kb] = bi8_buffer_load16(rw, voff_w + kill + kb * 64, k0, true);
+#pragma unroll
+        for (int b = 0; b < NBS; ++b) sw[b] = bi8_buffer_load_f32(rs, voff_s + kill, (sc * NBS + b) * srow);
     };
 #pragma unroll
-    for (int d = 0; d < D; ++d) {
-        wf[d][0] = wf[d][1] = bi8_v4i{0, 0, 0, 0};
-        load_stage(d, wf[d], swf[d]);
-    }
+    for (int d = 0; d < D; ++d) load_stage(d, wf[d], swf[d], std::true_type{});
 
     // x -> codes and scales in LDS.  Chunk c = 16 bytes of x; K % 128 == 0 makes every aligned group of L chunks one
     // K-block of one row, and a group is either all inside x or all past its end.
@@ -1194,23 +1232,23 @@ __global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const v
     __syncthreads();
 
     // the A operands follow the W ring one slot behind its refill: read from LDS a whole ring ahead of their use
-    const bool m_ok = r16 < M;
-    const int8_t *arow = s_a + (m_ok ? r16 : 0) * K + q * 16;
+    // (MFMA lanes of rows >= M read row 0: an output row depends on its own A row only, and those rows are not stored)
+    const int8_t *arow = s_a + (r16 < M ? r16 : 0) * K + q * 16;
     bi8_v4i af[D][2];
     auto read_a = [&](int t, bi8_v4i *a) {
         const int s = wave + NW * t;
         const int sc = s < nstages ? s : nstages - 1;              // stages past the end fold with column scale 0
-        a[0] = a[1] = bi8_v4i{0, 0, 0, 0};
-        if (m_ok) {
-            a[0] = *(const bi8_v4i *)(arow + sc * kStageK);
-            a[1] = *(const bi8_v4i *)(arow + sc * kStageK + 64);
-        }
+        a[0] = *(const bi8_v4i *)(arow + sc * kStageK);
+        a[1] = *(const bi8_v4i *)(arow + sc * kStageK + 64);
     };
 #pragma unroll
     for (int d = 0; d < D; ++d) read_a(d, af[d]);
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const int mine = (nstages - wave + NW - 1) / NW;
-    for (int base = 0; base < mine; base += D) {
+    // D stages from the ring; REFILL 2: every slot refilled (those stages exist), 1: refilled with checked loads,
+    // 0: not refilled (the last group)
+    auto group = [&](int base, auto refill) {
+        constexpr int REFILL = decltype(refill)::value;
 #pragma unroll
         for (int d = 0; d < D; ++d) {
             const int t = base + d;
@@ -1228,8 +1266,9 @@ __global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const v
             float swv[NBS];
 #pragma unroll
             for (int b = 0; b < NBS; ++b) swv[b] = swf[d][b];
-            load_stage(t + D, wf[d], swf[d]);                       // refill the slot
-            read_a(t + D, af[d]);
+            if constexpr (REFILL == 2) load_stage(t + D, wf[d], swf[d], std::false_type{});
+            if constexpr (REFILL == 1) load_stage(t + D, wf[d], swf[d], std::true_type{});
+            if constexpr (REFILL != 0) read_a(t + D, af[d]);
 #pragma unroll
             for (int b = 0; b < NBS; ++b) {
                 const bi8_v4f sx = *(const bi8_v4f *)(s_sx + (sb + b) * 4);
@@ -1237,7 +1276,14 @@ __global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const v
                 for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf((float)p[b][r] * sx[r], swv[b], acc[r]);
             }
         }
+    };
+    int base = 0;
+    for (; base + 2 * D <= mine; base += D) group(base, std::integral_constant<int, 2>{});
+    if (base + D < mine) {
+        group(base, std::integral_constant<int, 1>{});
+        base += D;
     }
+    group(base, std::integral_constant<int, 0>{});
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
     __syncthreads();
@@ -1458,7 +1504,8 @@ extern "C" int bi8_linear_few_rows(const void *x, int dtype, const int8_t *W, co
     if (!x || !W || !sW || !C) return BI8_ERR_NULL_POINTER;
     const int64_t vec = dtype == BI8_F32 ? 4 : 8;
     if (M < 1 || M > kFewRowsMax || N < 1 || (block != 64 && block != 128) || K < kStageK || K % kStageK != 0 || ldx % vec != 0 ||
-        ldw % 16 != 0 || !bi8_aligned(x, 16) || !bi8_aligned(W, 16) || !bi8_aligned(sW, 4) || (N + 15) / 16 > 0x7fffffffLL)
+        ldw % 16 != 0 || ldw >= (1 << 22) || (K / block) * N * 4 >= 0x7fffffffLL || !bi8_aligned(x, 16) || !bi8_aligned(W, 16) ||
+        !bi8_aligned(sW, 4) || (N + 15) / 16 > 0x7fffffffLL)
         return BI8_ERR_UNSUPPORTED;
     const size_t lds = (4 * 4 * 64 + (size_t)(K / block) * 4) * sizeof(float) + (size_t)M * (size_t)K;
     if (lds > kFewRowsLdsMax) return BI8_ERR_UNSUPPORTED;
