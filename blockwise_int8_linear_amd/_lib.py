@@ -25,6 +25,8 @@ SIGNATURES = {
     "bi8_quantize_dual": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_dequantize_rowwise": (_ci, [_vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_gemm_nt_dequant": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
+    "bi8_gemm_nt_dequant_ws": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp, _i64, _vp]),
+    "bi8_gemm_workspace_bytes": (_i64, [_i64, _i64, _i64, _ci]),
     "bi8_gemm_nt_partials": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_linear_few_rows": (_ci, [_vp, _ci, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
 }

@@ -116,6 +116,11 @@ struct GemmArgs {
     int64_t M, N, K, lda, ldw, ldc;
     int tiles_m, tiles_n;
     int bias_dtype;
+    // split of the contraction over gridDim.y workgroups per tile (0 or 1: none): split `y` handles `split_stages`
+    // 128-byte stages of K from y * split_stages on and writes fp32 partial sums to ws[y][M][N]
+    float *ws;
+    int64_t ws_bytes;
+    int splits, split_stages;
 };
 
 __device__ __forceinline__ float load_bias(const GemmArgs &g, int64_t n) {
@@ -140,8 +145,25 @@ template <int BM, int BN, int BLK, int NBUF> struct TileLds {
 
 // BM x BN output tile per workgroup, WM x WN waves (each TM x TN subtiles of 32x32), BLK = quantization block.
 template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
-__global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g) {
+__global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
     using L = TileLds<BM, BN, BLK, NBUF>;
+    GemmArgs g = g_in;
+    if constexpr (!PARTIALS && CDT == BI8_F32) {
+        // One split of K is the same problem on shifted operands: codes from byte k0 of every row, scale rows from
+        // K-block k0 / BLK, fp32 output (scaled, no bias) into this split's slab of the workspace.
+        if (g.splits > 1) {
+            const int64_t k0 = (int64_t)blockIdx.y * g.split_stages * kStageK;
+            const int64_t left = g.K - k0, chunk = (int64_t)g.split_stages * kStageK;
+            g.A += k0;
+            g.W += k0;
+            g.sA += (k0 / BLK) * g.M;
+            g.sW += (k0 / BLK) * g.N;
+            g.K = left < chunk ? left : chunk;
+            g.C = g.ws + (int64_t)blockIdx.y * g.M * g.N;
+            g.ldc = g.N;
+            g.bias = nullptr;
+        }
+    }
     constexpr int kBufs = NBUF;
     constexpr int NW = WM * WN;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -1366,6 +1388,39 @@ __global__ __launch_bounds__(256) void gemm_generic(const GemmArgs g, int block)
     }
 }
 
+// Sum of the split-K slabs, in ascending split order (deterministic), then the cast and the bias of the one-pass
+// epilogue: one output element per thread.
+template <int CDT>
+__global__ __launch_bounds__(256) void splitk_reduce(const GemmArgs g) {
+    const int64_t mn = g.M * g.N;
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= mn) return;
+    float v = g.ws[e];
+    for (int sp = 1; sp < g.splits; ++sp) v += g.ws[sp * mn + e];
+    const int64_t m = e / g.N, n = e % g.N;
+    const bool has_bias = g.bias != nullptr;
+    store_c<CDT>(g.C, m * g.ldc + n, v, has_bias, has_bias ? load_bias(g, n) : 0.0f);
+}
+
+// How many ways to split K for a problem that the tile kernels run on few workgroups, and with which tile
+// (kind 0: 64x128, 1: 128x128): as many splits as fill the 256 CUs once, at least kSplitMinStages stages
+// of K each, at most kSplitMax; 1 = no split.
+constexpr int kSplitMax = 8, kSplitMinStages = 8;   // measured: 4 x 8 stages beat 8 x 4 at K = 4096, 8 x 11 beat 4 x 22 at K = 11008
+static int split_ways(int64_t tiles, int64_t nstages) {
+    if (tiles <= 0 || tiles > 128) return 1;
+    int64_t sp = 256 / tiles;
+    if (sp > kSplitMax) sp = kSplitMax;
+    if (sp > nstages / kSplitMinStages) sp = nstages / kSplitMinStages;
+    return sp < 2 ? 1 : (int)sp;
+}
+static int plan_split(int64_t M, int64_t N, int64_t K, int &kind) {
+    const int64_t nstages = K / kStageK;
+    kind = M > 64 ? 1 : 0;
+    const int64_t tiles = M > 64 ? ((M + 127) / 128) * ((N + 127) / 128) : ((M + 63) / 64) * ((N + 127) / 128);
+    // (splitting the 256x128 tile where the 128x128 tiles are too many to split measured slower than not splitting)
+    return split_ways(tiles, nstages);
+}
+
 template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
 int launch_tile(GemmArgs g, hipStream_t st) {
     constexpr int kLds = TileLds<BM, BN, BLK, NBUF>::kBytes;
@@ -1379,7 +1434,7 @@ int launch_tile(GemmArgs g, hipStream_t st) {
         hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
         if (e != hipSuccess) return bi8_hip_rc(e);
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(WM * WN * 64), kLds, st, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn), (unsigned)(g.splits > 1 ? g.splits : 1)), dim3(WM * WN * 64), kLds, st, g);
     return bi8_launch_rc();
 }
 
@@ -1418,6 +1473,26 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
     }
     // small grids: one workgroup per CU at best, so the tile is spread over as many waves as its shape allows
     // (measured 25-37 % faster than 2x2 waves of 64x64 at M = 96 ... 1024)
+    if constexpr (!PARTIALS) {
+        // few tiles and a caller-provided workspace: split K over several workgroups per tile, then sum the slabs
+        int kind;
+        const int sp = plan_split(g.M, g.N, g.K, kind);
+        if (sp > 1 && g.ws && bi8_aligned(g.ws, 16)) {
+            const int64_t nstages = g.K / kStageK;
+            GemmArgs gs = g;
+            gs.split_stages = (int)((nstages + sp - 1) / sp);
+            gs.splits = (int)((nstages + gs.split_stages - 1) / gs.split_stages);      // every split has work
+            if ((int64_t)gs.splits * g.M * g.N * 4 <= g.ws_bytes && gs.splits > 1) {
+                const int rc = kind == 1 ? launch_tile<128, 128, 4, 2, 3, BLK, BI8_F32, false>(gs, st)
+                                         : launch_tile<64, 128, 2, 2, 3, BLK, BI8_F32, false>(gs, st);
+                if (rc != BI8_OK) return rc;
+                const int64_t blocks = (g.M * g.N + 255) / 256;
+                if (blocks > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+                hipLaunchKernelGGL((splitk_reduce<CDT>), dim3((unsigned)blocks), dim3(256), 0, st, gs);
+                return bi8_launch_rc();
+            }
+        }
+    }
     if (g.M > 64) return launch_tile<128, 128, 4, 2, 3, BLK, CDT, PARTIALS>(g, st);
     return launch_tile<64, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
 }
@@ -1471,21 +1546,38 @@ template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hip
 
 }  // namespace
 
-extern "C" int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float *sA, const float *sW, const void *bias,
-                                   int bias_dtype, void *C, int c_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw,
-                                   int64_t ldc, int block, void *stream) {
+extern "C" int bi8_gemm_nt_dequant_ws(const int8_t *A, const int8_t *W, const float *sA, const float *sW, const void *bias,
+                                      int bias_dtype, void *C, int c_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw,
+                                      int64_t ldc, int block, void *workspace, int64_t workspace_bytes, void *stream) {
     if (c_dtype < 0 || c_dtype > 2 || (bias && (bias_dtype < 0 || bias_dtype > 2))) return BI8_ERR_BAD_DTYPE;
     if (block < 1 || block > (1 << 20)) return BI8_ERR_BAD_BLOCK;
-    if (M < 0 || N < 0 || K < 0 || lda < K || ldw < K || ldc < N) return BI8_ERR_BAD_SHAPE;
+    if (M < 0 || N < 0 || K < 0 || lda < K || ldw < K || ldc < N || workspace_bytes < 0) return BI8_ERR_BAD_SHAPE;
     if (M == 0 || N == 0) return BI8_OK;
     if (!C || (K > 0 && (!A || !W || !sA || !sW))) return BI8_ERR_NULL_POINTER;
-    GemmArgs g{A, W, sA, sW, bias, C, nullptr, M, N, K, lda, ldw, ldc, 0, 0, bias_dtype};
+    GemmArgs g{A, W, sA, sW, bias, C, nullptr, M, N, K, lda, ldw, ldc, 0, 0, bias_dtype, (float *)workspace,
+               workspace ? workspace_bytes : 0, 0, 0};
     hipStream_t st = (hipStream_t)stream;
     switch (c_dtype) {
     case BI8_F32: return dispatch<BI8_F32, false>(g, block, st);
     case BI8_BF16: return dispatch<BI8_BF16, false>(g, block, st);
     default: return dispatch<BI8_F16, false>(g, block, st);
     }
+}
+
+extern "C" int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float *sA, const float *sW, const void *bias,
+                                   int bias_dtype, void *C, int c_dtype, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw,
+                                   int64_t ldc, int block, void *stream) {
+    return bi8_gemm_nt_dequant_ws(A, W, sA, sW, bias, bias_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, block, nullptr, 0, stream);
+}
+
+extern "C" int64_t bi8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int block) {
+    // mirrors dispatch / pick_tile: only the tile kernels on few tiles split K
+    if (M <= 32 || N <= 0 || K <= 0 || K % kStageK != 0 || (block != 32 && block != 64 && block != 128)) return 0;
+    if ((block == 128 || block == 64) && ((M + 255) / 256) * ((N + 255) / 256) >= kWideMinTiles) return 0;
+    if (M > 128 && ((M + 255) / 256) * ((N + 127) / 128) >= 192) return 0;
+    int kind;
+    const int sp = plan_split(M, N, K, kind);
+    return sp > 1 ? (int64_t)sp * M * N * 4 : 0;
 }
 
 template <int DT> int launch_few_rows(const GemmArgs &g, const void *x, int64_t ldx, int block, size_t lds, hipStream_t st) {

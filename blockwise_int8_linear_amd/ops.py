@@ -161,6 +161,7 @@ def _gemm_operands(a: torch.Tensor, b: torch.Tensor):
 
 
 _FAST_BLOCKS = (32, 64, 128)
+_SPLIT_MAX_ROWS = 16384            # 128 = 128 row tiles at most: beyond that no problem has few enough tiles to split
 _PAD_MIN_WORK = 1 << 22            # M*N*K below which the general kernel is as quick as two padded copies
 
 
@@ -205,11 +206,16 @@ def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
             bias = bias.float()
         bias = bias.contiguous()
         bias_ptr, bias_dt = bias.data_ptr(), _DT[bias.dtype]
+    lib = _lib.load()
+    # few output tiles: the library splits K over several workgroups per tile if it is given scratch memory
+    ws_bytes = lib.bi8_gemm_workspace_bytes(M, N, K, block) if 32 < M <= _SPLIT_MAX_ROWS or N <= _SPLIT_MAX_ROWS else 0
+    ws = torch.empty(ws_bytes, device=a.device, dtype=torch.uint8) if ws_bytes else None
     with _on_device(a):
-        rc = _lib.load().bi8_gemm_nt_dequant(a.data_ptr(), w.data_ptr(), state_x.data_ptr(), state_w.data_ptr(),
-                                             bias_ptr, bias_dt, c.data_ptr(), _DT[out_dtype], M, N, K,
-                                             _ld(a), _ld(w), max(N, 1), block, _stream(a))
-    _lib.check(rc, "bi8_gemm_nt_dequant")
+        rc = lib.bi8_gemm_nt_dequant_ws(a.data_ptr(), w.data_ptr(), state_x.data_ptr(), state_w.data_ptr(),
+                                        bias_ptr, bias_dt, c.data_ptr(), _DT[out_dtype], M, N, K,
+                                        _ld(a), _ld(w), max(N, 1), block, ws.data_ptr() if ws is not None else None, ws_bytes,
+                                        _stream(a))
+    _lib.check(rc, "bi8_gemm_nt_dequant_ws")
     return c
 
 

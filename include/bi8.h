@@ -111,6 +111,22 @@ int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float *sA, const
                         int block, void *stream);
 
 /*
+ * bi8_gemm_nt_dequant with a caller-provided scratch buffer.  On problems with few output tiles (a few hundred rows
+ * of activations, or the grad-weight GEMM of a narrow layer) the contraction is split over several workgroups per
+ * tile, which write fp32 partial sums to the workspace; a second kernel adds them in a fixed order, casts and adds
+ * the bias.  (The reference's kernel has the same idea as SPLIT_K with atomic adds, triton_functions.py:121-139; its
+ * launcher always passes SPLIT_K = 1.)  Results agree with bi8_gemm_nt_dequant to fp32 rounding of the sum over
+ * K-blocks.  bi8_gemm_workspace_bytes tells how many bytes the split of a given problem wants (0: it would not
+ * split); a NULL, misaligned (16 bytes) or smaller workspace makes the call identical to bi8_gemm_nt_dequant.
+ * The workspace is only used by the kernels of this call, in stream order.
+ */
+int64_t bi8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int block);
+int bi8_gemm_nt_dequant_ws(const int8_t *A, const int8_t *W, const float *sA, const float *sW,
+                           const void *bias, int bias_dtype, void *C, int c_dtype,
+                           int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                           int block, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
  * The int32 block partial products of the same kernel, before any scaling (what tl.dot yields at
  * triton_functions.py:115):  P int32 [ceil(K/block), M, N], contiguous.  Parity/debug entry point.
  */

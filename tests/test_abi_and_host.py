@@ -21,7 +21,7 @@ def _header_decls():
     text = open(os.path.join(ROOT, "include", "bi8.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     decls = {}
-    for m in re.finditer(r"(?:int|const char \*)\s*(bi8_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+    for m in re.finditer(r"(?:int64_t|int|const char \*)\s*(bi8_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
         args = [a.strip() for a in m.group(2).split(",")] if m.group(2).strip() != "void" else []
         decls[m.group(1)] = args
     return decls
@@ -31,7 +31,8 @@ def test_library_exports_every_declared_symbol():
     decls = _header_decls()
     assert set(decls) == {"bi8_version", "bi8_strerror", "bi8_quantize_rowwise", "bi8_quantize_transposed",
                           "bi8_dequantize_rowwise", "bi8_gemm_nt_dequant", "bi8_gemm_nt_partials",
-                          "bi8_linear_few_rows", "bi8_quantize_dual"}
+                          "bi8_linear_few_rows", "bi8_quantize_dual", "bi8_gemm_nt_dequant_ws",
+                          "bi8_gemm_workspace_bytes"}
     lib = _lib.load()
     for name in decls:
         assert hasattr(lib, name), f"{name} not exported"

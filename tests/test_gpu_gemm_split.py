@@ -1,0 +1,109 @@
+"""bi8_gemm_nt_dequant_ws: the contraction split over several workgroups per tile through a caller-provided workspace.
+Against the CPU checker to the GEMM tolerance, and against the one-pass entry point (same numbers up to the fp32
+rounding of a different summation order)."""
+import ctypes
+
+import pytest
+import torch
+
+from oracle import oracle_torch
+from util import DTYPES
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = {"f32": 1e-3, "bf16": 1e-2, "f16": 1e-2}
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from blockwise_int8_linear_amd import _lib
+    return _lib.load()
+
+
+def _problem(M, N, K, block, seed):
+    g = torch.Generator().manual_seed(seed)
+    A = torch.randint(-127, 128, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+    W = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int32).to(torch.int8)
+    sa = torch.rand(K // block, M, generator=g) * 3 + 0.01
+    sw = torch.rand(K // block, N, generator=g) * 0.1 + 1e-4
+    bias = torch.randn(N, generator=g)
+    return A, W, sa, sw, bias
+
+
+def _run(lib, A, W, sa, sw, bias, block, out, ws_bytes):
+    M, K = A.shape
+    N = W.shape[0]
+    dt = {"f32": 0, "bf16": 1, "f16": 2}[out]
+    C = torch.empty(M, N, device=DEV, dtype=DTYPES[out])
+    ws = torch.empty(max(ws_bytes, 1), device=DEV, dtype=torch.uint8)
+    st = torch.cuda.current_stream().cuda_stream
+    b = bias.to(DEV) if bias is not None else None
+    rc = lib.bi8_gemm_nt_dequant_ws(A.data_ptr(), W.data_ptr(), sa.data_ptr(), sw.data_ptr(), b.data_ptr() if b is not None else None, 0,
+                                    C.data_ptr(), dt, M, N, K, K, K, N, block, ws.data_ptr() if ws_bytes else None, ws_bytes, st)
+    assert rc == 0
+    torch.cuda.synchronize()
+    return C
+
+
+@pytest.mark.parametrize("out", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("M,N,K,block", [(128, 512, 2048, 128), (100, 300, 2048, 64), (48, 700, 2560, 128), (200, 130, 4096, 32),
+                                         (384, 256, 8192, 64), (128, 4096, 4096, 128), (33, 128, 2048, 128)])
+def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
+    A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
+    want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
+    assert want > 0 and want % (M * N * 4) == 0 and 2 <= want // (M * N * 4) <= 8
+    Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
+    split = _run(lib, Ad, Wd, sad, swd, None, block, out, want)
+    one = _run(lib, Ad, Wd, sad, swd, None, block, out, 0)
+    ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw, block, None, DTYPES[out])
+    P = oracle_torch.gemm_nt_partials(A, W, block)
+    mag = torch.zeros(M, N, dtype=torch.float64)
+    for j in range(K // block):
+        mag += P[j].abs().double() * sa[j].double()[:, None] * sw[j].double()[None, :]
+    mag /= 127.0 * 127.0
+    bound = TOL[out] * ref.double().abs() + 4e-6 * mag + 1e-30
+    assert ((split.cpu().double() - ref.double()).abs() <= bound).all()
+    assert ((split.double() - one.double()).abs().cpu() <= 2 * bound).all()        # each is within the bound of the checker
+    # the bias is added after the cast, in the output type (triton_functions.py:127-131): exactly this identity
+    with_bias = _run(lib, Ad, Wd, sad, swd, bias, block, out, want)
+    assert torch.equal(with_bias, split + bias.to(DEV).to(DTYPES[out]))
+
+
+def test_workspace_too_small_or_absent_is_the_one_pass_result(lib):
+    M, N, K, block = 128, 512, 2048, 128
+    A, W, sa, sw, bias = _problem(M, N, K, block, seed=3)
+    Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
+    want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
+    one = _run(lib, Ad, Wd, sad, swd, bias, block, "bf16", 0)
+    small = _run(lib, Ad, Wd, sad, swd, bias, block, "bf16", want - 4)
+    assert torch.equal(one, small)
+    C = torch.empty(M, N, device=DEV, dtype=torch.bfloat16)
+    rc = lib.bi8_gemm_nt_dequant(Ad.data_ptr(), Wd.data_ptr(), sad.data_ptr(), swd.data_ptr(), bias.to(DEV).data_ptr(), 0, C.data_ptr(), 1,
+                                 M, N, K, K, K, N, block, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0 and torch.equal(C, one)
+
+
+def test_no_workspace_wanted_where_nothing_would_split(lib):
+    assert lib.bi8_gemm_workspace_bytes(8192, 8192, 8192, 128) == 0       # plenty of tiles
+    assert lib.bi8_gemm_workspace_bytes(16, 4096, 4096, 128) == 0         # few-row kernels
+    assert lib.bi8_gemm_workspace_bytes(128, 4096, 4100, 128) == 0        # K not a multiple of 128: general kernel
+    assert lib.bi8_gemm_workspace_bytes(128, 4096, 1024, 128) == 0        # eight stages of K: too few to split
+    assert lib.bi8_gemm_workspace_bytes(128, 4096, 4096, 16) == 0         # block size of the general kernel
+
+
+def test_operator_uses_the_split(lib):
+    """through the Python operator (which allocates the workspace): same tolerance, and deterministic from call to call"""
+    import blockwise_int8_linear_amd as pkg
+    M, N, K, block = 128, 1024, 4096, 128
+    A, W, sa, sw, bias = _problem(M, N, K, block, seed=9)
+    cfg = pkg.block_linear_config
+    old = (cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE)
+    cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = block, torch.float32
+    try:
+        c1 = pkg.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa.to(DEV), sw.to(DEV), bias.to(DEV))
+        c2 = pkg.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa.to(DEV), sw.to(DEV), bias.to(DEV))
+    finally:
+        cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = old
+    ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw, block, bias, torch.float32)
+    assert torch.equal(c1, c2)
+    assert torch.allclose(c1.cpu(), ref, rtol=1e-4, atol=1e-4 * ref.abs().max().item())
