@@ -272,8 +272,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
         a_addr[ks] = (L::kAReg + (wm * (BM / WM) + l32) * kStageK + frag_sw) ^ (ks << 5);
         w_addr[ks] = (L::kWReg + (wn * (BN / WN) + l32) * kStageK + frag_sw) ^ (ks << 5);
     }
-    const int sa_addr = L::kSAReg + (wm * (BM / WM) + 4 * h) * 4;
-    const int sw_addr = L::kSWReg + (wn * (BN / WN) + l32) * 4;
+    int sa_addr = L::kSAReg + (wm * (BM / WM) + 4 * h) * 4;
+    int sw_addr = L::kSWReg + (wn * (BN / WN) + l32) * 4;
+    // keep the region offsets inside these ten registers (every access = one of them + an immediate under 64 KiB);
+    // otherwise the compiler folds them into immediates too large for the instruction and keeps an address register
+    // per access
+    asm volatile("" : "+v"(a_addr[0]), "+v"(a_addr[1]), "+v"(a_addr[2]), "+v"(a_addr[3]), "+v"(w_addr[0]), "+v"(w_addr[1]), "+v"(w_addr[2]),
+                 "+v"(w_addr[3]), "+v"(sa_addr), "+v"(sw_addr));
 
     float acc[TM][TN][16];
 #pragma unroll
@@ -681,8 +686,12 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     a_base[1] = a_base[0] ^ 64;
     w_base[1] = w_base[0] ^ 64;
     // a subtile's outputs: lane -> column r16, rows 4q .. 4q+3
-    const int sa_base = L::kSAReg + (wm * 64 + 4 * q) * 4;
-    const int sw_base = L::kSWReg + (wn * 128 + r16) * 4;
+    int sa_base = L::kSAReg + (wm * 64 + 4 * q) * 4;
+    int sw_base = L::kSWReg + (wn * 128 + r16) * 4;
+    // The region offsets (64 KiB and up) stay inside these six registers: every access below is one of them plus an
+    // immediate under 64 KiB.  Left to itself the compiler folds each region offset into the immediates, finds them
+    // too large for the instruction's 16-bit field, and keeps a separate address register per access (24 spilled).
+    asm volatile("" : "+v"(a_base[0]), "+v"(a_base[1]), "+v"(w_base[0]), "+v"(w_base[1]), "+v"(sa_base), "+v"(sw_base));
 
     float acc[4][8][4];
 #pragma unroll
@@ -1467,7 +1476,9 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
     // 256x256 tiles once they fill most of the 256 CUs (measured crossover against the 256x128 tile: ~160 tiles)
     if constexpr ((BLK == 128 || BLK == 64) && !PARTIALS)
         if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= kWideMinTiles) return launch_wide<BLK, CDT>(g, st);
-    if constexpr (kBigFits) {
+    // (block 64: the 256x128 instantiation holds the row scales of both K-blocks of a stage and spills 25 registers;
+    // the 128x128 tile measured 8-10 % faster on every shape below the 256x256 kernel's threshold)
+    if constexpr (kBigFits && (BLK != 64 || PARTIALS)) {
         const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
         if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : 3, BLK, CDT, PARTIALS>(g, st);
     }
