@@ -1504,6 +1504,7 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
             }
         }
     }
+    // (64x128 tiles for problems of 129-255 tiles of 128x128 measured 5-10 % slower than the half-empty 128x128 grid)
     if (g.M > 64) return launch_tile<128, 128, 4, 2, 3, BLK, CDT, PARTIALS>(g, st);
     return launch_tile<64, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
 }

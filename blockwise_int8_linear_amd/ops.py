@@ -161,7 +161,6 @@ def _gemm_operands(a: torch.Tensor, b: torch.Tensor):
 
 
 _FAST_BLOCKS = (32, 64, 128)
-_SPLIT_MAX_ROWS = 16384            # 128 = 128 row tiles at most: beyond that no problem has few enough tiles to split
 _PAD_MIN_WORK = 1 << 22            # M*N*K below which the general kernel is as quick as two padded copies
 
 
@@ -208,7 +207,7 @@ def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
         bias_ptr, bias_dt = bias.data_ptr(), _DT[bias.dtype]
     lib = _lib.load()
     # few output tiles: the library splits K over several workgroups per tile if it is given scratch memory
-    ws_bytes = lib.bi8_gemm_workspace_bytes(M, N, K, block) if 32 < M <= _SPLIT_MAX_ROWS or N <= _SPLIT_MAX_ROWS else 0
+    ws_bytes = lib.bi8_gemm_workspace_bytes(M, N, K, block) if M > 32 else 0
     ws = torch.empty(ws_bytes, device=a.device, dtype=torch.uint8) if ws_bytes else None
     with _on_device(a):
         rc = lib.bi8_gemm_nt_dequant_ws(a.data_ptr(), w.data_ptr(), state_x.data_ptr(), state_w.data_ptr(),

@@ -169,6 +169,35 @@ def test_eval_path_in_a_hip_graph(pkg):
                 assert torch.isfinite(static_y.float()).all()
 
 
+def test_split_of_k_in_a_hip_graph(pkg):
+    """128 rows: the GEMM splits K through a workspace that the operator allocates (inside the capture, from the
+    graph's pool); replays with new inputs equal the eager results bit for bit"""
+    K, N, block, dtype = 4096, 1024, 128, torch.bfloat16
+    torch.manual_seed(8)
+    with cfg_as(pkg, block, dtype):
+        lin = pkg.BlockInt8Linear(K, N, bias=True, device=DEV, dtype=dtype).eval()
+        static_x = torch.zeros(128, K, device=DEV, dtype=dtype)
+        with torch.no_grad():
+            lin(static_x)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    lin(static_x)
+            torch.cuda.current_stream().wait_stream(side)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                static_y = lin(static_x)
+            for i in range(3):
+                x = torch.randn(128, K, device=DEV, dtype=dtype) * (i + 1)
+                eager = lin(x)
+                torch.cuda.synchronize()
+                static_x.copy_(x)
+                graph.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(static_y, eager)
+
+
 def test_reference_benchmark_sweep_and_accuracy_demo(pkg):
     """the sweep of triton_functions.py:521-566 at two small sizes (every provider returns positive rates) and the
     demo scenario of block_linear.py:161-224 (errors of a few percent at most, smaller for smaller blocks)"""
