@@ -19,7 +19,16 @@ constexpr int kThreads = 256;
 constexpr int kPitch = kTC + 1;    // fp32 half-tile pitch: column walks hit distinct banks
 constexpr int kQPitch = kTR + 4;   // code tile pitch in bytes (33 dwords)
 
-template <int DT, int B>
+// 16-byte accesses at addresses that are only aligned to the element (rows of odd length, e.g. the GPT-2 vocabulary
+// 50257): the amdhsa ABI runs with unaligned access enabled, so these are single instructions.
+typedef bi8_v4u bi8_v4u_unaligned __attribute__((aligned(2)));
+typedef bi8_v2u bi8_v2u_unaligned __attribute__((aligned(1)));
+typedef uint32_t bi8_u32_unaligned __attribute__((aligned(1)));
+
+// ALIGNED: rows of x start on 16-byte boundaries and C is a multiple of the elements per 16 bytes, rows of q on 8-byte
+// boundaries.  Otherwise whole 16-byte chunks move with unaligned accesses and the last, partial chunk of a row
+// element by element.
+template <int DT, int B, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == BI8_F32 ? 2 : 3))) void quantize_dual_tile(const void *__restrict__ x, int8_t *__restrict__ q,
                                                                float *__restrict__ scales, int8_t *__restrict__ qT,
                                                                float *__restrict__ scalesT, int64_t R, int64_t C, int64_t ldx,
@@ -49,8 +58,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
         for (int p = 0; p < NP; ++p) {
             const int r = p * RPP + lr;
             raw[p] = bi8_v4u{0u, 0u, 0u, 0u};
-            if (tile < ntiles && r0 + r < R && c0 + cc < C)
-                raw[p] = __builtin_nontemporal_load((const bi8_v4u *)(xb + ((r0 + r) * ldx + c0 + cc) * ES));
+            if (tile < ntiles && r0 + r < R && c0 + cc < C) {
+                const char *src = xb + ((r0 + r) * ldx + c0 + cc) * ES;
+                if constexpr (ALIGNED) {
+                    raw[p] = __builtin_nontemporal_load((const bi8_v4u *)src);
+                } else if (c0 + cc + VEC <= C) {
+                    raw[p] = *(const bi8_v4u_unaligned *)src;
+                } else {                           // the row ends inside this chunk
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        if (c0 + cc + e < C) {
+                            if constexpr (DT == BI8_F32) raw[p][e] = ((const uint32_t *)src)[e];
+                            else raw[p][e >> 1] |= (uint32_t)((const uint16_t *)src)[e] << (16 * (e & 1));
+                        }
+                    }
+                }
+            }
         }
     };
 
@@ -102,11 +125,20 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
                 }
                 if (live) {
                     int8_t *dst = q + row * ldq + col;
-                    if constexpr (VEC == 4) {
-                        __builtin_nontemporal_store(bi8_pack4(code[0], code[1], code[2], code[3]), (uint32_t *)dst);
+                    if (ALIGNED || col + VEC <= C) {
+                        if constexpr (VEC == 4) {
+                            const uint32_t w = bi8_pack4(code[0], code[1], code[2], code[3]);
+                            if constexpr (ALIGNED) __builtin_nontemporal_store(w, (uint32_t *)dst);
+                            else *(bi8_u32_unaligned *)dst = w;
+                        } else {
+                            const bi8_v2u w = {bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
+                            if constexpr (ALIGNED) __builtin_nontemporal_store(w, (bi8_v2u *)dst);
+                            else *(bi8_v2u_unaligned *)dst = w;
+                        }
                     } else {
-                        bi8_v2u w = {bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
-                        __builtin_nontemporal_store(w, (bi8_v2u *)dst);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e)
+                            if (col + e < C) dst[e] = (int8_t)(code[e] & 0xffu);
                     }
                 }
             }
@@ -192,7 +224,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
     }
 }
 
-template <int DT, int B>
+template <int DT, int B, bool ALIGNED>
 int launch_dual(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq,
                 int64_t ldqt, hipStream_t st) {
     const int64_t tiles_c = (C + 2 * kTC - 1) / (2 * kTC);
@@ -200,18 +232,18 @@ int launch_dual(const void *x, int8_t *q, float *scales, int8_t *qT, float *scal
     const int64_t ntiles = tiles_c * tiles_r;
     const int64_t resident = 3 * 256;              // at most three workgroups fit a CU (42 KiB of LDS each)
     const int64_t grid = ntiles < resident ? ntiles : resident;
-    hipLaunchKernelGGL((quantize_dual_tile<DT, B>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT, R, C, ldx, ldq,
-                       ldqt, tiles_c, ntiles);
+    hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT, R, C,
+                       ldx, ldq, ldqt, tiles_c, ntiles);
     return bi8_launch_rc();
 }
 
-template <int DT>
+template <int DT, bool ALIGNED>
 int dispatch(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq,
              int64_t ldqt, int block, hipStream_t st) {
     switch (block) {
-    case 32: return launch_dual<DT, 32>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
-    case 64: return launch_dual<DT, 64>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
-    default: return launch_dual<DT, 128>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
+    case 32: return launch_dual<DT, 32, ALIGNED>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
+    case 64: return launch_dual<DT, 64, ALIGNED>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
+    default: return launch_dual<DT, 128, ALIGNED>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
     }
 }
 
@@ -225,18 +257,27 @@ extern "C" int bi8_quantize_dual(const void *x, int x_dtype, int8_t *q, float *s
     if (R == 0 || C == 0) return BI8_OK;
     if (!x || !q || !scales || !qT || !scalesT) return BI8_ERR_NULL_POINTER;
     const int64_t vec = x_dtype == BI8_F32 ? 4 : 8;
-    const bool one_pass = (block == 32 || block == 64 || block == 128) && C % vec == 0 && ldx % vec == 0 && bi8_aligned(x, 16) &&
-                          ldq % 8 == 0 && bi8_aligned(q, 8) && ldqt % 16 == 0 && bi8_aligned(qT, 16);
+    const int64_t esize = x_dtype == BI8_F32 ? 4 : 2;
+    // one kernel: block 32 / 64 / 128, x aligned to its element type, the transposed codes in 16-byte aligned rows
+    const bool one_pass = (block == 32 || block == 64 || block == 128) && bi8_aligned(x, esize) && ldqt % 16 == 0 && bi8_aligned(qT, 16);
     if (!one_pass) {
-        // other block sizes, odd row lengths, misaligned views: the two single-direction entry points, same results
+        // other block sizes, transposed rows of odd length: the two single-direction entry points, same results
         const int rc = bi8_quantize_rowwise(x, x_dtype, q, scales, R, C, ldx, ldq, block, stream);
         if (rc != BI8_OK) return rc;
         return bi8_quantize_transposed(x, x_dtype, qT, scalesT, R, C, ldx, ldqt, block, stream);
     }
+    const bool aligned = C % vec == 0 && ldx % vec == 0 && bi8_aligned(x, 16) && ldq % 8 == 0 && bi8_aligned(q, 8);
     hipStream_t st = (hipStream_t)stream;
+    if (aligned) {
+        switch (x_dtype) {
+        case BI8_F32: return dispatch<BI8_F32, true>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+        case BI8_BF16: return dispatch<BI8_BF16, true>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+        default: return dispatch<BI8_F16, true>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+        }
+    }
     switch (x_dtype) {
-    case BI8_F32: return dispatch<BI8_F32>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
-    case BI8_BF16: return dispatch<BI8_BF16>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
-    default: return dispatch<BI8_F16>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+    case BI8_F32: return dispatch<BI8_F32, false>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+    case BI8_BF16: return dispatch<BI8_BF16, false>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+    default: return dispatch<BI8_F16, false>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
     }
 }

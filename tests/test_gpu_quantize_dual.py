@@ -57,6 +57,17 @@ def test_dual_cases_the_one_pass_kernel_does_not_take(ops, dtype):
     _check(ops, big[:, 8:8 + 512].contiguous(), 128, x_dev=big.to(DEV)[:, 8:8 + 512])        # aligned view, ld 700
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("block", [64, 128])
+def test_dual_rows_of_odd_length(ops, dtype, block):
+    """rows that are only element-aligned (the GPT-2 vocabulary, 50257, as the row length) with 16-byte aligned
+    transposed rows: one pass with unaligned 16-byte accesses, the last chunk of each row element by element"""
+    for (R, C) in [(256, 50257), (128, 517), (384, 1001), (64, 9), (1024, 131), (272, 4099)]:
+        _check(ops, outlier_tensor(R, C, DTYPES[dtype], seed=R + C + block), block)
+    big = outlier_tensor(130, 700, DTYPES[dtype], seed=11)
+    _check(ops, big[:128, 3:3 + 515].contiguous(), block, x_dev=big.to(DEV)[:128, 3:3 + 515])     # view at an odd element offset
+
+
 def test_dual_special_values(ops):
     x = torch.randn(256, 256, generator=torch.Generator().manual_seed(1))
     x[0, :128] = 0.0                       # zero row block
