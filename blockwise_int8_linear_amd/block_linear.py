@@ -17,7 +17,10 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from . import block_linear_config
 from .ops import (
+    _int8_matmul,
+    _quantize_block_dual,
     dequantize_block_rowwise,
     int8_matmul_block64_rowwise_dequantize,
     linear_few_rows,
@@ -62,11 +65,14 @@ class blockwise_int8_linear(torch.autograd.Function):
             X_int8, state_X = quantize_block_rowwise(X)
             Xt_int8 = Xt_state = None
         if need_gx:
-            W_int8, state_W, Wt_int8, Wt_state = quantize_block_dual(W)         # [N,K] and [K,N], [N/B,K]
+            # [N,K] and [K,N], [N/B,K]; the transposed codes sit in rows padded with zero codes to a multiple of 128
+            # (they are a GEMM operand contracted over N, which may be e.g. a 50257-word vocabulary)
+            W_int8, state_W, Wt_int8, Wt_state, _, Wt_store = _quantize_block_dual(W, block_linear_config.GROUP_SIZE, pad=True)
         else:
             W_int8, state_W = quantize_block_rowwise(W)
-            Wt_int8 = Wt_state = None
-        ctx.save_for_backward(Xt_int8, Xt_state, Wt_int8, Wt_state)
+            Wt_int8 = Wt_state = Wt_store = None
+        ctx.save_for_backward(Xt_int8, Xt_state, Wt_store, Wt_state)
+        ctx.contraction_n = W.shape[0]
         out = int8_matmul_block64_rowwise_dequantize(X_int8, W_int8.t(), state_X, state_W, bias)
         return out.view(*X_3D.size()[:-1], -1)
 
@@ -74,17 +80,20 @@ class blockwise_int8_linear(torch.autograd.Function):
     def backward(ctx, G_3D):
         G = G_3D.reshape(-1, G_3D.size(-1))
         grad_X = grad_W = grad_bias = None
-        Xt_int8, Xt_state, Wt_int8, Wt_state = ctx.saved_tensors
+        Xt_int8, Xt_state, Wt_store, Wt_state = ctx.saved_tensors
         need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        g_store = None
         if need_gx and need_gw:
-            g_int8, g_state, gt_int8, gt_state = quantize_block_dual(G)         # one read of G for both GEMMs
+            # one read of G for both GEMMs; the row codes padded like the transposed W codes they are multiplied with
+            g_int8, g_state, gt_int8, gt_state, g_store, _ = _quantize_block_dual(G, block_linear_config.GROUP_SIZE, pad=True)
         elif need_gx:
             g_int8, g_state = quantize_block_rowwise(G)
         elif need_gw:
             gt_int8, gt_state = quantize_block_transposed(G)                    # [N,M], [M/B,N]
         if need_gx:
             # grad_X [M,K] = G [M,N] @ W [N,K]: contraction over N, W quantized along N
-            grad_X = int8_matmul_block64_rowwise_dequantize(g_int8, Wt_int8.t(), g_state, Wt_state)
+            Wt_int8 = Wt_store[:, :ctx.contraction_n]
+            grad_X = _int8_matmul(g_int8, Wt_int8.t(), g_state, Wt_state, None, g_store, Wt_store)
             grad_X = grad_X.view(*G_3D.size()[:-1], -1)
         if need_gw:
             # grad_W [N,K] = G.T [N,M] @ X [M,K]: contraction over the tokens, both quantized along M

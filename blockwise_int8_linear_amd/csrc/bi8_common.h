@@ -14,6 +14,12 @@ typedef uint32_t bi8_v4u __attribute__((ext_vector_type(4)));
 typedef uint32_t bi8_v2u __attribute__((ext_vector_type(2)));
 typedef float bi8_v4f __attribute__((ext_vector_type(4)));
 
+// Multi-dword accesses at addresses that are only aligned to the element (rows of odd length, e.g. the GPT-2
+// vocabulary 50257): the amdhsa ABI runs with unaligned access enabled, so these are single instructions.
+typedef bi8_v4u bi8_v4u_unaligned __attribute__((aligned(2)));
+typedef bi8_v2u bi8_v2u_unaligned __attribute__((aligned(1)));
+typedef uint32_t bi8_u32_unaligned __attribute__((aligned(1)));
+
 static inline int bi8_hip_rc(hipError_t e) { return e == hipSuccess ? BI8_OK : BI8_ERR_HIP_BASE + (int)e; }
 static inline int bi8_launch_rc() { return bi8_hip_rc(hipGetLastError()); }
 static inline bool bi8_pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }

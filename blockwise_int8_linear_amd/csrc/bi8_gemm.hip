@@ -900,7 +900,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     if constexpr (CDT != BI8_F32) {
         // 16-bit outputs leave through LDS: in the accumulator layout a store instruction would write 32-byte
         // runs of four rows; from a row-major copy of the wave's 64x128 tile it writes 256-byte runs.
-        if (g.ldc % 8 == 0 && ((uintptr_t)g.C & 15) == 0) {
+        {
             __syncthreads();                       // every wave is done with the stage buffers
             uint8_t *tile = lds + wave * (64 * L::kOutPitch);
 #pragma unroll
@@ -927,7 +927,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
                 if (m < g.M) {
                     uint16_t *dst = (uint16_t *)g.C + m * g.ldc + n;
                     if (n + 8 <= g.N) {
-                        *(bi8_v4u *)dst = v;
+                        *(bi8_v4u_unaligned *)dst = v;          // rows of odd length start on 2-byte boundaries
                     } else {
                         for (int e = 0; e < 8 && n + e < g.N; ++e) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
                     }

@@ -19,12 +19,6 @@ constexpr int kThreads = 256;
 constexpr int kPitch = kTC + 1;    // fp32 half-tile pitch: column walks hit distinct banks
 constexpr int kQPitch = kTR + 4;   // code tile pitch in bytes (33 dwords)
 
-// 16-byte accesses at addresses that are only aligned to the element (rows of odd length, e.g. the GPT-2 vocabulary
-// 50257): the amdhsa ABI runs with unaligned access enabled, so these are single instructions.
-typedef bi8_v4u bi8_v4u_unaligned __attribute__((aligned(2)));
-typedef bi8_v2u bi8_v2u_unaligned __attribute__((aligned(1)));
-typedef uint32_t bi8_u32_unaligned __attribute__((aligned(1)));
-
 // ALIGNED: rows of x start on 16-byte boundaries and C is a multiple of the elements per 16 bytes, rows of q on 8-byte
 // boundaries.  Otherwise whole 16-byte chunks move with unaligned accesses and the last, partial chunk of a row
 // element by element.

@@ -111,23 +111,39 @@ def quantize_block_transposed(x: torch.Tensor, fblock_size=None):
     return output, _scales_out(output_maxs)
 
 
+def _code_buffer(rows: int, cols: int, device, pad: bool):
+    """int8 [rows, cols]; with `pad`, a view of a buffer whose rows are padded with zero codes to a multiple of 128
+    (what the tiled GEMM kernels want of a contraction dimension), so that no padded copy is needed later"""
+    if pad and cols % 128 != 0 and rows > 0 and cols > 0:
+        ld = ceil_div(cols, 128) * 128
+        store = torch.empty((rows, ld), device=device, dtype=torch.int8)
+        store[:, cols:].zero_()
+        return store[:, :cols], store
+    t = torch.empty((rows, cols), device=device, dtype=torch.int8)
+    return t, t
+
+
+def _quantize_block_dual(x: torch.Tensor, fblock_size, pad: bool):
+    r, c = x.shape
+    assert x.is_cuda
+    x = _rows(_float_operand(x))
+    pad = pad and fblock_size in _FAST_BLOCKS
+    q, q_store = _code_buffer(r, c, x.device, pad)
+    qt, qt_store = _code_buffer(c, r, x.device, pad)
+    s = torch.empty((ceil_div(c, fblock_size), r), device=x.device, dtype=torch.float32)
+    st = torch.empty((ceil_div(r, fblock_size), c), device=x.device, dtype=torch.float32)
+    with _on_device(x):
+        rc = _lib.load().bi8_quantize_dual(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), qt.data_ptr(), st.data_ptr(),
+                                           r, c, _ld(x), max(q_store.shape[1], 1), max(qt_store.shape[1], 1), fblock_size, _stream(x))
+    _lib.check(rc, "bi8_quantize_dual")
+    return q, _scales_out(s), qt, _scales_out(st), q_store, qt_store
+
+
 def quantize_block_dual(x: torch.Tensor, fblock_size=None):
     """``quantize_block_rowwise(x)`` and ``quantize_block_transposed(x)`` from one pass over x:
     x [R,C] -> (int8 [R,C], scales [ceil(C/B), R], int8 [C,R], scales [ceil(R/B), C]), the same bits as the two calls.
     A training step needs both directions of X, W and G (block_linear.py:77-78, :92-94, :100-103)."""
-    fblock_size = fblock_size or block_linear_config.GROUP_SIZE
-    r, c = x.shape
-    assert x.is_cuda
-    x = _rows(_float_operand(x))
-    q = torch.empty((r, c), device=x.device, dtype=torch.int8)
-    s = torch.empty((ceil_div(c, fblock_size), r), device=x.device, dtype=torch.float32)
-    qt = torch.empty((c, r), device=x.device, dtype=torch.int8)
-    st = torch.empty((ceil_div(r, fblock_size), c), device=x.device, dtype=torch.float32)
-    with _on_device(x):
-        rc = _lib.load().bi8_quantize_dual(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), qt.data_ptr(), st.data_ptr(),
-                                           r, c, _ld(x), max(c, 1), max(r, 1), fblock_size, _stream(x))
-    _lib.check(rc, "bi8_quantize_dual")
-    return q, _scales_out(s), qt, _scales_out(st)
+    return _quantize_block_dual(x, fblock_size or block_linear_config.GROUP_SIZE, pad=False)[:4]
 
 
 def dequantize_block_rowwise(x: torch.Tensor, state_x: torch.Tensor, fblock_size=None):
@@ -164,7 +180,14 @@ _FAST_BLOCKS = (32, 64, 128)
 _PAD_MIN_WORK = 1 << 22            # M*N*K below which the general kernel is as quick as two padded copies
 
 
-def _pad_contraction(a, w, state_x, state_w, block):
+def _zero_padded(t, store):
+    """`store` if it is t's buffer with rows padded with zero codes (see _code_buffer), else None"""
+    if store is None or store is t or store.shape[0] != t.shape[0] or store.data_ptr() != t.data_ptr():
+        return None
+    return store
+
+
+def _pad_contraction(a, w, state_x, state_w, block, a_store=None, w_store=None):
     """The tiled GEMM kernels want K to be a multiple of 128 and 16-byte aligned operand rows; a contraction like
     the GPT-2 vocabulary (50257, the grad-input GEMM of the output layer) would fall to the general kernel, which is
     ~40x slower.  Zero codes add nothing to any block partial, so such operands are copied once into buffers
@@ -176,8 +199,9 @@ def _pad_contraction(a, w, state_x, state_w, block):
     if not ragged or block not in _FAST_BLOCKS or K == 0 or M * N * K < _PAD_MIN_WORK:
         return a, w, state_x, state_w, K
     k_pad = ceil_div(K, 128) * 128
-    a = torch.nn.functional.pad(a, (0, k_pad - K))
-    w = torch.nn.functional.pad(w, (0, k_pad - K))
+    a_store, w_store = _zero_padded(a, a_store), _zero_padded(w, w_store)
+    a = a_store if a_store is not None and a_store.shape[1] == k_pad else torch.nn.functional.pad(a, (0, k_pad - K))
+    w = w_store if w_store is not None and w_store.shape[1] == k_pad else torch.nn.functional.pad(w, (0, k_pad - K))
     extra = k_pad // block - state_x.shape[0]
     if extra > 0:
         state_x = torch.nn.functional.pad(state_x, (0, 0, 0, extra))
@@ -188,6 +212,11 @@ def _pad_contraction(a, w, state_x, state_w, block):
 def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
     """a int8 [M,K], b int8 [K,N] (any strides), state_x [K/B, M], state_w [K/B, N], bias [N] or None
     -> [M,N] of INPUT_OUTPUT_TORCH_TYPE; triton_functions.py:142-168.  B = GROUP_SIZE at call time."""
+    return _int8_matmul(a, b, state_x, state_w, bias)
+
+
+def _int8_matmul(a, b, state_x, state_w, bias=None, a_store=None, w_store=None):
+    """the launcher; a_store / w_store: the zero-padded buffers that a and b.t() are views of, if any"""
     block = block_linear_config.GROUP_SIZE
     out_dtype = block_linear_config.INPUT_OUTPUT_TORCH_TYPE
     a, w = _gemm_operands(a, b)
@@ -196,7 +225,7 @@ def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
     nblk = ceil_div(K, block)
     assert tuple(state_x.shape) == (nblk, M) and tuple(state_w.shape) == (nblk, N), "scale shapes must be [ceil(K/block), rows]"
     state_x, state_w = _scales_in(state_x), _scales_in(state_w)
-    a, w, state_x, state_w, K = _pad_contraction(a, w, state_x, state_w, block)
+    a, w, state_x, state_w, K = _pad_contraction(a, w, state_x, state_w, block, a_store, w_store)
     c = torch.empty((M, N), device=a.device, dtype=out_dtype)
     bias_ptr, bias_dt = None, 0
     if bias is not None:
