@@ -359,13 +359,27 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) wf[b][ks] = *(const bi8_v4i *)(lds + (w_addr[ks] + ow) + b * 32 * kStageK);
         };
-        load_a(0);
-        load_w(0);
-        if constexpr (PARTIALS || NBS > 1) {       // these variants keep the simple order: everything up front
+        // K-block blk of every row / column subtile (blocks shorter than the stage: their operands are read one
+        // block at a time, during the last subtile of the block before, so a stage's operands are never all live)
+        auto load_block = [&](int blk) {
 #pragma unroll
-            for (int b = 1; b < TN; ++b) load_w(b);
+            for (int ks = blk * KSB; ks < (blk + 1) * KSB; ++ks) {
 #pragma unroll
-            for (int a = 1; a < TM; ++a) load_a(a);
+                for (int b = 0; b < TN; ++b) wf[b][ks] = *(const bi8_v4i *)(lds + (w_addr[ks] + ow) + b * 32 * kStageK);
+#pragma unroll
+                for (int a = 0; a < TM; ++a) af[a][ks] = *(const bi8_v4i *)(lds + (a_addr[ks] + oa) + a * 32 * kStageK);
+            }
+        };
+        if constexpr (PARTIALS) {                  // the simple order: everything up front
+#pragma unroll
+            for (int b = 0; b < TN; ++b) load_w(b);
+#pragma unroll
+            for (int a = 0; a < TM; ++a) load_a(a);
+        } else if constexpr (NBS > 1) {
+            load_block(0);
+        } else {
+            load_a(0);
+            load_w(0);
         }
 
         if constexpr (PARTIALS) {
@@ -398,6 +412,11 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
                     if (a == 0 && b + 1 < TN) load_w(b + 1);
                     if (b == TN - 1 && a + 1 < TM) load_a(a + 1);
                     __builtin_amdgcn_sched_barrier(0);
+                } else {
+                    if (t % NSUB == NSUB - 1 && blk + 1 < NBS) {
+                        load_block(blk + 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
 #pragma unroll
                 for (int ks = 0; ks < KSB; ++ks) {
@@ -1476,9 +1495,7 @@ template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipS
     // 256x256 tiles once they fill most of the 256 CUs (measured crossover against the 256x128 tile: ~160 tiles)
     if constexpr ((BLK == 128 || BLK == 64) && !PARTIALS)
         if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= kWideMinTiles) return launch_wide<BLK, CDT>(g, st);
-    // (block 64: the 256x128 instantiation holds the row scales of both K-blocks of a stage and spills 25 registers;
-    // the 128x128 tile measured 8-10 % faster on every shape below the 256x256 kernel's threshold)
-    if constexpr (kBigFits && (BLK != 64 || PARTIALS)) {
+    if constexpr (kBigFits) {
         const int64_t big = ((g.M + 255) / 256) * ((g.N + 127) / 128);
         if (g.M > 128 && big >= 192) return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : 3, BLK, CDT, PARTIALS>(g, st);
     }
