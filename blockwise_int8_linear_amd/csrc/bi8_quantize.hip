@@ -15,7 +15,10 @@ constexpr int kRows = 4 * kRowsPerWave;    // rows per workgroup tile
 constexpr int kChunks = 1;                 // 1 KiB wave-loads per row per tile (2 and 4 measured slower)
 constexpr int kThreads = 256;
 
-template <int DT, int L>
+// ALIGNED: rows of x on 16-byte boundaries, K a multiple of the elements per 16 bytes, rows of q aligned to their
+// 4- or 8-byte stores.  Otherwise (odd row length or leading dimension, e.g. the GPT-2 vocabulary 50257) whole chunks
+// move with unaligned 16-byte loads and 4- or 8-byte stores, the last, partial chunk of a row element by element.
+template <int DT, int L, bool ALIGNED>
 __global__ __launch_bounds__(kThreads) void quantize_rows_vec(const void *__restrict__ x, int8_t *__restrict__ q,
                                                               float *__restrict__ scales, int64_t M, int64_t K,
                                                               int64_t ldx, int64_t ldq, int64_t nblk, int tiles_k) {
@@ -44,8 +47,22 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_vec(const void *__rest
         for (int c = 0; c < kChunks; ++c) {
             const int64_t col = col0 + (c * BI8_WAVE + lane) * VEC;
             bi8_v4u v = {0u, 0u, 0u, 0u};
-            if (row < M && col < K)
-                v = __builtin_nontemporal_load((const bi8_v4u *)(xb + (row * ldx + col) * ES));
+            if (row < M && col < K) {
+                const char *src = xb + (row * ldx + col) * ES;
+                if constexpr (ALIGNED) {
+                    v = __builtin_nontemporal_load((const bi8_v4u *)src);
+                } else if (col + VEC <= K) {
+                    v = *(const bi8_v4u_unaligned *)src;
+                } else {                           // the row ends inside this chunk
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        if (col + e < K) {
+                            if constexpr (DT == BI8_F32) v[e] = ((const uint32_t *)src)[e];
+                            else v[e >> 1] |= (uint32_t)((const uint16_t *)src)[e] << (16 * (e & 1));
+                        }
+                    }
+                }
+            }
             raw[i][c] = v;
         }
     }
@@ -80,11 +97,20 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_vec(const void *__rest
             }
             if (row < M && col < K) {
                 int8_t *dst = q + row * ldq + col;
-                if constexpr (VEC == 4) {
-                    __builtin_nontemporal_store(bi8_pack4(code[0], code[1], code[2], code[3]), (uint32_t *)dst);
+                if (ALIGNED || col + VEC <= K) {
+                    if constexpr (VEC == 4) {
+                        const uint32_t w = bi8_pack4(code[0], code[1], code[2], code[3]);
+                        if constexpr (ALIGNED) __builtin_nontemporal_store(w, (uint32_t *)dst);
+                        else *(bi8_u32_unaligned *)dst = w;
+                    } else {
+                        const bi8_v2u w = {bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
+                        if constexpr (ALIGNED) __builtin_nontemporal_store(w, (bi8_v2u *)dst);
+                        else *(bi8_v2u_unaligned *)dst = w;
+                    }
                 } else {
-                    bi8_v2u w = {bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
-                    __builtin_nontemporal_store(w, (bi8_v2u *)dst);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        if (col + e < K) dst[e] = (int8_t)(code[e] & 0xffu);
                 }
             }
         }
@@ -122,58 +148,7 @@ __global__ __launch_bounds__(kThreads) void quantize_rows_generic(const void *__
     }
 }
 
-// Rows that are not 16-byte aligned (odd row length or leading dimension, e.g. 50257), blocks 32 / 64 / 128: one
-// wave per 512 consecutive elements of a row, lane l holds elements 64k + l (k = 0..7), so every load instruction
-// reads 64 consecutive elements and every store 64 consecutive code bytes; a K-block is 32 or 64 adjacent lanes
-// of one k, or (B = 128) the whole wave over two k.
-template <int DT, int B>
-__global__ __launch_bounds__(kThreads) void quantize_rows_loose(const void *__restrict__ x, int8_t *__restrict__ q,
-                                                                float *__restrict__ scales, int64_t M, int64_t K, int64_t ldx,
-                                                                int64_t ldq, int64_t chunks_per_row) {
-    constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
-    constexpr int U = 8;
-    const int lane = threadIdx.x & 63;
-    const int64_t unit = (int64_t)blockIdx.x * (kThreads / 64) + (threadIdx.x >> 6);
-    const int64_t row = unit / chunks_per_row;
-    if (row >= M) return;
-    const int64_t k0 = (unit % chunks_per_row) * (64 * U);
-    float v[U], m[U];
-#pragma unroll
-    for (int k = 0; k < U; ++k) {
-        const int64_t idx = k0 + 64 * k + lane;
-        v[k] = idx < K ? bi8_load_elem<DT>(x, row * ldx + idx) : 0.0f;
-        m[k] = __builtin_fmaxf(0.0f, __builtin_fabsf(v[k]));        // ignores NaN
-    }
-#pragma unroll
-    for (int k = 0; k < U; ++k) {
-        if constexpr (B == 128) {
-            if ((k & 1) == 0) m[k] = m[k + 1] = bi8_group_max<64>(__builtin_fmaxf(m[k], m[k + 1]));
-        } else {
-            m[k] = bi8_group_max<B>(m[k]);
-        }
-    }
-#pragma unroll
-    for (int k = 0; k < U; ++k) {
-        const int64_t idx = k0 + 64 * k + lane;
-        if (idx < K) {
-            const bool special = (v[k] != v[k]) || !bi8_scale_is_ordinary(m[k]);
-            const uint32_t code = special ? bi8_code_slow(v[k], m[k]) : bi8_code_fast<NCORR>(v[k], m[k], 1.0f / m[k]);
-            q[row * ldq + idx] = (int8_t)(code & 0xffu);
-            if (idx % B == 0) scales[(idx / B) * M + row] = m[k];
-        }
-    }
-}
-
-template <int DT, int B>
-int launch_loose(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int64_t ldx, int64_t ldq, hipStream_t st) {
-    const int64_t chunks = (K + 511) / 512;
-    const int64_t grid = (M * chunks + 3) / 4;
-    if (grid > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-    hipLaunchKernelGGL((quantize_rows_loose<DT, B>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, M, K, ldx, ldq, chunks);
-    return bi8_launch_rc();
-}
-
-template <int DT, int L>
+template <int DT, int L, bool ALIGNED>
 int launch_vec(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int64_t ldx, int64_t ldq, hipStream_t st) {
     constexpr int VEC = Bi8Vec<DT>::kElems;
     constexpr int B = L * VEC;
@@ -182,31 +157,33 @@ int launch_vec(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, in
     const int64_t tiles_m = (M + kRows - 1) / kRows;
     if (tiles_k * tiles_m > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     const int64_t nblk = (K + B - 1) / B;
-    hipLaunchKernelGGL((quantize_rows_vec<DT, L>), dim3((unsigned)(tiles_k * tiles_m)), dim3(kThreads), 0, st, x, q, scales, M, K,
+    hipLaunchKernelGGL((quantize_rows_vec<DT, L, ALIGNED>), dim3((unsigned)(tiles_k * tiles_m)), dim3(kThreads), 0, st, x, q, scales, M, K,
                        ldx, ldq, nblk, (int)tiles_k);
     return bi8_launch_rc();
+}
+
+template <int DT, bool ALIGNED>
+int dispatch_vec(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int64_t ldx, int64_t ldq, int lanes, hipStream_t st) {
+    switch (lanes) {
+    case 1: return launch_vec<DT, 1, ALIGNED>(x, q, scales, M, K, ldx, ldq, st);
+    case 2: return launch_vec<DT, 2, ALIGNED>(x, q, scales, M, K, ldx, ldq, st);
+    case 4: return launch_vec<DT, 4, ALIGNED>(x, q, scales, M, K, ldx, ldq, st);
+    case 8: return launch_vec<DT, 8, ALIGNED>(x, q, scales, M, K, ldx, ldq, st);
+    case 16: return launch_vec<DT, 16, ALIGNED>(x, q, scales, M, K, ldx, ldq, st);
+    case 32: return launch_vec<DT, 32, ALIGNED>(x, q, scales, M, K, ldx, ldq, st);
+    default: return launch_vec<DT, 64, ALIGNED>(x, q, scales, M, K, ldx, ldq, st);
+    }
 }
 
 template <int DT>
 int dispatch(const void *x, int8_t *q, float *scales, int64_t M, int64_t K, int64_t ldx, int64_t ldq, int block, hipStream_t st) {
     constexpr int VEC = Bi8Vec<DT>::kElems;
-    const bool vec_ok = bi8_pow2(block) && block >= VEC && block <= 64 * VEC && K % VEC == 0 && ldx % VEC == 0 &&
-                        ldq % VEC == 0 && bi8_aligned(x, 16) && bi8_aligned(q, VEC);
+    // one K-block = 1 .. 64 lanes of 16 input bytes each
+    const bool vec_ok = bi8_pow2(block) && block >= VEC && block <= 64 * VEC && bi8_aligned(x, 16 / VEC);
     if (vec_ok) {
-        switch (block / VEC) {
-        case 1: return launch_vec<DT, 1>(x, q, scales, M, K, ldx, ldq, st);
-        case 2: return launch_vec<DT, 2>(x, q, scales, M, K, ldx, ldq, st);
-        case 4: return launch_vec<DT, 4>(x, q, scales, M, K, ldx, ldq, st);
-        case 8: return launch_vec<DT, 8>(x, q, scales, M, K, ldx, ldq, st);
-        case 16: return launch_vec<DT, 16>(x, q, scales, M, K, ldx, ldq, st);
-        case 32: return launch_vec<DT, 32>(x, q, scales, M, K, ldx, ldq, st);
-        case 64: return launch_vec<DT, 64>(x, q, scales, M, K, ldx, ldq, st);
-        }
-    }
-    switch (block) {
-    case 32: return launch_loose<DT, 32>(x, q, scales, M, K, ldx, ldq, st);
-    case 64: return launch_loose<DT, 64>(x, q, scales, M, K, ldx, ldq, st);
-    case 128: return launch_loose<DT, 128>(x, q, scales, M, K, ldx, ldq, st);
+        const bool aligned = K % VEC == 0 && ldx % VEC == 0 && ldq % VEC == 0 && bi8_aligned(x, 16) && bi8_aligned(q, VEC);
+        return aligned ? dispatch_vec<DT, true>(x, q, scales, M, K, ldx, ldq, block / VEC, st)
+                       : dispatch_vec<DT, false>(x, q, scales, M, K, ldx, ldq, block / VEC, st);
     }
     const int64_t nblk = (K + block - 1) / block;
     const int64_t units = M * nblk;

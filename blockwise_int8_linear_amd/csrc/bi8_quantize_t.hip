@@ -16,9 +16,10 @@ constexpr int kPitch = kTC + 1;    // fp32 tile pitch: column walks hit distinct
 constexpr int kQPitch = kTR + 4;   // code tile pitch in bytes (33 dwords)
 
 // B in {32, 64, 128}: thread (c = tid % 64, g = tid / 64) owns source rows 32g .. 32g+31 of column c.
-// VLOAD / VSTORE: the source rows / the output rows are 16-byte aligned, so a lane moves 16 bytes at a time; without
-// them the same tile is read element by element (64 consecutive elements per wave instruction) and written byte by
-// byte (64 consecutive bytes per wave instruction): odd leading dimensions such as the GPT-2 vocabulary, 50257.
+// VLOAD: the source rows are 16-byte aligned and C is a multiple of the elements per 16 bytes; without it whole
+// chunks are read with unaligned 16-byte loads and the last, partial chunk of a row element by element.  VSTORE: the
+// output rows are 16-byte aligned, so a lane stores 16 codes at a time; without it the code tile is written byte by
+// byte (64 consecutive bytes per wave instruction).  Odd leading dimensions such as the GPT-2 vocabulary, 50257.
 template <int DT, int B, bool VLOAD, bool VSTORE>
 __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__restrict__ x, int8_t *__restrict__ qT,
                                                                float *__restrict__ scalesT, int64_t R, int64_t C,
@@ -35,34 +36,34 @@ __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__res
 
     const int tid = threadIdx.x;
     const char *xb = (const char *)x;
-    constexpr int NP = VLOAD ? kTR / RPP : (kTR * kTC) / kThreads / 4;   // 16-byte loads (or groups of 4 elements) per thread per tile
+    constexpr int NP = kTR / RPP;                  // 16-byte loads per thread per tile
 
     // A workgroup walks tiles blockIdx.x, blockIdx.x + gridDim.x, ...; the loads of the next tile are issued before
     // the current one is processed, so every workgroup has global loads in flight all the time.
     auto load_tile = [&](int64_t tile, bi8_v4u *raw) {
         const int64_t r0 = (tile / tiles_c) * kTR;
         const int64_t c0 = (tile % tiles_c) * kTC;
-        if constexpr (VLOAD) {
 #pragma unroll
-            for (int p = 0; p < NP; ++p) {
-                const int r = p * RPP + tid / LPR;
-                const int cc = (tid % LPR) * VEC;
-                raw[p] = bi8_v4u{0u, 0u, 0u, 0u};
-                if (tile < ntiles && r0 + r < R && c0 + cc < C)
-                    raw[p] = __builtin_nontemporal_load((const bi8_v4u *)(xb + ((r0 + r) * ldx + c0 + cc) * ES));
-            }
-        } else {
-            // element e = tid + 256 * k of the tile in row-major order, as fp32 bits: raw[p][i] is k = 4p + i
+        for (int p = 0; p < NP; ++p) {
+            const int r = p * RPP + tid / LPR;
+            const int cc = (tid % LPR) * VEC;
+            raw[p] = bi8_v4u{0u, 0u, 0u, 0u};
+            if (tile < ntiles && r0 + r < R && c0 + cc < C) {
+                const char *src = xb + ((r0 + r) * ldx + c0 + cc) * ES;
+                if constexpr (VLOAD) {
+                    raw[p] = __builtin_nontemporal_load((const bi8_v4u *)src);
+                } else if (c0 + cc + VEC <= C) {
+                    raw[p] = *(const bi8_v4u_unaligned *)src;
+                } else {                           // the row ends inside this chunk
 #pragma unroll
-            for (int p = 0; p < NP; ++p)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int e = tid + kThreads * (4 * p + i);
-                    const int r = e / kTC, cc = e % kTC;
-                    float f = 0.0f;
-                    if (tile < ntiles && r0 + r < R && c0 + cc < C) f = bi8_load_elem<DT>(x, (r0 + r) * ldx + c0 + cc);
-                    raw[p][i] = bi8_f2u(f);
+                    for (int e = 0; e < VEC; ++e) {
+                        if (c0 + cc + e < C) {
+                            if constexpr (DT == BI8_F32) raw[p][e] = ((const uint32_t *)src)[e];
+                            else raw[p][e >> 1] |= (uint32_t)((const uint16_t *)src)[e] << (16 * (e & 1));
+                        }
+                    }
                 }
+            }
         }
     };
     bi8_v4u raw[NP];
@@ -72,24 +73,14 @@ __global__ __launch_bounds__(kThreads) void quantize_cols_tile(const void *__res
         const int64_t c0 = (tile % tiles_c) * kTC;
 
         // phase 1: rows of the tile -> fp32 in LDS; then start the next tile's loads
-        if constexpr (VLOAD) {
 #pragma unroll
-            for (int p = 0; p < NP; ++p) {
-                const int r = p * RPP + tid / LPR;
-                const int cc = (tid % LPR) * VEC;
-                float f[VEC];
-                bi8_unpack<DT>(raw[p], f);
+        for (int p = 0; p < NP; ++p) {
+            const int r = p * RPP + tid / LPR;
+            const int cc = (tid % LPR) * VEC;
+            float f[VEC];
+            bi8_unpack<DT>(raw[p], f);
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) s_x[r * kPitch + cc + e] = f[e];
-            }
-        } else {
-#pragma unroll
-            for (int p = 0; p < NP; ++p)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int e = tid + kThreads * (4 * p + i);
-                    s_x[(e / kTC) * kPitch + e % kTC] = bi8_u2f(raw[p][i]);
-                }
+            for (int e = 0; e < VEC; ++e) s_x[r * kPitch + cc + e] = f[e];
         }
         load_tile(tile + gridDim.x, raw);
         __syncthreads();
