@@ -1493,6 +1493,7 @@ constexpr int64_t kWideMinTiles = 160;
 template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipStream_t st) {
     constexpr bool kBigFits = TileLds<256, 128, BLK, 3>::kFits;
     // 256x256 tiles once they fill most of the 256 CUs (measured crossover against the 256x128 tile: ~160 tiles)
+    // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
     if constexpr ((BLK == 128 || BLK == 64) && !PARTIALS)
         if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= kWideMinTiles) return launch_wide<BLK, CDT>(g, st);
     if constexpr (kBigFits) {
