@@ -39,7 +39,7 @@ def test_gemm_random(ops, seed):
     out = rng.choice(["f32", "bf16", "f16"])
     M = rng.choice([rng.randint(1, 40), _pick_dim(rng, 1, 700)])
     N = _pick_dim(rng, 1, 700)
-    K = rng.choice([128 * rng.randint(1, 12), _pick_dim(rng, 1, 1500)])
+    K = rng.choice([128 * rng.randint(1, 12), 128 * rng.randint(16, 40), _pick_dim(rng, 1, 1500)])     # long K: split over workgroups
     pad_a, pad_w = rng.choice([0, 0, 16, 5]), rng.choice([0, 0, 32, 3])
     g = torch.Generator().manual_seed(seed)
     A = torch.randint(-127, 128, (M, K + pad_a), generator=g, dtype=torch.int32).to(torch.int8)
@@ -89,6 +89,9 @@ def test_quantize_dequantize_random(ops, seed):
     qt, st = ops.quantize_block_transposed(xd, block)
     qto, sto = oracle.quantize_block_transposed(xc, block, threads=True)
     assert torch.equal(st.cpu().view(torch.int32), sto.view(torch.int32)) and torch.equal(qt.cpu(), qto), (M, K, pad, block, dtype)
+    q2, s2, qt2, st2 = ops.quantize_block_dual(xd, block)               # both directions from one read: the same bits
+    assert torch.equal(q2, q) and torch.equal(qt2, qt), (M, K, pad, block, dtype)
+    assert torch.equal(s2.view(torch.int32), s.view(torch.int32)) and torch.equal(st2.view(torch.int32), st.view(torch.int32))
     cfg = ops.block_linear_config
     old = cfg.INPUT_OUTPUT_TORCH_TYPE
     cfg.INPUT_OUTPUT_TORCH_TYPE = DTYPES[dtype]
@@ -135,3 +138,31 @@ def test_gemm_random_large(ops, seed):
     err = (C.cpu().double() - ref.double()).abs()
     bound = TOL[out] * ref.double().abs() + 4e-6 * mag + 1e-30
     assert (err <= bound).all(), f"M={M} N={N} K={K} block={block} out={out}: max excess {(err - bound).max().item():.3e}"
+
+
+@pytest.mark.parametrize("seed", range(N_CASES // 2))
+def test_few_rows_random(ops, seed):
+    """the one-kernel eval path (quantize + GEMM) against the two launchers, 1..4 rows, random K, N, block and type"""
+    rng = random.Random(4000 + seed)
+    block = rng.choice([64, 128])
+    dtype = rng.choice(["f32", "bf16", "f16"])
+    M, K, N = rng.randint(1, 4), 128 * rng.randint(1, 48), _pick_dim(rng, 1, 3000)
+    cfg = ops.block_linear_config
+    old = (cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE)
+    cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = block, DTYPES[dtype]
+    try:
+        g = torch.Generator().manual_seed(seed)
+        w = (torch.randn(N, K, generator=g) * 0.02).to(DTYPES[dtype]).to(DEV)
+        x = outlier_tensor(M, K, DTYPES[dtype], seed=seed).to(DEV)
+        bias = torch.randn(N, generator=g).to(DTYPES[dtype]).to(DEV) if rng.random() < 0.5 else None
+        Wq, Ws = ops.quantize_block_rowwise(w)
+        xq, xs = ops.quantize_block_rowwise(x)
+        two = ops.int8_matmul_block64_rowwise_dequantize(xq, Wq.t(), xs, Ws, bias)
+        one = ops.linear_few_rows(x, Wq, Ws, bias)
+    finally:
+        cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = old
+    if one is None:
+        assert 4096 + 16 * (K // block) + M * K > 65536, (M, K, N, block, dtype)
+    else:
+        view = torch.int32 if dtype == "f32" else torch.int16
+        assert torch.equal(one.view(view), two.view(view)), (M, K, N, block, dtype)
