@@ -723,10 +723,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     constexpr int kMagicBits = 0x4B400000;        // bit pattern of 1.5 * 2^23
     const bi8_v4i magic = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
     bi8_v4i A[4][2], Bf[2][2];                     // [row subtile][kb], [column parity][kb]
-    bi8_v4i c[2][2];                               // int32 partials: [pair parity][row subtile of the pair]
     bi8_v4f sx[4];                                 // row scales per row subtile
     float swb[2] = {0.0f, 0.0f}, swc[2] = {0.0f, 0.0f}, swr[2] = {0.0f, 0.0f};   // per column parity: b, -(1.5*2^23)*b, raw
-    c[0][0] = c[0][1] = c[1][0] = c[1][1] = magic;  // "partial 0" for the fold that precedes the first pair
 #pragma unroll
     for (int i = 0; i < 4; ++i) sx[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -749,79 +747,68 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             dst[r] = __builtin_fmaf(u, s[r], dst[r]);
         }
     };
-    // one pair = row subtiles (a0, a1) of one column: four MFMAs, each followed by a quarter of the previous pair's fold
-    auto pair = [&](bi8_v4i *cn, const bi8_v4i *a0, const bi8_v4i *a1, const bi8_v4i *b, const bi8_v4i *cp, const bi8_v4f &s0,
-                    const bi8_v4f &s1, float fb, float fc, float *d0, float *d1) {
-        cn[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b[0], magic, 0, 0, 0);
-        fold2(cp[0], 0, s0, fb, fc, d0);
-        __builtin_amdgcn_sched_barrier(0);
-        cn[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[0], b[0], magic, 0, 0, 0);
-        fold2(cp[0], 2, s0, fb, fc, d0);
-        __builtin_amdgcn_sched_barrier(0);
-        cn[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b[1], cn[0], 0, 0, 0);
-        fold2(cp[1], 0, s1, fb, fc, d1);
-        __builtin_amdgcn_sched_barrier(0);
-        cn[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[1], b[1], cn[1], 0, 0, 0);
-        fold2(cp[1], 2, s1, fb, fc, d1);
-        __builtin_amdgcn_sched_barrier(0);
-    };
     auto wait_vm = [&](auto pending_c) {
         constexpr int kPending = decltype(pending_c)::value;
         __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
     };
 
-    // On entry to a stage (buffer F): A[0], A[1], Bf[0], swr[0] already hold this stage's row subtiles 0, 1 and
-    // column 0 (read during the previous stage's last column); c[1] is the previous stage's last pair (rows 2, 3
-    // of column 7), still to be folded with the OLD sx[2], sx[3], swb[1], swc[1].
+    // Column-burst schedule (BLK = 128): the eight MFMAs of column j back to back, then the whole fold of column
+    // j - 1 (32 FMAs).  cB[parity][row subtile] are the partials; on entry A[0..3], Bf[0], swr[0] hold this stage's
+    // operands of column 0 and cB[1] the previous stage's column 7, still to be folded with the OLD sx, swb[1], swc[1].
+    bi8_v4i cB[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) cB[0][i] = cB[1][i] = magic;
     auto stage = [&](auto buf_c) {                  // BLK = 128
         constexpr int F = decltype(buf_c)::value, G = 1 - F;
-        read_a(A[2], 2, F);
-        read_a(A[3], 3, F);
-        read_sx(sx[0], 0, F);
-        read_sx(sx[1], 1, F);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             constexpr int kPrevCol[8] = {7, 0, 1, 2, 3, 4, 5, 6};
             const int jb = j & 1;
-            swb[jb] = bi8_u2f((bi8_f2u(swr[jb]) + 2u) & ~3u);      // column scale -> 22 significant bits
-            swc[jb] = -BI8_MAGIC * swb[jb];                        // exact
-            // the rest of the NEXT stage's loads, two per column, into the other buffer (released one column ago)
+            swb[jb] = bi8_u2f((bi8_f2u(swr[jb]) + 2u) & ~3u);
+            swc[jb] = -BI8_MAGIC * swb[jb];
             if (j < kLateCols) issue_one(G, kEarly + 2 * j);
             if (j < 7) {
                 read_b(Bf[jb ^ 1], swr[jb ^ 1], j + 1, F);
             } else {
-                // every operand of this stage is in registers or on its way (lgkmcnt): synchronize
-                __builtin_amdgcn_s_waitcnt(0xC07F);                // lgkmcnt(0) only
-                wait_vm(std::integral_constant<int, 0>{});         // this wave's loads of the next stage have landed
+                __builtin_amdgcn_s_waitcnt(0xC07F);
+                wait_vm(std::integral_constant<int, 0>{});
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int idx = 0; idx < kEarly - 1; ++idx) issue_one(F, idx);   // the stage after next, into the buffer just released
-                read_b(Bf[0], swr[0], 0, G);                       // the next stage's column 0
+                for (int idx = 0; idx < kEarly - 1; ++idx) issue_one(F, idx);
+                read_b(Bf[0], swr[0], 0, G);
             }
             __builtin_amdgcn_sched_barrier(0);
-            // rows 0, 1 of column j; meanwhile fold rows 2, 3 of the column before
-            pair(c[0], A[0], A[1], Bf[jb], c[1], sx[2], sx[3], swb[jb ^ 1], swc[jb ^ 1], acc[2][kPrevCol[j]], acc[3][kPrevCol[j]]);
-            if (j == 0) {
-                read_sx(sx[2], 2, F);
-                read_sx(sx[3], 3, F);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cB[jb][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[i][0], Bf[jb][0], magic, 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cB[jb][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[i][1], Bf[jb][1], cB[jb][i], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j == 7) {                          // every MFMA of this stage is issued: the next stage's row subtiles
+                issue_one(F, kEarly - 1);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) read_a(A[i], i, G);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                fold2(cB[jb ^ 1][i], 0, sx[i], swb[jb ^ 1], swc[jb ^ 1], acc[i][kPrevCol[j]]);
+                fold2(cB[jb ^ 1][i], 2, sx[i], swb[jb ^ 1], swc[jb ^ 1], acc[i][kPrevCol[j]]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (j == 0) {                          // this stage's row scales: first needed by the fold in column 1
+#pragma unroll
+                for (int i = 0; i < 4; ++i) read_sx(sx[i], i, F);
             }
             if (j < kLateCols) issue_one(G, kEarly + 2 * j + 1);
-            if (j == 7) {                                          // the next stage's row subtiles 0, 1
-                issue_one(F, kEarly - 1);
-                read_a(A[0], 0, G);
-                read_a(A[1], 1, G);
-            }
             __builtin_amdgcn_sched_barrier(0);
-            // rows 2, 3 of column j; meanwhile fold rows 0, 1 of column j
-            pair(c[1], A[2], A[3], Bf[jb], c[0], sx[0], sx[1], swb[jb], swc[jb], acc[0][j], acc[1][j]);
         }
     };
 
     // ---- BLK = 64: a stage is two K-blocks, each ONE MFMA per subtile.  The stage runs as 16 column steps (K-block
-    // kb = step / 8, column = step % 8); a pair is two MFMAs, each followed by the whole fold of one subtile of the
-    // previous pair (twice the vector work per MFMA of the block-128 schedule).  W fragments (one 16-byte chunk
-    // column) and column scales are read one step ahead, the row scales of K-block 1 at step 8.
+    // kb = step / 8, column = step % 8): the four MFMAs of a step, then the whole fold of the step before (twice the
+    // vector work per MFMA of the block-128 schedule).  W fragments (one 16-byte chunk column) and column scales are
+    // read one step ahead, the row scales of K-block 1 after the fold of step 8.
     bi8_v4i Bh[2];                                 // [step parity]
     auto read_bh = [&](bi8_v4i &dst, float &raw, int step, int buf) {
         const int kb = step >> 3, j = step & 7;
@@ -831,33 +818,14 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     auto read_sx64 = [&](bi8_v4f &dst, int i, int kb, int buf) {
         dst = *(const bi8_v4f *)(lds + sa_base + buf * L::kSBuf + kb * L::kSRow + i * 16 * 4);
     };
-    auto pair64 = [&](bi8_v4i *cn, const bi8_v4i &a0, const bi8_v4i &a1, const bi8_v4i &b, const bi8_v4i *cp, const bi8_v4f &s0,
-                      const bi8_v4f &s1, float fb, float fc, float *d0, float *d1) {
-        cn[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b, magic, 0, 0, 0);
-        fold2(cp[0], 0, s0, fb, fc, d0);
-        fold2(cp[0], 2, s0, fb, fc, d0);
-        __builtin_amdgcn_sched_barrier(0);
-        cn[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b, magic, 0, 0, 0);
-        fold2(cp[1], 0, s1, fb, fc, d1);
-        fold2(cp[1], 2, s1, fb, fc, d1);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    auto stage64 = [&](auto buf_c) {
+    auto stage64 = [&](auto buf_c) {               // same burst schedule: four MFMAs, then the fold of the step before
         constexpr int F = decltype(buf_c)::value, G = 1 - F;
-        read_a(A[2], 2, F);
-        read_a(A[3], 3, F);
-        read_sx64(sx[0], 0, 0, F);
-        read_sx64(sx[1], 1, 0, F);
 #pragma unroll
         for (int h = 0; h < 16; ++h) {
-            const int kb = h >> 3, j = h & 7, hb = h & 1, jprev = (h + 15) & 7;
+            const int kb = h >> 3, hb = h & 1, jprev = (h + 15) & 7;
             swb[hb] = bi8_u2f((bi8_f2u(swr[hb]) + 2u) & ~3u);      // column scale -> 22 significant bits
             swc[hb] = -BI8_MAGIC * swb[hb];                        // exact
             if (h < kLateCols) issue_one(G, kEarly + 2 * h);
-            if (h == 8) {                                          // K-block 1: row subtiles 0, 1 (2, 3 after the pending fold)
-                read_sx64(sx[0], 0, 1, F);
-                read_sx64(sx[1], 1, 1, F);
-            }
             if (h < 15) {
                 read_bh(Bh[hb ^ 1], swr[hb ^ 1], h + 1, F);
             } else {
@@ -870,19 +838,29 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
                 read_bh(Bh[0], swr[0], 0, G);                      // the next stage's first step
             }
             __builtin_amdgcn_sched_barrier(0);
-            pair64(c[0], A[0][kb], A[1][kb], Bh[hb], c[1], sx[2], sx[3], swb[hb ^ 1], swc[hb ^ 1], acc[2][jprev], acc[3][jprev]);
-            if (h == 0 || h == 8) {
-                read_sx64(sx[2], 2, kb, F);
-                read_sx64(sx[3], 3, kb, F);
-            }
-            if (h < kLateCols) issue_one(G, kEarly + 2 * h + 1);
-            if (h == 15) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cB[hb][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[i][kb], Bh[hb], magic, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (h == 15) {                                         // every MFMA of this stage is issued
                 issue_one(F, kEarly - 1);
-                read_a(A[0], 0, G);
-                read_a(A[1], 1, G);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) read_a(A[i], i, G);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // the step before: at h = 0 the previous stage's last step, at h = 8 the last step of K-block 0, both with
+            // the row scales still in sx
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                fold2(cB[hb ^ 1][i], 0, sx[i], swb[hb ^ 1], swc[hb ^ 1], acc[i][jprev]);
+                fold2(cB[hb ^ 1][i], 2, sx[i], swb[hb ^ 1], swc[hb ^ 1], acc[i][jprev]);
             }
             __builtin_amdgcn_sched_barrier(0);
-            pair64(c[1], A[2][kb], A[3][kb], Bh[hb], c[0], sx[0], sx[1], swb[hb], swc[hb], acc[0][j], acc[1][j]);
+            if (h == 0 || h == 8) {                                // this K-block's row scales: first needed one step on
+#pragma unroll
+                for (int i = 0; i < 4; ++i) read_sx64(sx[i], i, kb, F);
+            }
+            if (h < kLateCols) issue_one(G, kEarly + 2 * h + 1);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -895,6 +873,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     __syncthreads();
     read_a(A[0], 0, 0);
     read_a(A[1], 1, 0);
+    read_a(A[2], 2, 0);
+    read_a(A[3], 3, 0);
     if constexpr (BLK == 128) read_b(Bf[0], swr[0], 0, 0);
     else read_bh(Bh[0], swr[0], 0, 0);
     // The trip count is rounded up to even and loads run two stages ahead: stages past the end of K read their
@@ -909,10 +889,11 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         }
     }
     wait_vm(std::integral_constant<int, 0>{});     // nothing may still be writing LDS when the wave ends
-    fold2(c[1][0], 0, sx[2], swb[1], swc[1], acc[2][7]);
-    fold2(c[1][0], 2, sx[2], swb[1], swc[1], acc[2][7]);
-    fold2(c[1][1], 0, sx[3], swb[1], swc[1], acc[3][7]);
-    fold2(c[1][1], 2, sx[3], swb[1], swc[1], acc[3][7]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {                  // the last column of the last (possibly padding) stage
+        fold2(cB[1][i], 0, sx[i], swb[1], swc[1], acc[i][7]);
+        fold2(cB[1][i], 2, sx[i], swb[1], swc[1], acc[i][7]);
+    }
 
     const float div = (float)(1.0 / (127.0 * 127.0));
     const bool has_bias = g.bias != nullptr;
