@@ -611,11 +611,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // The large-problem kernel.  Twice the output per byte of operand moved from L2 to LDS compared to the 256x128
 // tile, which is what bounds gemm_tile at large sizes.  8 waves as 4 (rows) x 2 (columns); one wave owns 64 x 128
 // outputs as 4 x 8 subtiles of 16x16 (v_mfma_i32_16x16x64_i8: four accumulator registers per subtile, so the
-// int32 partials in flight cost 16 registers and the row scales of a stage 16), 128 fp32 accumulators per lane.
-// Per stage (128 bytes of K = one K-block) a wave keeps its 64 rows of A in registers and streams the eight
-// column subtiles of W through two register buffers, one column ahead.  Work is issued in "pairs" (two row
-// subtiles of one column = four MFMAs); each MFMA is followed by a quarter of the fold of the previous pair, so the
-// matrix pipe and the vector ALU overlap.  Two LDS stage buffers, ONE barrier per stage, placed where the last
+// int32 partials of two columns in flight cost 32 registers and the row scales of a stage 16), 128 fp32
+// accumulators per lane.  Per stage (128 bytes of K = one K-block) a wave keeps its 64 rows of A in registers and
+// streams the eight column subtiles of W through two register buffers, one column ahead.  A column's eight MFMAs
+// are issued back to back, then the whole fold of the column before: a wave's vector instructions run under its own
+// MFMAs only (the two waves of a SIMD do not overlap one's MFMAs with the other's vector work), and long runs of
+// each measured faster than alternating instruction by instruction.  Two LDS stage buffers, ONE barrier per stage, placed where the last
 // operand of the stage has been read (top of the eighth column): it certifies that the next stage has landed
 // and releases this stage's buffer to the loads of the stage after next.
 // Measured on MI355X: a SIMD issues about one instruction of any kind per 4 cycles, so the kernel is bound by its
