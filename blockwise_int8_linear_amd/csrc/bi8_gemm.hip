@@ -5,7 +5,7 @@
 //   C[m,n] = cast( (1/127^2) * sum_j sA[j,m] * sW[j,n] * P_j[m,n] ),   P_j = int32 dot over K-block j
 //
 // NT GEMM, both operands K-contiguous.  Four kernels, chosen by shape in dispatch():
-//   gemm_wide    block 128, problems of >= 160 tiles of 256x256: v_mfma_i32_16x16x64_i8, 64x128 per wave;
+//   gemm_wide    blocks 128 / 64, problems of >= 129 tiles of 256x256: v_mfma_i32_16x16x64_i8, 64x128 per wave;
 //   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x128 / 64x128 tiles, 64x64 per wave; also
 //                the int32 block partials;
 //   gemm_gemv    M <= 16, blocks 64/128 (decode): one pass over W, 16 columns per workgroup, K split over 4 waves,
@@ -1471,10 +1471,13 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
 }
 
 // tile shape by problem shape: the big tile when there is enough work to fill 256 CUs with it
-constexpr int64_t kWideMinTiles = 160;
+// Up to 128 tiles of 256x256 the same problem is at most 256 tiles of 256x128: one round of workgroups on the 256 CUs,
+// where the smaller tile wins (1424 against 1072 TOP/s at 2048x4096x4096).  From 129 on the 256x128 grid needs a second,
+// mostly empty round and the 256x256 kernel wins (1284 against 978 TOP/s at 2304x4096x4096, 144 tiles).
+constexpr int64_t kWideMinTiles = 129;
 template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipStream_t st) {
     constexpr bool kBigFits = TileLds<256, 128, BLK, 3>::kFits;
-    // 256x256 tiles once they fill most of the 256 CUs (measured crossover against the 256x128 tile: ~160 tiles)
+    // 256x256 tiles from kWideMinTiles on
     // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
     if constexpr ((BLK == 128 || BLK == 64) && !PARTIALS)
         if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= kWideMinTiles) return launch_wide<BLK, CDT>(g, st);
