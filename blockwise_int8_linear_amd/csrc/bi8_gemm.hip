@@ -623,8 +623,12 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // instruction count; two fold instructions per output per K-block are 2/3 of it.
 template <int NBS> struct WideLds {                 // NBS = K-blocks per stage
     static constexpr int kABuf = 256 * kStageK, kWBuf = 256 * kStageK;       // 32 KiB per operand per stage
-    static constexpr int kSRow = 256 * 4;                                    // one scale row of the tile
-    static constexpr int kSBuf = NBS * kSRow;                                // the stage's scale rows, one per K-block
+    static constexpr int kSRow = 256 * 4;                                    // one row-scale row of the tile
+    static constexpr int kSBuf = NBS * kSRow;                                // the stage's row scales, one row per K-block
+    // column scales are stored prepared: per column the pair (b, -1.5*2^23*b), b = the scale rounded to 22 significant
+    // bits; a wave's 128 columns as [column pair 2p, 2p+1][r16][b0, c0, b1, c1], so a lane reads two columns' pairs at once
+    static constexpr int kCRow = 256 * 8;
+    static constexpr int kCBuf = NBS * kCRow;
     static constexpr int kAReg = 0;
     static constexpr int kWReg = kAReg + 2 * kABuf;
     static constexpr int kSAReg = kWReg + 2 * kWBuf;
@@ -632,7 +636,8 @@ template <int NBS> struct WideLds {                 // NBS = K-blocks per stage
     // after the K loop the same memory holds each wave's 64x128 tile of 16-bit outputs, row-major; the pitch
     // (256 + 16 bytes) puts the four row groups of one accumulator register into different banks
     static constexpr int kOutPitch = 272;
-    static constexpr int kStages = kSWReg + 2 * kSBuf;                       // 132 KiB
+    static constexpr int kDummy = kSWReg + 2 * kCBuf;                        // 1 KiB written and never read
+    static constexpr int kStages = kDummy + 1024;                            // 135 / 141 KiB
     static constexpr int kOut = 8 * 64 * kOutPitch;                          // 136 KiB
     static constexpr int kBytes = kOut > kStages ? kOut : kStages;           // of the CU's 160 KiB
 };
@@ -670,12 +675,25 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     const int64_t nblk = g.K / BLK;
     const bool s_is_a = wave < 4;
     const int s_part = wave & 3;
-    const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
-    const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
-    const bi8_rsrc s_rsrc = s_is_a ? sa_rsrc : sw_rsrc;
+    const bi8_brsrc sa_brsrc = bi8_make_brsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
+    const bi8_brsrc sw_brsrc = bi8_make_brsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
+    const bi8_brsrc s_brsrc = s_is_a ? sa_brsrc : sw_brsrc;
     const uint32_t s_off = (uint32_t)((s_part * 64 + lane) * 4);
-    const uint32_t s_dst = (uint32_t)((s_is_a ? L::kSAReg : L::kSWReg) + s_part * 256);
     const uint32_t s_inc = (uint32_t)((s_is_a ? g.M : g.N) * 4);
+    // The scales come into a register of the fetching lane, which stores them to LDS just before the barrier that
+    // publishes the stage.  Row scales are stored as they are.  Column scales are stored prepared, so that the
+    // preparation is done once per column instead of once per wave row and lane group: lane -> tile column
+    // s_part * 64 + lane = wave column (s_part >> 1), subtile j = 4 * (s_part & 1) + lane / 16, r16 = lane % 16.
+    // Both kinds run the same instructions (no branch: a branch in the K loop costs the register allocator its
+    // footing): two 4-byte stores, the second of a row-scale lane to a slot nobody reads.
+    float s_raw[NBS];
+#pragma unroll
+    for (int kb = 0; kb < NBS; ++kb) s_raw[kb] = 0.0f;
+    const int c_dst = L::kSWReg + (s_part >> 1) * 1024 + (((2 * (s_part & 1) + (lane >> 5)) * 16 + (lane & 15)) * 2 + ((lane >> 4) & 1)) * 8;
+    int p_dst0 = s_is_a ? L::kSAReg + (s_part * 64 + lane) * 4 : c_dst;
+    int p_dst1 = s_is_a ? L::kDummy + (s_part * 64 + lane) * 4 : c_dst + 4;
+    const int p_buf0 = s_is_a ? L::kSBuf : L::kCBuf, p_row0 = s_is_a ? L::kSRow : L::kCRow;
+    const int p_buf1 = s_is_a ? 0 : L::kCBuf, p_row1 = s_is_a ? 0 : L::kCRow;
     uint32_t s_pos = 0, k_pos = 0;                 // scale-row and K position of the next stage to load
     constexpr int kLoadsPerStage = 4 + 4 + NBS;
     // A wave's nine or ten load instructions of a stage are spread out so that the texture path never sees all of
@@ -691,9 +709,19 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         } else if (idx < 8) {
             bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + (idx - 4) * NW) * 1024, w_off, k_pos, w_wave + (idx - 4) * w_step);
         } else if (idx < kLoadsPerStage) {
-            bi8_buffer_to_lds4(s_rsrc, lds_base + s_dst + buf * L::kSBuf + (idx - 8) * L::kSRow, s_off, s_pos);
+            s_raw[idx - 8] = bi8_buffer_load_f32(s_brsrc, (int)s_off, (int)s_pos);
             s_pos += s_inc;
             if (idx == kLoadsPerStage - 1) k_pos += kStageK;
+        }
+    };
+
+    // the fetching lanes' scales of the stage that goes to buffer `buf` (all loads have been waited for)
+    auto publish_scales = [&](int buf) {
+#pragma unroll
+        for (int kb = 0; kb < NBS; ++kb) {
+            const float b = bi8_u2f((bi8_f2u(s_raw[kb]) + 2u) & ~3u);     // 22 significant bits
+            *(float *)(lds + p_dst0 + buf * p_buf0 + kb * p_row0) = s_is_a ? s_raw[kb] : b;
+            *(float *)(lds + p_dst1 + buf * p_buf1 + kb * p_row1) = -BI8_MAGIC * b;          // exact
         }
     };
 
@@ -707,11 +735,11 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     w_base[1] = w_base[0] ^ 64;
     // a subtile's outputs: lane -> column r16, rows 4q .. 4q+3
     int sa_base = L::kSAReg + (wm * 64 + 4 * q) * 4;
-    int sw_base = L::kSWReg + (wn * 128 + r16) * 4;
+    int sw_base = L::kSWReg + wn * 1024 + r16 * 16;
     // The region offsets (64 KiB and up) stay inside these six registers: every access below is one of them plus an
     // immediate under 64 KiB.  Left to itself the compiler folds each region offset into the immediates, finds them
     // too large for the instruction's 16-bit field, and keeps a separate address register per access (24 spilled).
-    asm volatile("" : "+v"(a_base[0]), "+v"(a_base[1]), "+v"(w_base[0]), "+v"(w_base[1]), "+v"(sa_base), "+v"(sw_base));
+    asm volatile("" : "+v"(a_base[0]), "+v"(a_base[1]), "+v"(w_base[0]), "+v"(w_base[1]), "+v"(sa_base), "+v"(sw_base), "+v"(p_dst0), "+v"(p_dst1));
 
     float acc[4][8][4];
 #pragma unroll
@@ -725,7 +753,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     const bi8_v4i magic = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
     bi8_v4i A[4][2], Bf[2][2];                     // [row subtile][kb], [column parity][kb]
     bi8_v4f sx[4];                                 // row scales per row subtile
-    float swb[2] = {0.0f, 0.0f}, swc[2] = {0.0f, 0.0f}, swr[2] = {0.0f, 0.0f};   // per column parity: b, -(1.5*2^23)*b, raw
+    bi8_v4f bc[2];                                 // per column pair (parity of the pair): b, -(1.5*2^23)*b of its two columns
+    bc[0] = bc[1] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int i = 0; i < 4; ++i) sx[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -733,15 +762,16 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) dst[kb] = *(const bi8_v4i *)(lds + a_base[kb] + buf * L::kABuf + i * 16 * kStageK);
     };
-    auto read_b = [&](bi8_v4i *dst, float &raw, int j, int buf) {
+    auto read_b = [&](bi8_v4i *dst, int j, int buf) {
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) dst[kb] = *(const bi8_v4i *)(lds + w_base[kb] + buf * L::kWBuf + j * 16 * kStageK);
-        raw = *(const float *)(lds + sw_base + buf * L::kSBuf + j * 16 * 4);
+        if ((j & 1) == 0) bc[(j >> 1) & 1] = *(const bi8_v4f *)(lds + sw_base + buf * L::kCBuf + (j >> 1) * 256);
     };
     auto read_sx = [&](bi8_v4f &dst, int i, int buf) { dst = *(const bi8_v4f *)(lds + sa_base + buf * L::kSBuf + i * 16 * 4); };
     // two elements of a finished partial: fma(f, b, c) = fl(b * P) (the partial carries the 1.5*2^23 offset), then
     // the row scale and the accumulation
-    auto fold2 = [&](const bi8_v4i &pt, int r0, const bi8_v4f &s, float b, float cm, float *dst) {
+    auto fold2 = [&](const bi8_v4i &pt, int r0, const bi8_v4f &s, int col, float *dst) {
+        const float b = bc[(col >> 1) & 1][2 * (col & 1)], cm = bc[(col >> 1) & 1][2 * (col & 1) + 1];
 #pragma unroll
         for (int r = r0; r < r0 + 2; ++r) {
             const float u = __builtin_fmaf(bi8_u2f((uint32_t)pt[r]), b, cm);
@@ -765,19 +795,18 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         for (int j = 0; j < 8; ++j) {
             constexpr int kPrevCol[8] = {7, 0, 1, 2, 3, 4, 5, 6};
             const int jb = j & 1;
-            swb[jb] = bi8_u2f((bi8_f2u(swr[jb]) + 2u) & ~3u);
-            swc[jb] = -BI8_MAGIC * swb[jb];
             if (j < kLateCols) issue_one(G, kEarly + 2 * j);
             if (j < 7) {
-                read_b(Bf[jb ^ 1], swr[jb ^ 1], j + 1, F);
+                read_b(Bf[jb ^ 1], j + 1, F);
             } else {
                 __builtin_amdgcn_s_waitcnt(0xC07F);
                 wait_vm(std::integral_constant<int, 0>{});
+                publish_scales(G);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int idx = 0; idx < kEarly - 1; ++idx) issue_one(F, idx);
-                read_b(Bf[0], swr[0], 0, G);
+                read_b(Bf[0], 0, G);
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -793,8 +822,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                fold2(cB[jb ^ 1][i], 0, sx[i], swb[jb ^ 1], swc[jb ^ 1], acc[i][kPrevCol[j]]);
-                fold2(cB[jb ^ 1][i], 2, sx[i], swb[jb ^ 1], swc[jb ^ 1], acc[i][kPrevCol[j]]);
+                fold2(cB[jb ^ 1][i], 0, sx[i], kPrevCol[j], acc[i][kPrevCol[j]]);
+                fold2(cB[jb ^ 1][i], 2, sx[i], kPrevCol[j], acc[i][kPrevCol[j]]);
             }
             __builtin_amdgcn_sched_barrier(0);
             if (j == 0) {                          // this stage's row scales: first needed by the fold in column 1
@@ -811,10 +840,10 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     // vector work per MFMA of the block-128 schedule).  W fragments (one 16-byte chunk column) and column scales are
     // read one step ahead, the row scales of K-block 1 after the fold of step 8.
     bi8_v4i Bh[2];                                 // [step parity]
-    auto read_bh = [&](bi8_v4i &dst, float &raw, int step, int buf) {
+    auto read_bh = [&](bi8_v4i &dst, int step, int buf) {
         const int kb = step >> 3, j = step & 7;
         dst = *(const bi8_v4i *)(lds + w_base[kb] + buf * L::kWBuf + j * 16 * kStageK);
-        raw = *(const float *)(lds + sw_base + buf * L::kSBuf + kb * L::kSRow + j * 16 * 4);
+        if ((j & 1) == 0) bc[(j >> 1) & 1] = *(const bi8_v4f *)(lds + sw_base + buf * L::kCBuf + kb * L::kCRow + (j >> 1) * 256);
     };
     auto read_sx64 = [&](bi8_v4f &dst, int i, int kb, int buf) {
         dst = *(const bi8_v4f *)(lds + sa_base + buf * L::kSBuf + kb * L::kSRow + i * 16 * 4);
@@ -824,19 +853,18 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
 #pragma unroll
         for (int h = 0; h < 16; ++h) {
             const int kb = h >> 3, hb = h & 1, jprev = (h + 15) & 7;
-            swb[hb] = bi8_u2f((bi8_f2u(swr[hb]) + 2u) & ~3u);      // column scale -> 22 significant bits
-            swc[hb] = -BI8_MAGIC * swb[hb];                        // exact
             if (h < kLateCols) issue_one(G, kEarly + 2 * h);
             if (h < 15) {
-                read_bh(Bh[hb ^ 1], swr[hb ^ 1], h + 1, F);
+                read_bh(Bh[hb ^ 1], h + 1, F);
             } else {
                 __builtin_amdgcn_s_waitcnt(0xC07F);                // lgkmcnt(0) only
                 wait_vm(std::integral_constant<int, 0>{});
+                publish_scales(G);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int idx = 0; idx < kEarly - 1; ++idx) issue_one(F, idx);
-                read_bh(Bh[0], swr[0], 0, G);                      // the next stage's first step
+                read_bh(Bh[0], 0, G);                              // the next stage's first step
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -852,8 +880,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             // the row scales still in sx
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                fold2(cB[hb ^ 1][i], 0, sx[i], swb[hb ^ 1], swc[hb ^ 1], acc[i][jprev]);
-                fold2(cB[hb ^ 1][i], 2, sx[i], swb[hb ^ 1], swc[hb ^ 1], acc[i][jprev]);
+                fold2(cB[hb ^ 1][i], 0, sx[i], jprev, acc[i][jprev]);
+                fold2(cB[hb ^ 1][i], 2, sx[i], jprev, acc[i][jprev]);
             }
             __builtin_amdgcn_sched_barrier(0);
             if (h == 0 || h == 8) {                                // this K-block's row scales: first needed one step on
@@ -871,13 +899,14 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
 #pragma unroll
     for (int idx = 0; idx < kEarly; ++idx) issue_one(1, idx);
     wait_vm(std::integral_constant<int, kEarly>{});
+    publish_scales(0);
     __syncthreads();
     read_a(A[0], 0, 0);
     read_a(A[1], 1, 0);
     read_a(A[2], 2, 0);
     read_a(A[3], 3, 0);
-    if constexpr (BLK == 128) read_b(Bf[0], swr[0], 0, 0);
-    else read_bh(Bh[0], swr[0], 0, 0);
+    if constexpr (BLK == 128) read_b(Bf[0], 0, 0);
+    else read_bh(Bh[0], 0, 0);
     // The trip count is rounded up to even and loads run two stages ahead: stages past the end of K read their
     // scales through the buffers' range check as zeros, so they add exactly 0 to the accumulators.
     for (int s = 0; s < nstages; s += 2) {
@@ -892,8 +921,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     wait_vm(std::integral_constant<int, 0>{});     // nothing may still be writing LDS when the wave ends
 #pragma unroll
     for (int i = 0; i < 4; ++i) {                  // the last column of the last (possibly padding) stage
-        fold2(cB[1][i], 0, sx[i], swb[1], swc[1], acc[i][7]);
-        fold2(cB[1][i], 2, sx[i], swb[1], swc[1], acc[i][7]);
+        fold2(cB[1][i], 0, sx[i], 7, acc[i][7]);
+        fold2(cB[1][i], 2, sx[i], 7, acc[i][7]);
     }
 
     const float div = (float)(1.0 / (127.0 * 127.0));
