@@ -220,8 +220,8 @@ def cpu_baseline(torch, xq, wq, sx, sw, B, chunk: int = 2048):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the GEMM (the metric is quoted at 8192)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-quantize", action="store_true")
