@@ -16,6 +16,22 @@ namespace {
 constexpr int kTR = 128;           // tile rows
 constexpr int kTC = 64;            // columns of one half
 constexpr int kThreads = 256;
+// Tile order, as in bi8_quantize_transposed: the tiles in flight at one time form a compact patch of the matrix
+// (bands of kSBR tile rows, chunks of kSBC tile columns inside a band, row by row inside a chunk), so that the reads
+// and row-direction writes (runs along the rows) and the column-direction writes (runs down the columns) of the patch
+// are all long runs in memory.
+// Measured on bf16 [8192,8192]: 16 x 16 tiles 64.0 us, row by row 65.4, 8 x 32 64.6, 32 x 8 69.
+constexpr int kSBR = 16, kSBC = 16;
+__device__ __forceinline__ void tile_coords(int64_t t, int64_t tiles_r, int64_t tiles_c, int64_t &tr, int64_t &tc) {
+    const int64_t band = t / (kSBR * tiles_c);
+    const int64_t rows_b = (tiles_r - band * kSBR < kSBR) ? (tiles_r - band * kSBR) : kSBR;
+    const int64_t in = t - band * kSBR * tiles_c;
+    const int64_t chunk = in / (rows_b * kSBC);
+    const int64_t wc = (tiles_c - chunk * kSBC < kSBC) ? (tiles_c - chunk * kSBC) : kSBC;
+    const int64_t in2 = in - chunk * rows_b * kSBC;
+    tr = band * kSBR + in2 / wc;
+    tc = chunk * kSBC + in2 % wc;
+}
 constexpr int kPitch = kTC + 1;    // fp32 half-tile pitch: column walks hit distinct banks
 constexpr int kQPitch = kTR + 4;   // code tile pitch in bytes (33 dwords)
 
@@ -45,9 +61,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
     const int lr = tid / LPR;                      // row inside a pass
     const int cc = (tid % LPR) * VEC;              // first column of this lane inside a half
 
+    const int64_t tiles_r = (R + kTR - 1) / kTR;
     auto load_half = [&](int64_t tile, int h, bi8_v4u *raw) {
-        const int64_t r0 = (tile / tiles_c) * kTR;
-        const int64_t c0 = (tile % tiles_c) * (2 * kTC) + h * kTC;
+        int64_t tr = 0, tc = 0;
+        if (tile < ntiles) tile_coords(tile, tiles_r, tiles_c, tr, tc);
+        const int64_t r0 = tr * kTR;
+        const int64_t c0 = tc * (2 * kTC) + h * kTC;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             const int r = p * RPP + lr;
@@ -75,8 +94,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
     load_half(blockIdx.x, 0, raw[0]);
     load_half(blockIdx.x, 1, raw[1]);
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
-        const int64_t r0 = (tile / tiles_c) * kTR;
-        const int64_t cbase = (tile % tiles_c) * (2 * kTC);
+        int64_t tr, tc;
+        tile_coords(tile, tiles_r, tiles_c, tr, tc);
+        const int64_t r0 = tr * kTR;
+        const int64_t cbase = tc * (2 * kTC);
 
         // ---- along the rows, from the registers ----------------------------------------------------------------
 #pragma unroll

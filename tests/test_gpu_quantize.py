@@ -144,9 +144,10 @@ def test_dequantize_parity(ops, out):
 @pytest.mark.parametrize("block", [32, 64, 128])
 def test_quantize_transposed_equals_two_step(ops, dtype, block):
     # the last four: odd row lengths of the source and/or of the output (unaligned loads / byte stores in the tile
-    # kernel), among them the GPT-2 vocabulary as either dimension
+    # kernel), among them the GPT-2 vocabulary as either dimension; the last two: more tiles than one patch of the tile
+    # order in both directions, with and without ragged last bands / chunks
     for (R, C) in [(256, 512), (8192, 768), (300, 1000), (1000, 72), (129, 64), (64, 50257 // 8 * 8),
-                   (300, 517), (517, 304), (333, 77), (64, 50257), (50257, 64)]:
+                   (300, 517), (517, 304), (333, 77), (64, 50257), (50257, 64), (2181, 2115), (2304, 4160)]:
         x_cpu = outlier_tensor(R, C, DTYPES[dtype], seed=R + C)
         q, s = _check_quant(ops, x_cpu, block, transposed=True)
         x = x_cpu.to(DEV)

@@ -43,7 +43,7 @@ def test_dual_parity(ops, dtype, block):
     # whole tiles, ragged tiles in either direction, a single partial tile, one row, one 16-byte column group, many
     # tiles per workgroup (more than 768 tiles), and shapes of the training configurations
     for (R, C) in [(256, 256), (128, 128), (300, 1000), (1000, 72), (129, 64), (5, 8), (1, 4096), (4096, 8),
-                   (8192, 768), (768, 3072), (2176, 2304), (77, 1048)]:
+                   (8192, 768), (768, 3072), (2176, 2304), (77, 1048), (2181, 2115)]:
         _check(ops, outlier_tensor(R, C, DTYPES[dtype], seed=R * 3 + C + block), block)
 
 
