@@ -1455,9 +1455,19 @@ static int split_ways(int64_t tiles, int64_t nstages) {
 static int plan_split(int64_t M, int64_t N, int64_t K, int &kind) {
     const int64_t nstages = K / kStageK;
     kind = M > 64 ? 1 : 0;
-    const int64_t tiles = M > 64 ? ((M + 127) / 128) * ((N + 127) / 128) : ((M + 63) / 64) * ((N + 127) / 128);
+    const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128), t64 = ((M + 63) / 64) * ((N + 127) / 128);
     // (splitting the 256x128 tile where the 128x128 tiles are too many to split measured slower than not splitting)
-    return split_ways(tiles, nstages);
+    const int sp = split_ways(kind ? t128 : t64, nstages);
+    // a short K caps the number of splits: when the 128x128 tiles then fill at most half of the CUs, the 64x128 tile
+    // puts twice as many workgroups to work
+    if (kind == 1 && t128 * sp <= 128) {
+        const int sp64 = split_ways(t64, nstages);
+        if (sp64 > 1 && t64 * sp64 > t128 * sp) {
+            kind = 0;
+            return sp64;
+        }
+    }
+    return sp;
 }
 
 template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
