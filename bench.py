@@ -121,7 +121,35 @@ def bench_extras(pkg, torch):
     g64()
     t = min(event_ms(g64, 10) for _ in range(2))
     out["gemm_block64_8192"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1)}
-    del a, w, sa, sw, c
+    del sa, sw, c
+
+    # Context, not part of the path: the vendor library's PLAIN int8 GEMM (int32 out, no scales, no fold) on random
+    # codes of the same shape, and the block-128 kernel on all-zero codes.  Both show how far the chip's power
+    # management moves the ceiling with the data: the published peak is quoted at 2.4 GHz, which the chip holds only
+    # when the operands do not toggle.
+    try:
+        wt = w.t()
+        for _ in range(30):
+            torch._int_mm(a, wt)
+        t = min(event_ms(lambda: torch._int_mm(a, wt), 30) for _ in range(2))
+        out["context_vendor_plain_int8_gemm_8192_random_codes"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1),
+                                                                   "what": "torch._int_mm (hipBLASLt), int32 out, no dequantize"}
+    except Exception as e:                          # not every torch build has it: the figure is context only
+        out["context_vendor_plain_int8_gemm_8192_random_codes"] = {"error": repr(e)[:120]}
+    del a, w
+    z = torch.zeros(S, S, device="cuda", dtype=torch.int8)
+    sa = torch.rand(S // 128, S, device="cuda") + 0.5
+    sw = torch.rand(S // 128, S, device="cuda") * 0.02
+    c = torch.empty(S, S, device="cuda", dtype=torch.bfloat16)
+
+    def gz():
+        assert lib.bi8_gemm_nt_dequant(z.data_ptr(), z.data_ptr(), sa.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
+                                       S, S, S, S, S, S, 128, st) == 0
+    for _ in range(30):
+        gz()
+    t = min(event_ms(gz, 20) for _ in range(2))
+    out["context_gemm_block128_8192_zero_codes"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1)}
+    del z, sa, sw, c
 
     B = 128
     for (K, N) in ((4096, 11008), (11008, 4096)):
