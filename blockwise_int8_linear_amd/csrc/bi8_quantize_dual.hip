@@ -7,7 +7,7 @@
 // A workgroup owns a 128 x 128 tile, held in registers as two 64-column halves (16 bytes per lane per row pass; the
 // next tile's loads are issued while this one is processed).  The row direction is finished straight from the
 // registers: the lanes of one row reduce their absmax with DPP, quantize and store their codes.  The column direction
-// runs half by half through LDS exactly as in bi8_quantize_transposed.  Both outputs are bit for bit those of the
+// runs half by half through LDS exactly as in bi8_quantize_transposed (tile kept in its own type, 16-byte LDS accesses).  Both outputs are bit for bit those of the
 // two separate entry points.
 #include "bi8_common.h"
 
@@ -32,8 +32,7 @@ __device__ __forceinline__ void tile_coords(int64_t t, int64_t tiles_r, int64_t 
     tr = band * kSBR + in2 / wc;
     tc = chunk * kSBC + in2 % wc;
 }
-constexpr int kPitch = kTC + 1;    // fp32 half-tile pitch: column walks hit distinct banks
-constexpr int kQPitch = kTR + 4;   // code tile pitch in bytes (33 dwords)
+constexpr int kQPitch = kTR + 16;  // code tile pitch in bytes: rows stay 16-byte aligned
 
 // ALIGNED: rows of x start on 16-byte boundaries and C is a multiple of the elements per 16 bytes, rows of q on 8-byte
 // boundaries.  Otherwise whole 16-byte chunks move with unaligned accesses and the last, partial chunk of a row
@@ -49,11 +48,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
     constexpr int RPP = kThreads / LPR;            // rows per load pass
     constexpr int NP = kTR / RPP;                  // load passes per half
     constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
-    constexpr int GPB = B / 32;                    // 32-row groups per column block
+    constexpr int ESZ = (int)ES;                   // bytes per element
+    constexpr int CPT = 4 / ESZ;                   // columns per thread in the column walk: one 32-bit word
+    constexpr int G = kThreads / (kTC / CPT);      // row groups: 4 (fp32) or 8
+    constexpr int RPT = kTR / G;                   // rows per thread: 32 (fp32) or 16
+    constexpr int GPW = B / RPT;                   // row groups per column block
+    constexpr int kXPitch = kTC * ESZ + (ESZ == 4 ? 0 : 16);   // bytes, 16-byte aligned (as in bi8_quantize_transposed)
     constexpr int LB = (B < kTC ? B : kTC) / VEC;  // lanes of one half row that share a row block
     static_assert(B == 32 || B == 64 || B == 128, "tile = one or more whole blocks in both directions");
-    __shared__ float s_x[kTR * kPitch];
-    __shared__ float s_max[4][kTC];
+    __shared__ __attribute__((aligned(16))) uint8_t s_x[kTR * kXPitch];
+    __shared__ float s_max[G][kTC];
     __shared__ __attribute__((aligned(16))) uint8_t s_q[kTC * kQPitch];
 
     const int tid = threadIdx.x;
@@ -163,56 +167,78 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int64_t c0 = cbase + h * kTC;
-            // phase 1: this half -> fp32 in LDS (the previous half's column reads ended before the barrier that
+            // phase 1: this half -> LDS as it is (the previous half's column reads ended before the barrier that
             // precedes its phase 4); then start the next tile's loads of this half
 #pragma unroll
-            for (int p = 0; p < NP; ++p) {
-                float f[VEC];
-                bi8_unpack<DT>(raw[h][p], f);
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) s_x[(p * RPP + lr) * kPitch + cc + e] = f[e];
-            }
+            for (int p = 0; p < NP; ++p) *(bi8_v4u *)&s_x[(p * RPP + lr) * kXPitch + (tid % LPR) * 16] = raw[h][p];
             load_half(tile + gridDim.x, h, raw[h]);
             __syncthreads();
 
-            // phase 2: column maxima over this thread's 32 rows, then over the block's row groups
-            const int c = tid & 63;
-            const int g = tid >> 6;
-            float v[32];
-            float m = 0.0f;
+            // phase 2: column maxima over this thread's rows (one 32-bit word column: one fp32 column or two 16-bit
+            // columns), then over the block's row groups
+            const int cw = tid % (kTC / CPT);
+            const int g = tid / (kTC / CPT);
+            float v[CPT][RPT];
+            float m[CPT];
             bool special = false;
 #pragma unroll
-            for (int i = 0; i < 32; ++i) {
-                v[i] = s_x[(g * 32 + i) * kPitch + c];
-                m = __builtin_fmaxf(m, __builtin_fabsf(v[i]));
-                special |= (v[i] != v[i]);
-            }
-            if constexpr (GPB > 1) {
-                s_max[g][c] = m;
-                __syncthreads();
-                const int gb = g & ~(GPB - 1);
+            for (int k = 0; k < CPT; ++k) m[k] = 0.0f;
 #pragma unroll
-                for (int k = 0; k < GPB; ++k) m = __builtin_fmaxf(m, s_max[gb + k][c]);
+            for (int i = 0; i < RPT; ++i) {
+                const uint32_t d = *(const uint32_t *)&s_x[(g * RPT + i) * kXPitch + cw * 4];
+                if constexpr (DT == BI8_F32) {
+                    v[0][i] = bi8_u2f(d);
+                } else if constexpr (DT == BI8_BF16) {
+                    v[0][i] = bi8_u2f(d << 16);
+                    v[1][i] = bi8_u2f(d & 0xffff0000u);
+                } else {
+                    v[0][i] = bi8_from_f16_bits(d & 0xffffu);
+                    v[1][i] = bi8_from_f16_bits(d >> 16);
+                }
+#pragma unroll
+                for (int k = 0; k < CPT; ++k) {
+                    m[k] = __builtin_fmaxf(m[k], __builtin_fabsf(v[k][i]));
+                    special |= (v[k][i] != v[k][i]);
+                }
             }
-            if ((g & (GPB - 1)) == 0) {
-                const int64_t jb = (r0 + g * 32) / B;
-                if (r0 + g * 32 < R && c0 + c < C) scalesT[jb * C + c0 + c] = m;
+            if constexpr (GPW > 1) {
+#pragma unroll
+                for (int k = 0; k < CPT; ++k) s_max[g][cw * CPT + k] = m[k];
+                __syncthreads();
+                const int gb = g & ~(GPW - 1);
+#pragma unroll
+                for (int qg = 0; qg < GPW; ++qg)
+#pragma unroll
+                    for (int k = 0; k < CPT; ++k) m[k] = __builtin_fmaxf(m[k], s_max[gb + qg][cw * CPT + k]);
+            }
+            if ((g & (GPW - 1)) == 0) {
+                const int64_t jb = (r0 + g * RPT) / B;
+#pragma unroll
+                for (int k = 0; k < CPT; ++k)
+                    if (r0 + g * RPT < R && c0 + cw * CPT + k < C) scalesT[jb * C + c0 + cw * CPT + k] = m[k];
             }
 
-            // phase 3: codes of this thread's 32 rows -> byte tile [column][row]
-            special |= !bi8_scale_is_ordinary(m);
-            uint32_t code[32];
-            if (__builtin_expect(special, 0)) {
+            // phase 3: codes of this thread's rows -> byte tile [column][row], 16 bytes per store
 #pragma unroll
-                for (int i = 0; i < 32; ++i) code[i] = bi8_code_slow(v[i], m);
-            } else {
-                const float y = 1.0f / m;
+            for (int k = 0; k < CPT; ++k) {
+                uint32_t code[RPT];
+                if (__builtin_expect(special || !bi8_scale_is_ordinary(m[k]), 0)) {
 #pragma unroll
-                for (int i = 0; i < 32; ++i) code[i] = bi8_code_fast<NCORR>(v[i], m, y);
+                    for (int i = 0; i < RPT; ++i) code[i] = bi8_code_slow(v[k][i], m[k]);
+                } else {
+                    const float y = 1.0f / m[k];
+#pragma unroll
+                    for (int i = 0; i < RPT; ++i) code[i] = bi8_code_fast<NCORR>(v[k][i], m[k], y);
+                }
+#pragma unroll
+                for (int i = 0; i < RPT / 16; ++i) {
+                    bi8_v4u w;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        w[e] = bi8_pack4(code[16 * i + 4 * e], code[16 * i + 4 * e + 1], code[16 * i + 4 * e + 2], code[16 * i + 4 * e + 3]);
+                    *(bi8_v4u *)&s_q[(cw * CPT + k) * kQPitch + g * RPT + 16 * i] = w;
+                }
             }
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                *(uint32_t *)&s_q[c * kQPitch + g * 32 + 4 * i] = bi8_pack4(code[4 * i], code[4 * i + 1], code[4 * i + 2], code[4 * i + 3]);
             __syncthreads();
 
             // phase 4: 16 codes per lane, 8 lanes per output row.  The next writes to s_x come after this barrier, the
@@ -225,8 +251,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
                 const int64_t orow = c0 + oc;
                 const int64_t ocol = r0 + seg * 16;
                 if (orow < C && ocol < R) {
-                    const uint32_t *src = (const uint32_t *)&s_q[oc * kQPitch + seg * 16];
-                    bi8_v4u w = {src[0], src[1], src[2], src[3]};
+                    const bi8_v4u w = *(const bi8_v4u *)&s_q[oc * kQPitch + seg * 16];
                     int8_t *dst = qT + orow * ldqt + ocol;
                     if (ocol + 16 <= R) {
                         __builtin_nontemporal_store(w, (bi8_v4u *)dst);
@@ -245,7 +270,9 @@ int launch_dual(const void *x, int8_t *q, float *scales, int8_t *qT, float *scal
     const int64_t tiles_c = (C + 2 * kTC - 1) / (2 * kTC);
     const int64_t tiles_r = (R + kTR - 1) / kTR;
     const int64_t ntiles = tiles_c * tiles_r;
-    const int64_t resident = 3 * 256;              // at most three workgroups fit a CU (42 KiB of LDS each)
+    // workgroups per CU: four with 16-bit inputs (29 KiB of LDS, under 128 registers: 62.7 us against 65.9 with three at
+    // bf16 [8192,8192]), three with fp32 (42 KiB)
+    const int64_t resident = (DT == BI8_F32 ? 3 : 4) * 256;
     const int64_t grid = ntiles < resident ? ntiles : resident;
     hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT, R, C,
                        ldx, ldq, ldqt, tiles_c, ntiles);
