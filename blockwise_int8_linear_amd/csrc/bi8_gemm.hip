@@ -22,6 +22,7 @@
 //     one chunk column cover all 64 banks, so the MFMA operand reads (ds_read_b128) run at full LDS rate;
 //   - the workgroup index is remapped so that the 32 workgroups resident on one XCD (one L2) cover a
 //     compact patch of output tiles.
+#include <atomic>
 #include <type_traits>
 
 #include "bi8_common.h"
@@ -1470,6 +1471,22 @@ static int plan_split(int64_t M, int64_t N, int64_t K, int &kind) {
     return sp;
 }
 
+// A kernel that uses more than 64 KiB of dynamic LDS has to be allowed to, once per device: remembered here so that
+// the launch path makes that runtime call only the first time.
+struct LdsOptIn {
+    std::atomic<uint64_t> done{0};                 // bit d: device d has the attribute
+    int ensure(const void *kern, int bytes) {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return bi8_hip_rc(e);
+        if (dev >= 0 && dev < 64 && ((done.load(std::memory_order_acquire) >> dev) & 1)) return BI8_OK;
+        e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return bi8_hip_rc(e);
+        if (dev >= 0 && dev < 64) done.fetch_or(1ull << dev, std::memory_order_release);
+        return BI8_OK;
+    }
+};
+
 template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
 int launch_tile(GemmArgs g, hipStream_t st) {
     constexpr int kLds = TileLds<BM, BN, BLK, NBUF>::kBytes;
@@ -1480,8 +1497,9 @@ int launch_tile(GemmArgs g, hipStream_t st) {
     g.tiles_n = (int)tn;
     auto kern = gemm_tile<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>;
     if (kLds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
-        if (e != hipSuccess) return bi8_hip_rc(e);
+        static LdsOptIn opted;                     // one per kernel instantiation
+        const int rc = opted.ensure((const void *)kern, kLds);
+        if (rc != BI8_OK) return rc;
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn), (unsigned)(g.splits > 1 ? g.splits : 1)), dim3(WM * WN * 64), kLds, st, g);
     return bi8_launch_rc();
@@ -1494,8 +1512,9 @@ template <int BLK, int CDT> int launch_wide(GemmArgs g, hipStream_t st) {
     g.tiles_m = (int)tm;
     g.tiles_n = (int)tn;
     auto kern = gemm_wide<BLK, CDT>;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, L::kBytes);
-    if (e != hipSuccess) return bi8_hip_rc(e);
+    static LdsOptIn opted;                         // one per kernel instantiation
+    const int rc = opted.ensure((const void *)kern, L::kBytes);
+    if (rc != BI8_OK) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(512), L::kBytes, st, g);
     return bi8_launch_rc();
 }
@@ -1509,48 +1528,78 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
     return bi8_launch_rc();
 }
 
-// tile shape by problem shape: the big tile when there is enough work to fill 256 CUs with it
+constexpr int kGemvMaxBlocks = 512;                // gemm_gemv keeps the row scales in LDS: 64 bytes per K-block, 32 KiB at most
+
+// ---- which kernel runs a problem ------------------------------------------------------------------------------------
+// One rule, used by the launcher, by bi8_gemm_workspace_bytes and by bi8_gemm_kernel_name.
+enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128 };
+static const char *const kGemmKernelNames[] = {"gemm_generic", "gemm_gemv", "gemm_skinny", "gemm_wide", "gemm_tile_256x128",
+                                                "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk",
+                                                "gemm_tile_64x128_splitk"};
+struct GemmPlan {
+    int kernel;
+    int splits, split_stages;      // of the split kernels: workgroups per tile along K and 128-byte stages of K per split
+};
 // Up to 128 tiles of 256x256 the same problem is at most 256 tiles of 256x128: one round of workgroups on the 256 CUs,
 // where the smaller tile wins (1424 against 1072 TOP/s at 2048x4096x4096).  From 129 on the 256x128 grid needs a second,
 // mostly empty round and the 256x256 kernel wins (1284 against 978 TOP/s at 2304x4096x4096, 144 tiles).
+// (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
 constexpr int64_t kWideMinTiles = 129;
-template <int BLK, int CDT, bool PARTIALS> int pick_tile(const GemmArgs &g, hipStream_t st) {
-    constexpr bool kBigFits = TileLds<256, 128, BLK, 3>::kFits;
-    // 256x256 tiles from kWideMinTiles on
-    // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
-    if constexpr ((BLK == 128 || BLK == 64) && !PARTIALS)
-        if (((g.M + 255) / 256) * ((g.N + 255) / 256) >= kWideMinTiles) return launch_wide<BLK, CDT>(g, st);
-    if constexpr (kBigFits) {
-        // 128x128 tiles while they fit one round of workgroups on the 256 CUs; beyond that the 256x128 tile (measured
-        // 25-40 % faster than two rounds of 128x128 tiles at 288-320 of them)
-        const int64_t t128 = ((g.M + 127) / 128) * ((g.N + 127) / 128);
-        if (g.M > 128 && t128 > 256) return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : 3, BLK, CDT, PARTIALS>(g, st);
+// `aligned`: A and W 16-byte aligned, the scales 4-byte aligned (the partials entry point has no scales);
+// ws_bytes: scratch memory the split kernels may use (0: none).
+static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block, bool aligned, bool partials,
+                          int64_t ws_bytes) {
+    GemmPlan p{kKGeneric, 1, 0};
+    // the tiled kernels address a tile's operand rows and the scale rows with 32-bit byte offsets
+    const int64_t max_ld = lda > ldw ? lda : ldw, max_mn = M > N ? M : N;
+    const bool offsets_ok = max_ld < (1 << 22) && (block <= 0 || (K / block + 1) * max_mn * 4 < 0x7fffffffLL);
+    const bool tile_ok = K > 0 && K % kStageK == 0 && lda % 16 == 0 && ldw % 16 == 0 && aligned && offsets_ok &&
+                         (block == 32 || block == 64 || block == 128);
+    if (!tile_ok) return p;
+    if (!partials) {
+        if (M <= 16 && (block == 64 || block == 128) && K / block <= kGemvMaxBlocks) {
+            p.kernel = kKGemv;
+            return p;
+        }
+        if (M <= 32) {
+            p.kernel = kKSkinny;
+            return p;
+        }
+        // 256x256 tiles when there is enough work to fill the 256 CUs with them
+        if ((block == 128 || block == 64) && ((M + 255) / 256) * ((N + 255) / 256) >= kWideMinTiles) {
+            p.kernel = kKWide;
+            return p;
+        }
+    }
+    // 128x128 tiles while they fit one round of workgroups on the 256 CUs; beyond that the 256x128 tile (measured
+    // 25-40 % faster than two rounds of 128x128 tiles at 288-320 of them)
+    const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
+    static_assert(!TileLds<256, 128, 32, 3>::kFits && TileLds<256, 128, 64, 3>::kFits, "block 32 has no 256x128 tile: its stage ring exceeds the LDS");
+    if (M > 128 && t128 > 256 && block != 32) {
+        p.kernel = kKTile256x128;
+        return p;
     }
     // small grids: one workgroup per CU at best, so the tile is spread over as many waves as its shape allows
     // (measured 25-37 % faster than 2x2 waves of 64x64 at M = 96 ... 1024)
-    if constexpr (!PARTIALS) {
-        // few tiles and a caller-provided workspace: split K over several workgroups per tile, then sum the slabs
+    if (!partials && ws_bytes > 0) {
+        // few tiles and scratch memory: split K over several workgroups per tile, then sum the slabs
         int kind;
-        const int sp = plan_split(g.M, g.N, g.K, kind);
-        if (sp > 1 && g.ws && bi8_aligned(g.ws, 16)) {
-            const int64_t nstages = g.K / kStageK;
-            GemmArgs gs = g;
-            gs.split_stages = (int)((nstages + sp - 1) / sp);
-            gs.splits = (int)((nstages + gs.split_stages - 1) / gs.split_stages);      // every split has work
-            if ((int64_t)gs.splits * g.M * g.N * 4 <= g.ws_bytes && gs.splits > 1) {
-                const int rc = kind == 1 ? launch_tile<128, 128, 4, 2, 3, BLK, BI8_F32, false>(gs, st)
-                                         : launch_tile<64, 128, 2, 2, 3, BLK, BI8_F32, false>(gs, st);
-                if (rc != BI8_OK) return rc;
-                const int64_t blocks = (g.M * g.N + 255) / 256;
-                if (blocks > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-                hipLaunchKernelGGL((splitk_reduce<CDT>), dim3((unsigned)blocks), dim3(256), 0, st, gs);
-                return bi8_launch_rc();
+        const int sp = plan_split(M, N, K, kind);
+        if (sp > 1) {
+            const int64_t nstages = K / kStageK;
+            const int stages = (int)((nstages + sp - 1) / sp);
+            const int splits = (int)((nstages + stages - 1) / stages);      // every split has work
+            if (splits > 1 && (int64_t)splits * M * N * 4 <= ws_bytes) {
+                p.kernel = kind == 1 ? kKSplit128x128 : kKSplit64x128;
+                p.splits = splits;
+                p.split_stages = stages;
+                return p;
             }
         }
     }
     // (64x128 tiles for problems of 129-255 tiles of 128x128 measured 5-10 % slower than the half-empty 128x128 grid)
-    if (g.M > 64) return launch_tile<128, 128, 4, 2, 3, BLK, CDT, PARTIALS>(g, st);
-    return launch_tile<64, 128, 2, 2, 3, BLK, CDT, PARTIALS>(g, st);
+    p.kernel = M > 64 ? kKTile128x128 : kKTile64x128;
+    return p;
 }
 
 template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {
@@ -1560,7 +1609,6 @@ template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-constexpr int kGemvMaxBlocks = 512;                // row scales in LDS: 64 bytes per K-block, 32 KiB at most
 template <int BLK, int CDT> int launch_gemv(GemmArgs g, hipStream_t st) {
     const int64_t tn = (g.N + 15) / 16;
     if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
@@ -1569,35 +1617,55 @@ template <int BLK, int CDT> int launch_gemv(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hipStream_t st) {
-    // the tiled kernels address a tile's operand rows and the scale rows with 32-bit byte offsets
-    const int64_t max_ld = g.lda > g.ldw ? g.lda : g.ldw, max_mn = g.M > g.N ? g.M : g.N;
-    const bool offsets_ok = max_ld < (1 << 22) && (block <= 0 || (g.K / block + 1) * max_mn * 4 < 0x7fffffffLL);
-    const bool tile_ok = g.K > 0 && g.K % kStageK == 0 && g.lda % 16 == 0 && g.ldw % 16 == 0 && bi8_aligned(g.A, 16) && bi8_aligned(g.W, 16) &&
-                         (PARTIALS || (bi8_aligned(g.sA, 4) && bi8_aligned(g.sW, 4))) && offsets_ok;
+template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, const GemmPlan &p, hipStream_t st) {
+    constexpr int kRing = 3;                       // stage buffers of the tile kernels that are not software-pipelined
+    switch (p.kernel) {
+    case kKTile256x128:
+        if constexpr (TileLds<256, 128, BLK, kRing>::kFits)
+            return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : kRing, BLK, CDT, PARTIALS>(g, st);
+        break;
+    case kKTile128x128: return launch_tile<128, 128, 4, 2, kRing, BLK, CDT, PARTIALS>(g, st);
+    case kKTile64x128: return launch_tile<64, 128, 2, 2, kRing, BLK, CDT, PARTIALS>(g, st);
+    default: break;
+    }
     if constexpr (!PARTIALS) {
-#ifndef BI8_NO_GEMV
-        if (tile_ok && g.M <= 16 && g.K / block <= kGemvMaxBlocks) {
-            if (block == 64) return launch_gemv<64, CDT>(g, st);
-            if (block == 128) return launch_gemv<128, CDT>(g, st);
+        switch (p.kernel) {
+        case kKGemv:
+            if constexpr (BLK != 32) return launch_gemv<BLK, CDT>(g, st);
+            break;
+        case kKSkinny: return launch_skinny<BLK, CDT>(g, st);
+        case kKWide:
+            if constexpr (BLK != 32) return launch_wide<BLK, CDT>(g, st);
+            break;
+        case kKSplit128x128:
+        case kKSplit64x128: {
+            GemmArgs gs = g;
+            gs.splits = p.splits;
+            gs.split_stages = p.split_stages;
+            const int rc = p.kernel == kKSplit128x128 ? launch_tile<128, 128, 4, 2, kRing, BLK, BI8_F32, false>(gs, st)
+                                                      : launch_tile<64, 128, 2, 2, kRing, BLK, BI8_F32, false>(gs, st);
+            if (rc != BI8_OK) return rc;
+            const int64_t blocks = (g.M * g.N + 255) / 256;
+            if (blocks > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+            hipLaunchKernelGGL((splitk_reduce<CDT>), dim3((unsigned)blocks), dim3(256), 0, st, gs);
+            return bi8_launch_rc();
         }
-#endif
-        if (tile_ok && g.M <= 32) {
-            switch (block) {
-            case 32: return launch_skinny<32, CDT>(g, st);
-            case 64: return launch_skinny<64, CDT>(g, st);
-            case 128: return launch_skinny<128, CDT>(g, st);
-            }
+        default: break;
         }
     }
-    if (tile_ok) {
-        switch (block) {
-        case 32: return pick_tile<32, CDT, PARTIALS>(g, st);
-        case 64: return pick_tile<64, CDT, PARTIALS>(g, st);
-        case 128: return pick_tile<128, CDT, PARTIALS>(g, st);
-        }
+    return BI8_ERR_UNSUPPORTED;                    // plan_gemm never pairs these (kernel, block)
+}
+
+template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hipStream_t st) {
+    const bool aligned = bi8_aligned(g.A, 16) && bi8_aligned(g.W, 16) && (PARTIALS || (bi8_aligned(g.sA, 4) && bi8_aligned(g.sW, 4)));
+    const int64_t ws_bytes = (g.ws && bi8_aligned(g.ws, 16)) ? g.ws_bytes : 0;
+    const GemmPlan p = plan_gemm(g.M, g.N, g.K, g.lda, g.ldw, block, aligned, PARTIALS, ws_bytes);
+    if (p.kernel == kKGeneric) return launch_generic<CDT, PARTIALS>(g, block, st);
+    switch (block) {
+    case 32: return launch_plan<32, CDT, PARTIALS>(g, p, st);
+    case 64: return launch_plan<64, CDT, PARTIALS>(g, p, st);
+    default: return launch_plan<128, CDT, PARTIALS>(g, p, st);
     }
-    return launch_generic<CDT, PARTIALS>(g, block, st);
 }
 
 }  // namespace
@@ -1627,13 +1695,15 @@ extern "C" int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float
 }
 
 extern "C" int64_t bi8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int block) {
-    // mirrors dispatch / pick_tile: only the tile kernels on few tiles split K
-    if (M <= 32 || N <= 0 || K <= 0 || K % kStageK != 0 || (block != 32 && block != 64 && block != 128)) return 0;
-    if ((block == 128 || block == 64) && ((M + 255) / 256) * ((N + 255) / 256) >= kWideMinTiles) return 0;
-    if (M > 128 && ((M + 127) / 128) * ((N + 127) / 128) > 256) return 0;
-    int kind;
-    const int sp = plan_split(M, N, K, kind);
-    return sp > 1 ? (int64_t)sp * M * N * 4 : 0;
+    if (M <= 0 || N <= 0 || K <= 0 || block < 1) return 0;
+    const GemmPlan p = plan_gemm(M, N, K, K, K, block, true, false, INT64_MAX);
+    return p.splits > 1 ? (int64_t)p.splits * M * N * 4 : 0;
+}
+
+extern "C" const char *bi8_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block,
+                                            int64_t workspace_bytes) {
+    if (M <= 0 || N <= 0 || K < 0 || block < 1) return "none";
+    return kGemmKernelNames[plan_gemm(M, N, K, lda, ldw, block, true, false, workspace_bytes).kernel];
 }
 
 template <int DT> int launch_few_rows(const GemmArgs &g, const void *x, int64_t ldx, int block, size_t lds, hipStream_t st) {

@@ -127,6 +127,16 @@ int bi8_gemm_nt_dequant_ws(const int8_t *A, const int8_t *W, const float *sA, co
                            int block, void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Name of the kernel family that bi8_gemm_nt_dequant_ws runs on a problem with 16-byte aligned operands and
+ * `workspace_bytes` of scratch memory ("gemm_wide", "gemm_tile_256x128", "gemm_tile_128x128", "gemm_tile_64x128",
+ * "gemm_tile_128x128_splitk", "gemm_tile_64x128_splitk", "gemm_gemv", "gemm_skinny", "gemm_generic"; "none" for an
+ * empty problem).  Static string.  The reference picks its kernel configuration with Triton's autotuner
+ * (triton_functions.py:41-65) and offers no way to ask which one ran; tests and benchmarks use this to say so.
+ */
+const char *bi8_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block,
+                                 int64_t workspace_bytes);
+
+/*
  * The int32 block partial products of the same kernel, before any scaling (what tl.dot yields at
  * triton_functions.py:115):  P int32 [ceil(K/block), M, N], contiguous.  Parity/debug entry point.
  */

@@ -32,7 +32,7 @@ def test_library_exports_every_declared_symbol():
     assert set(decls) == {"bi8_version", "bi8_strerror", "bi8_quantize_rowwise", "bi8_quantize_transposed",
                           "bi8_dequantize_rowwise", "bi8_gemm_nt_dequant", "bi8_gemm_nt_partials",
                           "bi8_linear_few_rows", "bi8_quantize_dual", "bi8_gemm_nt_dequant_ws",
-                          "bi8_gemm_workspace_bytes"}
+                          "bi8_gemm_workspace_bytes", "bi8_gemm_kernel_name"}
     lib = _lib.load()
     for name in decls:
         assert hasattr(lib, name), f"{name} not exported"
@@ -59,7 +59,7 @@ def test_ctypes_signatures_match_header():
 
 def test_version_and_error_strings():
     lib = _lib.load()
-    assert lib.bi8_version() == _lib.ABI_VERSION == 2
+    assert lib.bi8_version() == _lib.ABI_VERSION == 3
     assert lib.bi8_strerror(0) == b"success"
     assert b"block" in lib.bi8_strerror(3)
     with pytest.raises(_lib.Bi8Error, match="leading dimension"):
@@ -193,3 +193,32 @@ def test_reference_module_names_can_be_aliased():
             compat.install()
     finally:
         del sys.modules["triton_functions"]
+
+
+def test_kernel_choice_by_shape():
+    """the dispatch rule is host arithmetic: which kernel family runs which problem (no GPU call)"""
+    lib = _lib.load()
+    name = lambda M, N, K, block, ws=0, lda=None, ldw=None: lib.bi8_gemm_kernel_name(M, N, K, lda or K, ldw or K, block, ws).decode()
+    assert name(8192, 8192, 8192, 128) == "gemm_wide" and name(8192, 8192, 8192, 64) == "gemm_wide"
+    assert name(8192, 8192, 8192, 32) == "gemm_tile_128x128"         # block 32 has neither 256x256 nor 256x128 tiles
+    assert name(2944, 2944, 512, 128) == "gemm_wide"                 # 12 x 12 = 144 tiles of 256x256
+    assert name(2048, 4096, 4096, 128) == "gemm_tile_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
+    assert name(2048, 2304, 512, 64) == "gemm_tile_256x128"
+    assert name(300, 500, 512, 128) == "gemm_tile_128x128" and name(48, 700, 640, 128) == "gemm_tile_64x128"
+    assert name(1, 4096, 4096, 128) == "gemm_gemv" and name(16, 11008, 4096, 64) == "gemm_gemv"
+    assert name(16, 4096, 4096, 32) == "gemm_skinny" and name(24, 4096, 4096, 128) == "gemm_skinny"
+    assert name(1, 128, 128 * 1024, 128) == "gemm_skinny"            # more K-blocks than the few-row kernel keeps scales for
+    assert name(128, 4096, 4096, 128) == "gemm_tile_128x128"         # no scratch memory: one pass
+    ws = lib.bi8_gemm_workspace_bytes(128, 4096, 4096, 128)
+    assert ws == 4 * 128 * 4096 * 4 and name(128, 4096, 4096, 128, ws) == "gemm_tile_64x128_splitk"
+    assert name(128, 4096, 4096, 128, ws - 1) == "gemm_tile_128x128"     # too small a workspace is not used
+    assert name(512, 4096, 4096, 128, 1 << 30) == "gemm_tile_128x128_splitk"
+    assert name(300, 500, 500, 128) == "gemm_generic" and name(300, 500, 512, 128, 0, 520) == "gemm_generic"
+    assert name(300, 500, 512, 48) == "gemm_generic"
+    assert name(0, 500, 512, 128) == "none"
+    # a split never wants more than 16 MiB: splits x tiles <= 256 tiles of 128 x 128 fp32
+    for M in (33, 64, 100, 128, 256, 512, 1000, 2048):
+        for N in (128, 768, 4096, 11008, 50257):
+            for K in (1024, 4096, 11008 , 8192 * 4):
+                for block in (32, 64, 128):
+                    assert lib.bi8_gemm_workspace_bytes(M, N, K, block) <= 16 << 20, (M, N, K, block)

@@ -1,0 +1,174 @@
+"""The int32 block partials of the kernels that produce the shipped outputs, recovered bit for bit.
+
+bi8_gemm_nt_partials runs its own kernel instantiations; the kernels behind bi8_gemm_nt_dequant (gemm_wide, the
+software-pipelined gemm_tile, gemm_gemv, gemm_skinny, the split of K) and bi8_linear_few_rows fold every partial
+into an fp32 accumulator straight away and never store it.  Here each of them is made to hand a partial back through
+its output: column scales all 1, row scales 1 for ONE K-block j and 0 for every other block, so that
+
+    C[m,n] = fl( P_j[m,n] * fl32(1/127^2) )          (every other block adds exactly 0)
+
+and P_j = round(C * 127^2) exactly: |P_j| <= 128 * 127^2 < 2^21 is an exact fp32 integer through the fold, and the
+one or two roundings that follow move C * 127^2 by less than 0.26.  16-bit outputs keep 8 (bf16) or 11 (fp16)
+significant bits, so those kernels are run on codes in {-1, 0, 1} (|P_j| <= 128, still exact after the cast); a
+mis-routed 16-byte chunk of an operand changes such partials as surely as full-range ones.
+Expected partials come from the CPU checker (the reference's tl.dot, triton_functions.py:115)."""
+import pytest
+import torch
+
+from oracle import oracle_torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import blockwise_int8_linear_amd as pkg
+    from blockwise_int8_linear_amd import _lib
+    _lib.load()
+    return pkg
+
+
+class cfg_as:
+    def __init__(self, ops, block, out):
+        self.cfg, self.block, self.out = ops.block_linear_config, block, out
+
+    def __enter__(self):
+        self.old = (self.cfg.GROUP_SIZE, self.cfg.INPUT_OUTPUT_TORCH_TYPE)
+        self.cfg.GROUP_SIZE, self.cfg.INPUT_OUTPUT_TORCH_TYPE = self.block, self.out
+
+    def __exit__(self, *a):
+        self.cfg.GROUP_SIZE, self.cfg.INPUT_OUTPUT_TORCH_TYPE = self.old
+
+
+def _codes(g, rows, K, full_range):
+    if full_range:
+        c = torch.randint(-127, 128, (rows, K), generator=g, dtype=torch.int32)
+        c[0] = 127                                  # saturated rows: the largest partial there is, +-128 * 127^2
+        c[-1] = -127
+    else:
+        c = torch.randint(-1, 2, (rows, K), generator=g, dtype=torch.int32)
+    return c.to(torch.int8)
+
+
+def _blocks_to_check(nblk):
+    return sorted(set(range(nblk)) if nblk <= 6 else {0, 1, nblk // 2, nblk - 2, nblk - 1})
+
+
+def _kernel(ops, M, N, K, block, ws):
+    from blockwise_int8_linear_amd import _lib
+    return _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, ws).decode()
+
+
+# (M, N, K, block, kernel the shipped operator runs on it)
+CASES = [
+    (2944, 2944, 512, 128, "gemm_wide"),            # 144 tiles of 256x256, four stages
+    (2944, 2900, 384, 128, "gemm_wide"),            # odd number of stages (the loop runs a padding stage), ragged N
+    (2944, 2944, 512, 64, "gemm_wide"),             # two K-blocks per stage
+    (2900, 2944, 384, 64, "gemm_wide"),
+    (2048, 2304, 512, 128, "gemm_tile_256x128"),    # the software-pipelined block-128 instantiation
+    (2000, 2304, 384, 128, "gemm_tile_256x128"),
+    (2048, 2304, 512, 64, "gemm_tile_256x128"),
+    (300, 500, 512, 128, "gemm_tile_128x128"),
+    (300, 500, 512, 32, "gemm_tile_128x128"),
+    (2304, 2304, 256, 32, "gemm_tile_128x128"),
+    (48, 700, 640, 64, "gemm_tile_64x128"),
+    (1, 384, 512, 128, "gemm_gemv"),
+    (16, 1000, 4096, 128, "gemm_gemv"),             # longer than the few-row kernel's register ring
+    (7, 1000, 1152, 64, "gemm_gemv"),
+    (24, 500, 2048, 128, "gemm_skinny"),
+    (16, 300, 1024, 32, "gemm_skinny"),
+    (128, 1024, 4096, 128, "gemm_tile_64x128_splitk"),
+    (512, 4096, 4096, 64, "gemm_tile_128x128_splitk"),
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "x".join(map(str, c[:4])) + "-" + c[4])
+@pytest.mark.parametrize("out", ["f32", "bf16"])
+def test_partials_of_the_shipping_kernels(ops, case, out):
+    from blockwise_int8_linear_amd import _lib
+    M, N, K, block, kernel = case
+    ws = _lib.load().bi8_gemm_workspace_bytes(M, N, K, block)          # what the operator asks for and passes
+    assert _kernel(ops, M, N, K, block, ws) == kernel
+    g = torch.Generator().manual_seed(M + 3 * N + K + block)
+    full = out == "f32"
+    A, W = _codes(g, M, K, full), _codes(g, N, K, full)
+    nblk = K // block
+    P_ref = oracle_torch.gemm_nt_partials(A, W, block)                  # int32 [nblk, M, N]
+    Ad, Wd = A.to(DEV), W.to(DEV)
+    sw = torch.ones(nblk, N, device=DEV)
+    with cfg_as(ops, block, DT[out]):
+        for j in _blocks_to_check(nblk):
+            sa = torch.zeros(nblk, M, device=DEV)
+            sa[j] = 1.0
+            C = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), sa, sw)
+            assert C.dtype == DT[out]
+            got = torch.round(C.double() * (127.0 * 127.0)).to(torch.int32)
+            want = P_ref[j].to(DEV)
+            if not torch.equal(got, want):
+                bad = (got != want).nonzero()
+                m, n = bad[0].tolist()
+                raise AssertionError(f"{kernel}: K-block {j}: {bad.shape[0]} partials differ, first at ({m},{n}): "
+                                     f"got {got[m, n].item()} want {want[m, n].item()}")
+        if full and "splitk" not in kernel:
+            # every scale 1: where the running sums of the partials stay below 2^24 (everywhere but the saturated rows
+            # and columns of a long K) the accumulator holds their exact integer sum, and the output is that sum
+            # times fl32(1/127^2), rounded once
+            exact = P_ref.long().abs().sum(0) < (1 << 24)
+            assert exact.float().mean() > 0.9
+            C = ops.int8_matmul_block64_rowwise_dequantize(Ad, Wd.t(), torch.ones(nblk, M, device=DEV), sw)
+            want = P_ref.sum(0).float() * torch.tensor(1.0 / (127.0 * 127.0), dtype=torch.float32)
+            assert torch.equal(C.cpu()[exact], want[exact])
+
+
+@pytest.mark.parametrize("case", CASES[:2] + CASES[4:5], ids=lambda c: "x".join(map(str, c[:4])) + "-" + c[4])
+def test_partials_of_the_f16_instantiations(ops, case):
+    M, N, K, block, kernel = case
+    g = torch.Generator().manual_seed(K + block)
+    A, W = _codes(g, M, K, False), _codes(g, N, K, False)
+    nblk = K // block
+    P_ref = oracle_torch.gemm_nt_partials(A, W, block)
+    sw = torch.ones(nblk, N, device=DEV)
+    with cfg_as(ops, block, torch.float16):
+        j = nblk - 1
+        sa = torch.zeros(nblk, M, device=DEV)
+        sa[j] = 1.0
+        C = ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa, sw)
+        assert torch.equal(torch.round(C.double() * (127.0 * 127.0)).to(torch.int32).cpu(), P_ref[j])
+
+
+@pytest.mark.parametrize("block", [64, 128])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("M", [1, 4])
+def test_partials_of_the_one_launch_decode_linear(ops, block, dtype, M):
+    """bi8_linear_few_rows quantizes x itself, so x is built to quantize to known codes: integers in one K-block j
+    with a +-127 among them (scale 127, codes = the integers), zeros elsewhere (scale 0, codes 0).  Then
+    C = fl(fl(127 * P_j) * fl32(1/127^2)) with column scales 1."""
+    N, K = 700, 2048
+    nblk = K // block
+    g = torch.Generator().manual_seed(block + M)
+    full = dtype == "f32"
+    W = _codes(g, N, K, False)                                          # |127 * P_j| stays below 2^24
+    for j in _blocks_to_check(nblk)[:4]:
+        codes = torch.zeros(M, K, dtype=torch.int32)
+        if full:
+            codes[:, j * block:(j + 1) * block] = torch.randint(-127, 128, (M, block), generator=g, dtype=torch.int32)
+        else:
+            codes[:, j * block:j * block + 48] = torch.randint(-1, 2, (M, 48), generator=g, dtype=torch.int32)
+        codes[:, j * block + 5] = 127
+        x = codes.to(DT[dtype])
+        assert torch.equal(x.to(torch.int32), codes)
+        P_ref = oracle_torch.gemm_nt_partials(codes.to(torch.int8), W, block)[j]
+        if not full:
+            assert P_ref.abs().max() < 256
+        with cfg_as(ops, block, DT[dtype]):
+            C = ops.linear_few_rows(x.to(DEV), W.to(DEV), torch.ones(nblk, N, device=DEV))
+            assert C is not None, "the fused kernel covers this case"
+            # the same through the two launches: identical bits
+            xq, sx = ops.quantize_block_rowwise(x.to(DEV))
+            assert torch.equal(xq.cpu().to(torch.int32), codes) and (sx[j] == 127).all() and sx.sum() == 127 * M
+            C2 = ops.int8_matmul_block64_rowwise_dequantize(xq, W.to(DEV).t(), sx, torch.ones(nblk, N, device=DEV))
+        assert torch.equal(C, C2)
+        got = torch.round(C.double() * (127.0 * 127.0) / 127.0).to(torch.int32).cpu()
+        assert torch.equal(got, P_ref)
