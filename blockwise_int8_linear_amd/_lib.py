@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbi8.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "bi8.h")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _i64, _vp, _ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
 
@@ -26,6 +26,8 @@ SIGNATURES = {
     "bi8_gemm_nt_dequant": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_gemm_nt_dequant_ws": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp, _i64, _vp]),
     "bi8_gemm_workspace_bytes": (_i64, [_i64, _i64, _i64, _ci]),
+    "bi8_static_scratch_bytes": (_i64, []),
+    "bi8_gemm_nt_dequant_static": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_gemm_kernel_name": (ctypes.c_char_p, [_i64, _i64, _i64, _i64, _i64, _ci, _i64]),
     "bi8_gemm_nt_partials": (_ci, [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_linear_few_rows": (_ci, [_vp, _ci, _vp, _vp, _vp, _ci, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),

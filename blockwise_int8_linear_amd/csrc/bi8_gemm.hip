@@ -1694,6 +1694,54 @@ extern "C" int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float
     return bi8_gemm_nt_dequant_ws(A, W, sA, sW, bias, bias_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, block, nullptr, 0, stream);
 }
 
+// ---- the entry point that allocates nothing ---------------------------------------------------------------------------
+// The split of K needs scratch memory for its fp32 slabs.  bi8_gemm_nt_dequant_ws takes it from the caller;
+// bi8_gemm_nt_dequant_static takes it from this array, one copy per GPU that loads the library, for callers that cannot
+// allocate (HIP graph capture, serving loops, harnesses that forbid hipMalloc).  A split never wants more than
+// splits x tiles <= 256 tiles of 128 x 128 fp32 = 16 MiB (plan_split), which is the size of the array.
+constexpr int64_t kScratchBytes = 16ll << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+// In host code `scratch` is only a handle for the runtime: the array's address on the current device comes from
+// hipGetSymbolAddress, once per device, and is what the kernels are given.
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> scratch_ptr[kMaxDevices];
+static int scratch_of_current_device(void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return bi8_hip_rc(e);
+    if (dev < 0 || dev >= kMaxDevices) return BI8_ERR_UNSUPPORTED;
+    void *p = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return bi8_hip_rc(e);
+        if (!p) return BI8_ERR_NULL_POINTER;
+        scratch_ptr[dev].store(p, std::memory_order_release);       // two threads racing here store the same address
+    }
+    *out = p;
+    return BI8_OK;
+}
+
+extern "C" int64_t bi8_static_scratch_bytes(void) { return kScratchBytes; }
+
+extern "C" int bi8_gemm_nt_dequant_static(const int8_t *A, const int8_t *W, const float *sA, const float *sW, const void *bias,
+                                          int bias_dtype, void *C, int c_dtype, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                          int64_t ldw, int64_t ldc, int block, void *stream) {
+    if (block < 1 || block > (1 << 20)) return BI8_ERR_BAD_BLOCK;
+    if (M < 0 || N < 0 || K < 0 || lda < K || ldw < K || ldc < N) return BI8_ERR_BAD_SHAPE;
+    // what the split of this problem wants, were scratch memory unlimited; more than the array holds is refused
+    // rather than run differently from bi8_gemm_nt_dequant_ws
+    const GemmPlan p = plan_gemm(M, N, K, lda, ldw, block, true, false, INT64_MAX);
+    if (p.splits > 1 && (int64_t)p.splits * M * N * 4 > kScratchBytes) return BI8_ERR_SCRATCH_TOO_SMALL;
+    void *ws = nullptr;
+    if (p.splits > 1) {
+        const int rc = scratch_of_current_device(&ws);
+        if (rc != BI8_OK) return rc;
+    }
+    return bi8_gemm_nt_dequant_ws(A, W, sA, sW, bias, bias_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, block, ws, ws ? kScratchBytes : 0,
+                                  stream);
+}
+
 extern "C" int64_t bi8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int block) {
     if (M <= 0 || N <= 0 || K <= 0 || block < 1) return 0;
     const GemmPlan p = plan_gemm(M, N, K, K, K, block, true, false, INT64_MAX);

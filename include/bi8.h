@@ -42,6 +42,7 @@ extern "C" {
 #define BI8_ERR_BAD_SHAPE 4   /* negative size, or a leading dimension smaller than the row length */
 #define BI8_ERR_TOO_LARGE 5   /* a dimension exceeds what one launch can index */
 #define BI8_ERR_UNSUPPORTED 6 /* valid arguments outside what this entry point covers; nothing was launched */
+#define BI8_ERR_SCRATCH_TOO_SMALL 7 /* the problem wants more scratch memory than the library's static buffer holds */
 #define BI8_ERR_HIP_BASE 1000 /* BI8_ERR_HIP_BASE + hipError_t */
 
 /* ABI version of this header (bumped on any signature change). */
@@ -125,6 +126,26 @@ int bi8_gemm_nt_dequant_ws(const int8_t *A, const int8_t *W, const float *sA, co
                            const void *bias, int bias_dtype, void *C, int c_dtype,
                            int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
                            int block, void *workspace, int64_t workspace_bytes, void *stream);
+
+/*
+ * bi8_gemm_nt_dequant_ws WITHOUT a workspace argument and without any allocation: the fp32 slabs of a split of K go
+ * to a static array in device memory that belongs to the library (bi8_static_scratch_bytes() = 16 MiB on every GPU
+ * the library runs on, held until the process ends).  No counterpart in the reference: it is for callers that
+ * cannot allocate -- code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The call
+ * makes no hipMalloc / hipFree and no allocating library call; the first call on a device looks up the array's
+ * address there (hipGetSymbolAddress), so make one call on each device outside any capture.
+ * Same kernels, same results (bit for bit) as bi8_gemm_nt_dequant_ws given bi8_gemm_workspace_bytes() of workspace.
+ * A problem whose split wants more than the array holds returns BI8_ERR_SCRATCH_TOO_SMALL and launches nothing (with
+ * the present split rule -- at most 256 slabs of 128 x 128 fp32 -- no problem does).
+ * All calls on one GPU share the array, which keeps the last call's contents (every call overwrites what it reads,
+ * nothing has to start at zero): calls that overlap on one GPU -- two streams, two host threads -- race on it.
+ * Serialize them on one stream, or give the overlapping ones their own workspace through bi8_gemm_nt_dequant_ws.
+ */
+int64_t bi8_static_scratch_bytes(void);
+int bi8_gemm_nt_dequant_static(const int8_t *A, const int8_t *W, const float *sA, const float *sW,
+                               const void *bias, int bias_dtype, void *C, int c_dtype,
+                               int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int64_t ldc,
+                               int block, void *stream);
 
 /*
  * Name of the kernel family that bi8_gemm_nt_dequant_ws runs on a problem with 16-byte aligned operands and

@@ -32,7 +32,8 @@ def test_library_exports_every_declared_symbol():
     assert set(decls) == {"bi8_version", "bi8_strerror", "bi8_quantize_rowwise", "bi8_quantize_transposed",
                           "bi8_dequantize_rowwise", "bi8_gemm_nt_dequant", "bi8_gemm_nt_partials",
                           "bi8_linear_few_rows", "bi8_quantize_dual", "bi8_gemm_nt_dequant_ws",
-                          "bi8_gemm_workspace_bytes", "bi8_gemm_kernel_name"}
+                          "bi8_gemm_workspace_bytes", "bi8_gemm_kernel_name", "bi8_static_scratch_bytes",
+                          "bi8_gemm_nt_dequant_static"}
     lib = _lib.load()
     for name in decls:
         assert hasattr(lib, name), f"{name} not exported"
@@ -59,7 +60,7 @@ def test_ctypes_signatures_match_header():
 
 def test_version_and_error_strings():
     lib = _lib.load()
-    assert lib.bi8_version() == _lib.ABI_VERSION == 3
+    assert lib.bi8_version() == _lib.ABI_VERSION == 4
     assert lib.bi8_strerror(0) == b"success"
     assert b"block" in lib.bi8_strerror(3)
     with pytest.raises(_lib.Bi8Error, match="leading dimension"):
