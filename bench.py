@@ -23,12 +23,17 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-INT8_PEAK_TOPS = 5033.2        # 256 CUs x 8192 int8 ops/clk/CU x 2.4 GHz (AMD quotes 5.0 POP/s dense)
+INT8_PEAK_TOPS = 5000.0        # MI355X, dense int8 MFMA, as published (256 CUs x 8192 ops/clk/CU x 2.4 GHz = 5033)
 HBM_PEAK_GBS = 8000.0          # HBM3E, 8 TB/s
 # Bytes that cross the L2 <-> fabric boundary in one 8192^3 block-128 launch of the headline kernel: FETCH_SIZE and
 # WRITE_SIZE of rocprofv3 --pmc runs of this file, scaled by what the same counters read for a 256 MiB copy
-# (x2.0 and x1.0); the runs and figures are in profiles/gemm_wide_8192x8192x8192_block128.md.  Not measured live.
+# (x2.0 and x1.0); the runs and figures are in profiles/gemm_wide_8192x8192x8192_block128.md.  Counters cannot be read
+# from inside the process, so this is a constant from those runs, labelled as such in the output ("traffic_source").
 GEMM_8192_TRAFFIC_BYTES = 980817527
+GEMM_8192_TRAFFIC_SOURCE = ("profiles/gemm_wide_8192x8192x8192_block128.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
+                            "command, scaled by a 256 MiB copy; a constant, not measured in this run")
+PREROLL_MAX = 400              # launches
+PREROLL_BATCH = 10
 
 
 def event_ms(fn, iters: int) -> float:
@@ -41,6 +46,19 @@ def event_ms(fn, iters: int) -> float:
     stop.record()
     stop.synchronize()
     return start.elapsed_time(stop) / iters
+
+
+def preroll(fn, torch):
+    """Untimed launches until the chip's clocks have settled: after idle the first launches run at ramping clocks (up
+    to 30 % slower, for about a hundred launches).  Batches of PREROLL_BATCH launches are timed with events until three
+    batches in a row agree within 0.7 %, at most PREROLL_MAX launches.  Returns (launches made, ms per launch of the last batch)."""
+    done, hist = 0, []
+    while done < PREROLL_MAX:
+        hist.append(event_ms(fn, PREROLL_BATCH))
+        done += PREROLL_BATCH
+        if len(hist) >= 3 and max(hist[-3:]) <= 1.007 * min(hist[-3:]):
+            break
+    return done, hist[-1]
 
 
 def bench_quantize(pkg, torch, iters: int):
@@ -253,6 +271,8 @@ def main():
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the GEMM (the metric is quoted at 8192)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-quantize", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the secondary figures (their small launches share kernel names with the round trip)")
+    ap.add_argument("--no-preroll", action="store_true", help="skip the untimed launches that let the clocks settle before the warm-up")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 256 MiB device-to-device copy 5 times (a kernel of known traffic, for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -292,23 +312,31 @@ def main():
     def step():
         return pkg.int8_matmul_block64_rowwise_dequantize(xq, wqt, sx, sw)
 
+    step()
+    torch.cuda.synchronize()
+    preroll_launches, preroll_ms = (0, None) if args.no_preroll else preroll(step, torch)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     # the timed region: exactly `steps` launches, wall clock between two synchronizations, and HIP events on the
-    # stream the kernel runs on (torch's current stream) around the same launches for the kernel's average duration
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # stream the kernel runs on (torch's current stream) before the first and after every launch: the kernel's
+    # average duration is (last - first) / steps, the per-launch durations give the median
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(args.steps):
+    evs[0].record()
+    for i in range(args.steps):
         step()
-    ev1.record()
+        evs[i + 1].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
     ops_per_launch = 2.0 * S * S * S
-    kern_ms = ev0.elapsed_time(ev1) / args.steps
+    kern_ms = evs[0].elapsed_time(evs[-1]) / args.steps
+    per_launch = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
+    median_ms = per_launch[len(per_launch) // 2] if len(per_launch) % 2 else 0.5 * (per_launch[len(per_launch) // 2 - 1] + per_launch[len(per_launch) // 2])
     achieved = ops_per_launch / kern_ms / 1e9       # TOPS
+    lib = _lib.load()
+    kernel = lib.bi8_gemm_kernel_name(S, S, S, S, S, B, lib.bi8_gemm_workspace_bytes(S, S, S, B)).decode()
 
     res = {
         "metric": "int8 block GEMM TOPS (% int8 MFMA peak) at 8192^3; quantize GB/s (% HBM)",
@@ -323,11 +351,15 @@ def main():
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": round(achieved / INT8_PEAK_TOPS, 4),
                      "traffic": GEMM_8192_TRAFFIC_BYTES if (S == 8192 and B == 128) else None,
-                     "kernel": "gemm_wide<128,bf16> (256x256 tile, 8 waves of 64x128, 2 LDS stage buffers, v_mfma_i32_16x16x64_i8)", "ops_per_launch": ops_per_launch,
-                     "avg_launch_ms": round(kern_ms, 4)},
+                     "traffic_source": GEMM_8192_TRAFFIC_SOURCE if (S == 8192 and B == 128) else None,
+                     "kernel": f"{kernel}<{B},bf16> (the library's choice for this shape: bi8_gemm_kernel_name)",
+                     "ops_per_launch": ops_per_launch, "avg_launch_ms": round(kern_ms, 4), "median_launch_ms": round(median_ms, 4),
+                     "frac_of_5033_TOPs_at_2p4GHz": round(achieved / 5033.2, 4),
+                     "preroll_launches": preroll_launches, "preroll_last_batch_ms": None if preroll_ms is None else round(preroll_ms, 4)},
     }
     if not args.no_quantize:
         res["quantize_roundtrip"] = bench_quantize(pkg, torch, 50)
+    if not args.no_quantize and not args.no_extras:
         res["extras"] = bench_extras(pkg, torch)
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(torch, xq.cpu(), wq.cpu(), sx.cpu(), sw.cpu(), B)
