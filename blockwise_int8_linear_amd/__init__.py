@@ -5,7 +5,10 @@ from .block_linear import (
     BlockInt8Linear,
     BlockLinear,
     blockwise_int8_linear,
+    blockwise_int8_linear_Wint8,
+    quantize_weight_for_training,
     replace_linear_with_blockwise_int8,
+    replace_linear_with_blockwise_int8_recursive,
 )
 from .ops import (
     dequantize_block_rowwise,
@@ -19,6 +22,7 @@ from .ops import (
 
 __all__ = [
     "block_linear_config", "BlockInt8Linear", "BlockLinear", "blockwise_int8_linear",
+    "blockwise_int8_linear_Wint8", "quantize_weight_for_training", "replace_linear_with_blockwise_int8_recursive",
     "replace_linear_with_blockwise_int8", "quantize_block_rowwise", "quantize_block_transposed",
     "dequantize_block_rowwise", "int8_matmul_block64_rowwise_dequantize", "int8_matmul_block_partials",
     "linear_few_rows", "quantize_block_dual",

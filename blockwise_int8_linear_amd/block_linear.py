@@ -10,7 +10,11 @@ Differences from the reference that do not change results:
   * switching the module back to training mode drops the cached int8 weights, so a later ``eval()``
     re-quantizes the current weights (the reference keeps serving the first cache, block_linear.py:138-139);
   * the eval path with at most 4 rows (token-by-token decode) quantizes and multiplies in one kernel
-    (block_linear.py:141-144 are two launches).
+    (block_linear.py:141-144 are two launches);
+  * ``blockwise_int8_linear_Wint8`` is the working form of the reference's function of that name
+    (block_linear.py:42-67, which passes un-quantized activations to the GEMM and multiplies the gradient with weight
+    codes blocked along the wrong dimension): the forward pass runs on weight codes quantized ahead of time, the
+    grad-input GEMM on a second copy of the weights quantized along the output features.
 """
 from __future__ import annotations
 
@@ -28,6 +32,12 @@ from .ops import (
     quantize_block_rowwise,
     quantize_block_transposed,
 )
+
+
+def replace_linear_with_blockwise_int8_recursive(model):
+    """``replace_linear_with_blockwise_int8`` applied to `model` and to every module below it: every ``nn.Linear``
+    of the tree becomes a ``BlockInt8Linear`` (the reference's helper handles one level, block_linear.py:18)."""
+    return model.apply(replace_linear_with_blockwise_int8)
 
 
 def replace_linear_with_blockwise_int8(model):
@@ -103,6 +113,65 @@ class blockwise_int8_linear(torch.autograd.Function):
         return grad_X, grad_W, grad_bias
 
 
+def quantize_weight_for_training(W):
+    """Both quantized copies of a weight W [N,K] that a training step multiplies with:
+    (W_int8 [N,K], state_W [ceil(K/B),N]) blocked along the input features for the forward GEMM (block_linear.py:79),
+    (Wt_int8 [K,N], Wt_state [ceil(N/B),K]) blocked along the output features for the grad-input GEMM (:93-94), from one
+    read of W.  Wt_int8 is a view of rows padded with zero codes to a multiple of 128 (returned last), which is what
+    the tiled GEMM kernels want of a contraction dimension such as a 50257-word vocabulary."""
+    W_int8, state_W, Wt_int8, Wt_state, _, Wt_store = _quantize_block_dual(W.detach(), block_linear_config.GROUP_SIZE, pad=True)
+    return W_int8, state_W, Wt_int8, Wt_state, Wt_store
+
+
+class blockwise_int8_linear_Wint8(torch.autograd.Function):
+    """y = x @ W.T + bias on weights quantized AHEAD of the call (what block_linear.py:42-67 set out to be).
+
+    ``apply(x, W_int8, state_W, bias, Wt_int8, Wt_state, weight=None, Wt_store=None)``:
+      W_int8 [N,K], state_W [K/B,N]    the weight blocked along K: forward GEMM, as in BlockInt8Linear.infer;
+      Wt_int8 [K,N], Wt_state [N/B,K]  the weight transposed and blocked along N: grad_X = G @ W contracts over N;
+      weight                           optional float tensor that stands for W in the autograd graph: it receives
+                                       grad_W = G.T @ X (block_linear.py:100-104) and is not read;
+      Wt_store                         optional zero-padded buffer that Wt_int8 is a view of (quantize_weight_for_training).
+    The first four arguments are the reference's; with the copies made by ``quantize_weight_for_training(W)`` the outputs
+    and gradients are bit for bit those of ``blockwise_int8_linear.apply(x, W, bias)``, without quantizing W in the step."""
+
+    @staticmethod
+    def forward(ctx, X_3D, W_int8, state_W, bias, Wt_int8, Wt_state, weight=None, Wt_store=None):
+        X = X_3D.reshape(-1, X_3D.size(-1))
+        need_gw = weight is not None and ctx.needs_input_grad[6]
+        if need_gw:
+            X_int8, state_X, Xt_int8, Xt_state = quantize_block_dual(X)         # [M,K] and [K,M], [M/B,K]
+        else:
+            X_int8, state_X = quantize_block_rowwise(X)
+            Xt_int8 = Xt_state = None
+        ctx.save_for_backward(Xt_int8, Xt_state, Wt_int8, Wt_state, Wt_store)
+        out = int8_matmul_block64_rowwise_dequantize(X_int8, W_int8.t(), state_X, state_W, bias)
+        return out.view(*X_3D.size()[:-1], -1)
+
+    @staticmethod
+    def backward(ctx, G_3D):
+        G = G_3D.reshape(-1, G_3D.size(-1))
+        grad_X = grad_W = grad_bias = None
+        Xt_int8, Xt_state, Wt_int8, Wt_state, Wt_store = ctx.saved_tensors
+        need_gx, need_gw = ctx.needs_input_grad[0], Xt_int8 is not None
+        g_store = None
+        if need_gx and need_gw:
+            g_int8, g_state, gt_int8, gt_state, g_store, _ = _quantize_block_dual(G, block_linear_config.GROUP_SIZE, pad=True)
+        elif need_gx:
+            g_int8, g_state = quantize_block_rowwise(G)
+        elif need_gw:
+            gt_int8, gt_state = quantize_block_transposed(G)                    # [N,M], [M/B,N]
+        if need_gx:
+            grad_X = _int8_matmul(g_int8, Wt_int8.t(), g_state, Wt_state, None, g_store, Wt_store)
+            grad_X = grad_X.view(*G_3D.size()[:-1], -1)
+        if need_gw:
+            grad_W = int8_matmul_block64_rowwise_dequantize(gt_int8, Xt_int8.t(), gt_state, Xt_state)
+        if ctx.needs_input_grad[3]:
+            grad_bias = G.sum(dim=0)
+        # one entry per argument that apply() was given (the last two are optional)
+        return (grad_X, None, None, grad_bias, None, None, grad_W, None)[:len(ctx.needs_input_grad)]
+
+
 class BlockInt8Linear(nn.Linear):
     """``nn.Linear`` replacement (block_linear.py:114-152).  Training mode: ``blockwise_int8_linear``.
     Eval mode: weights quantized once into the buffers ``W_int8`` [N,K] int8 and ``state_W``
@@ -110,11 +179,27 @@ class BlockInt8Linear(nn.Linear):
 
     def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None):
         super().__init__(in_features, out_features, bias, device, dtype)
+        # training on weight codes quantized ahead of the step (blockwise_int8_linear_Wint8): the codes are made when
+        # the weight has changed since they were last made (frozen weights, several micro-batches per optimizer step:
+        # once), not in every forward and again in every backward pass
+        self.quantized_weight_training = False
+        self._train_cache = None
+        self._eval_cache_of = None                 # state of the weight the eval cache was quantized from
+
+    def _weight_state(self):
+        """changes whenever the weight's values may have: in-place updates bump the version, assignments move the data"""
+        w = self.weight
+        return (w._version, w.data_ptr(), block_linear_config.GROUP_SIZE)
 
     def prepare_for_eval(self):
         W_int8, state_W = quantize_block_rowwise(self.weight.detach())
         self.register_buffer("W_int8", W_int8)
         self.register_buffer("state_W", state_W)
+        self._eval_cache_of = self._weight_state()
+
+    def prepare_for_quantized_weight_training(self):
+        """(re)make the two quantized copies of the weight that ``blockwise_int8_linear_Wint8`` multiplies with"""
+        self._train_cache = (self._weight_state(),) + quantize_weight_for_training(self.weight)
 
     def weight_quant_training(self, x=None):
         """Replace the weight by its quantize->dequantize image (block_linear.py:130-135).  As in the
@@ -124,7 +209,9 @@ class BlockInt8Linear(nn.Linear):
         self.weight = dequantize_block_rowwise(W_int8, state_W)
 
     def infer(self, x):
-        if getattr(self, "W_int8", None) is None:
+        # quantize the weight on first use (block_linear.py:138-139) and again when it has changed since: the reference
+        # keeps serving the first cache
+        if getattr(self, "W_int8", None) is None or self._eval_cache_of != self._weight_state():
             self.prepare_for_eval()
         X = x.reshape(-1, x.size(-1))
         out = None
@@ -140,6 +227,11 @@ class BlockInt8Linear(nn.Linear):
     def forward(self, x):
         if not self.training:
             return self.infer(x)
+        if self.quantized_weight_training:
+            if self._train_cache is None or self._train_cache[0] != self._weight_state():
+                self.prepare_for_quantized_weight_training()
+            _, W_int8, state_W, Wt_int8, Wt_state, Wt_store = self._train_cache
+            return blockwise_int8_linear_Wint8.apply(x, W_int8, state_W, self.bias, Wt_int8, Wt_state, self.weight, Wt_store)
         return blockwise_int8_linear.apply(x, self.weight, self.bias)
 
     def train(self, mode: bool = True):
@@ -154,6 +246,9 @@ class BlockInt8Linear(nn.Linear):
             if prefix + name in state_dict and name not in self._buffers:
                 self.register_buffer(name, torch.empty_like(state_dict[prefix + name], device=self.weight.device))
         super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+        if prefix + "W_int8" in state_dict:
+            # the checkpoint's codes go with the checkpoint's weight, or stand alone in a checkpoint of codes only
+            self._eval_cache_of = self._weight_state()
 
 
 BlockLinear = BlockInt8Linear

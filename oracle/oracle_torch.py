@@ -11,6 +11,7 @@ IEEE binary32 sequence as the C file's.
     gemm_nt_partials                  triton_functions.py:115
     int8_matmul_block_dequantize      triton_functions.py:106-131, :142-168
     linear_forward / linear_backward  block_linear.py:71-80, :83-112
+    linear_wint8_forward / _backward  block_linear.py:42-67 as intended (see the functions)
 
 NaN inputs are outside this file's domain (``amax`` propagates them; the C checker ignores them).
 """
@@ -98,4 +99,29 @@ def linear_backward(G3, x, W, block: int, out_dtype=torch.bfloat16, has_bias=Tru
     gtq, gts = quantize_block_rowwise(G.t().contiguous(), block)            # :101, :103
     grad_W = int8_matmul_block_dequantize(gtq, xtq, gts, xts, block, None, out_dtype)  # :104
     grad_b = G.sum(dim=0) if has_bias else None                 # :110
+    return grad_X.reshape(*x.shape), grad_W, grad_b
+
+
+def linear_wint8_forward(x, wq, sw, bias, block: int, out_dtype=torch.bfloat16):
+    """The forward pass block_linear.py:43-47 set out to be: the weight arrives quantized along K (wq int8 [N,K],
+    sw [nblk,N]), the activations are quantized here (the reference's line :47 forgets to, and so passes its
+    arguments one position off), one GEMM."""
+    X = x.reshape(-1, x.shape[-1])                              # :45
+    xq, sx = quantize_block_rowwise(X, block)
+    out = int8_matmul_block_dequantize(xq, wq, sx, sw, block, bias, out_dtype)   # :47
+    return out.reshape(*x.shape[:-1], -1)
+
+
+def linear_wint8_backward(G3, x, wtq, wts, block: int, out_dtype=torch.bfloat16, has_bias=True):
+    """The backward pass block_linear.py:49-67 set out to be.  grad_X = G @ W contracts over the output features, so
+    it needs the weight quantized along N: wtq int8 [K,N], wts [ceil(N/block), K] (the reference's line :57 multiplies
+    with the K-blocked codes and their scales, which have the wrong shape for that).  grad_W and grad_bias as :58-65."""
+    G = G3.reshape(-1, G3.shape[-1])                            # :51
+    X = x.reshape(-1, x.shape[-1])
+    gq, gs = quantize_block_rowwise(G, block)                   # :56
+    grad_X = int8_matmul_block_dequantize(gq, wtq, gs, wts, block, None, out_dtype)     # :57, on the N-blocked copy
+    xtq, xts = quantize_block_rowwise(X.t().contiguous(), block)            # :59, :61
+    gtq, gts = quantize_block_rowwise(G.t().contiguous(), block)            # :60, :62
+    grad_W = int8_matmul_block_dequantize(gtq, xtq, gts, xts, block, None, out_dtype)   # :63
+    grad_b = G.sum(dim=0) if has_bias else None                 # :65
     return grad_X.reshape(*x.shape), grad_W, grad_b

@@ -140,6 +140,14 @@ def test_model_surgery_on_cpu_modules():
     assert set(net.a.state_dict()) == {"weight", "bias"}
     net.apply(pkg.replace_linear_with_blockwise_int8)
     assert isinstance(net.seq[0], pkg.BlockInt8Linear)
+    # the helper that recurses by itself: every level, same storage, training flags kept
+    net2 = nn.Sequential(nn.Linear(8, 8), nn.Sequential(nn.Linear(8, 8), nn.ReLU(), nn.Sequential(nn.Linear(8, 4, bias=False))))
+    ptrs = [p.data_ptr() for p in net2.parameters()]
+    assert pkg.replace_linear_with_blockwise_int8_recursive(net2) is net2
+    lins = [m for m in net2.modules() if isinstance(m, nn.Linear)]
+    assert len(lins) == 3 and all(isinstance(m, pkg.BlockInt8Linear) and m.training for m in lins)
+    assert [p.data_ptr() for p in net2.parameters()] == ptrs and lins[2].bias is None
+    assert not lins[0].quantized_weight_training
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

@@ -131,3 +131,56 @@ def test_backward_wiring_against_dense_algebra():
     assert (gX.reshape(-1, 128) - G2 @ W).norm() / (G2 @ W).norm() < 3e-2
     assert (gW - G2.t() @ X2).norm() / (G2.t() @ X2).norm() < 3e-2
     assert torch.equal(gb, G2.sum(0))
+
+
+def _lossless(g, rows, cols, block, scale):
+    """integers in [-127,127] times a power of two, +-127 somewhere in every block of every row: block quantization
+    is lossless on it (scale 127 * 2^e, codes = the integers), so the quantized products ARE the dense products"""
+    t = torch.randint(-127, 128, (rows, cols), generator=g, dtype=torch.int32).float()
+    t[:, ::block] = 127.0
+    t[::2, ::block] = -127.0
+    return t * scale
+
+
+def test_weight_only_training_functions_against_dense_algebra():
+    """linear_wint8_forward / _backward (what block_linear.py:42-67 set out to be), pinned three ways: with the two
+    quantized copies made from W they are linear_forward / linear_backward bit for bit; on data that block
+    quantization represents exactly they equal the DENSE products G @ W, G.T @ X, X @ W.T to fp32 rounding (a
+    transposed operand, scales of the other copy or blocks along the wrong dimension miss by O(1)); and grad_X does
+    change when it is given the K-blocked copy's scales instead (the reference's mistake at :57)."""
+    g = torch.Generator().manual_seed(11)
+    B, M, K, N = 32, 96, 128, 64
+    x = torch.randn(2, M // 2, K, generator=g); W = torch.randn(N, K, generator=g) * 0.05
+    G = torch.randn(2, M // 2, N, generator=g); bias = torch.randn(N, generator=g)
+    wq, sw = oracle_torch.quantize_block_rowwise(W, B)
+    wtq, wts = oracle_torch.quantize_block_rowwise(W.t().contiguous(), B)
+    for od in (torch.float32, torch.bfloat16):
+        assert torch.equal(oracle_torch.linear_wint8_forward(x, wq, sw, bias, B, od), oracle_torch.linear_forward(x, W, bias, B, od))
+        a = oracle_torch.linear_wint8_backward(G, x, wtq, wts, B, od)
+        b = oracle_torch.linear_backward(G, x, W, B, od)
+        assert all(torch.equal(u, v) for u, v in zip(a, b))
+    # lossless data, N != K and M != N so that no transposition goes unnoticed
+    X = _lossless(g, M, K, B, 0.25); Wl = _lossless(g, N, K, B, 2.0 ** -9)
+    X[:, ::B] = 127 * 0.25; X[::3, ::B] = -127 * 0.25
+    Gl = _lossless(g, M, N, B, 0.5)
+    # ... also along the other direction: every column block of B rows holds a +-127 too
+    for t, s in ((X, 0.25), (Wl, 2.0 ** -9), (Gl, 0.5)):
+        t[::B, :] = 127 * s
+    wq, sw = oracle_torch.quantize_block_rowwise(Wl, B)
+    wtq, wts = oracle_torch.quantize_block_rowwise(Wl.t().contiguous(), B)
+    assert torch.equal(wq.float() * (2.0 ** -9), Wl) and (sw == 127 * 2.0 ** -9).all() and torch.equal(wtq, wq.t())
+    y = oracle_torch.linear_wint8_forward(X, wq, sw, None, B, torch.float32)
+    gX, gW, gb = oracle_torch.linear_wint8_backward(Gl, X, wtq, wts, B, torch.float32)
+    for got, dense in ((y, X.double() @ Wl.double().t()), (gX, Gl.double() @ Wl.double()), (gW, Gl.double().t() @ X.double())):
+        assert got.shape == dense.shape
+        assert ((got.double() - dense).abs() <= 2e-6 * dense.abs() + 1e-6 * dense.abs().max()).all()
+    assert torch.equal(gb, Gl.sum(0))
+    # the reference's line :57 (K-blocked codes and scales in the grad-input GEMM) is a different function
+    W2 = torch.randn(K, K, generator=g) * 0.05                     # square, so that the shapes allow the mistake
+    G2 = torch.randn(M, K, generator=g)
+    wq2, sw2 = oracle_torch.quantize_block_rowwise(W2, B)
+    wtq2, wts2 = oracle_torch.quantize_block_rowwise(W2.t().contiguous(), B)
+    right, _, _ = oracle_torch.linear_wint8_backward(G2, X, wtq2, wts2, B, torch.float32)
+    wrong, _, _ = oracle_torch.linear_wint8_backward(G2, X, wq2, sw2, B, torch.float32)
+    dense = G2 @ W2
+    assert (right - dense).norm() / dense.norm() < 3e-2 < (wrong - dense).norm() / dense.norm()

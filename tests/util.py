@@ -84,11 +84,15 @@ def assert_close_rms(got, ref, tol, bias=None):
     """elementwise |got - ref| <= tol * (|ref| + |bias|) + 3e-4 * rms(ref): the relative bound of the output type, plus
     an absolute term for elements that are small through cancellation (their error scales with the terms, not the
     sum).  The bias is added to the ROUNDED product in the output type (triton_functions.py:127-131), so where product
-    and bias cancel, one unit in the last place of the product is large against the sum: the relative bound counts both."""
+    and bias cancel, one unit in the last place of the product is large against the sum: the relative bound counts both,
+    and the second rounding (of the sum) may move the result by one more unit in the last place of the output type."""
+    ulp = {torch.float32: 2.0 ** -23, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[got.dtype]
     got, ref = got.double(), ref.double()
     rms = ref.pow(2).mean().sqrt().item()
     err = (got - ref).abs()
-    bound = tol * (ref.abs() + (2 * bias.double().abs() if bias is not None else 0.0)) + 3e-4 * rms + 1e-30
+    bound = tol * ref.abs() + 3e-4 * rms + 1e-30
+    if bias is not None:
+        bound = bound + 2 * tol * bias.double().abs() + ulp * ref.abs()
     if not (err <= bound).all():
         i = (err - bound).argmax()
         raise AssertionError(f"{int((err > bound).sum())} of {err.numel()} outside the bound; worst at flat index {i.item()}: got "
