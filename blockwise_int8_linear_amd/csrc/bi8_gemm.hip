@@ -1074,7 +1074,7 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
     static_assert(BLK == 64 || BLK == 128, "one or two 64-byte MFMAs per K-block");
     extern __shared__ __attribute__((aligned(16))) float gemv_lds[];
     float(*red)[4][64] = (float(*)[4][64])gemv_lds;                 // [wave][register][lane]
-    float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][16 rows]
+    float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][16 rows], plus one stage of zeros
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1119,10 +1119,11 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
     const int mine = (nstages - wave + NW - 1) / NW;                // stages of this wave (wave < NW <= nstages not required)
 #pragma unroll
     for (int d = 0; d < D; ++d) load_stage(d, wf[d], af[d], swf[d], std::true_type{});
-    // the row scales go to LDS while the first stages are on their way
-    for (int i = tid; i < nblk * 16; i += 256) {
+    // the row scales go to LDS while the first stages are on their way; one more stage of zeros behind them for the
+    // ring slots past the end of K (zero codes times a zero scale: a row scale of inf must not meet them)
+    for (int i = tid; i < (nblk + NBS) * 16; i += 256) {
         const int jb = i >> 4, m = i & 15;
-        s_sx[i] = m < g.M ? g.sA[(int64_t)jb * g.M + m] : 0.0f;
+        s_sx[i] = (jb < nblk && m < g.M) ? g.sA[(int64_t)jb * g.M + m] : 0.0f;
     }
     __syncthreads();
     // D stages from the ring; REFILL 2: every slot is refilled (all of those stages exist), 1: refilled with checked
@@ -1134,7 +1135,7 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
         for (int d = 0; d < D; ++d) {
             const int t = base + d;
             const int s = wave + NW * t;
-            const int sb = (s < nstages ? s : nstages - 1) * NBS;
+            const int sb = (s < nstages ? s : nstages) * NBS;        // past the end: the stage of zero row scales
             const bi8_v4i zero = {0, 0, 0, 0};
             bi8_v4i p[NBS];
             if constexpr (NBS == 1) {
@@ -1209,8 +1210,8 @@ __global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const v
     const int nstages = K / kStageK;
     const int nblk = nstages * NBS;
     float(*red)[4][64] = (float(*)[4][64])gemv_lds;                 // [wave][register][lane]
-    float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][4 rows]
-    int8_t *s_a = (int8_t *)(s_sx + (size_t)nblk * 4);               // [M][K], 16-byte aligned
+    float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][4 rows], plus one stage of zeros
+    int8_t *s_a = (int8_t *)(s_sx + (size_t)(nblk + NBS) * 4);       // [M][K], 16-byte aligned
     const int64_t n0 = (int64_t)blockIdx.x * 16;
     const int64_t n = n0 + r16;
     const int64_t wrows = g.N - n0 < 16 ? g.N - n0 : 16;
@@ -1289,8 +1290,8 @@ __global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const v
             }
         }
     }
-    for (int i = tid; i < nblk * 4; i += 256)
-        if ((i & 3) >= M) s_sx[i] = 0.0f;
+    for (int i = tid; i < (nblk + NBS) * 4; i += 256)
+        if (i >= nblk * 4 || (i & 3) >= M) s_sx[i] = 0.0f;
     __syncthreads();
 
     // the A operands follow the W ring one slot behind its refill: read from LDS a whole ring ahead of their use
@@ -1315,7 +1316,7 @@ __global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const v
         for (int d = 0; d < D; ++d) {
             const int t = base + d;
             const int s = wave + NW * t;
-            const int sb = (s < nstages ? s : nstages - 1) * NBS;
+            const int sb = (s < nstages ? s : nstages) * NBS;        // past the end: the stage of zero row scales
             const bi8_v4i zero = {0, 0, 0, 0};
             bi8_v4i p[NBS];
             if constexpr (NBS == 1) {
@@ -1612,7 +1613,7 @@ template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {
 template <int BLK, int CDT> int launch_gemv(GemmArgs g, hipStream_t st) {
     const int64_t tn = (g.N + 15) / 16;
     if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-    const size_t lds = (4 * 4 * 64 + (size_t)(g.K / BLK) * 16) * sizeof(float);
+    const size_t lds = (4 * 4 * 64 + (size_t)(g.K / BLK + kStageK / BLK) * 16) * sizeof(float);
     hipLaunchKernelGGL((gemm_gemv<BLK, CDT>), dim3((unsigned)tn), dim3(256), lds, st, g);
     return bi8_launch_rc();
 }
@@ -1773,7 +1774,7 @@ extern "C" int bi8_linear_few_rows(const void *x, int dtype, const int8_t *W, co
         ldw % 16 != 0 || ldw >= (1 << 22) || (K / block) * N * 4 >= 0x7fffffffLL || !bi8_aligned(x, 16) || !bi8_aligned(W, 16) ||
         !bi8_aligned(sW, 4) || (N + 15) / 16 > 0x7fffffffLL)
         return BI8_ERR_UNSUPPORTED;
-    const size_t lds = (4 * 4 * 64 + (size_t)(K / block) * 4) * sizeof(float) + (size_t)M * (size_t)K;
+    const size_t lds = (4 * 4 * 64 + (size_t)(K / block + kStageK / block) * 4) * sizeof(float) + (size_t)M * (size_t)K;
     if (lds > kFewRowsLdsMax) return BI8_ERR_UNSUPPORTED;
     GemmArgs g{nullptr, W, nullptr, sW, bias, C, nullptr, M, N, K, 0, ldw, ldc, 0, 0, bias_dtype};
     hipStream_t st = (hipStream_t)stream;

@@ -263,7 +263,7 @@ def linear_few_rows(x, W_int8, state_W, bias=None):
     N = W_int8.shape[0]
     if not (1 <= M <= _FEW_ROWS and block in (64, 128) and K > 0 and K % 128 == 0 and N > 0 and x.dtype == dtype
             and x.dtype in _DT and W_int8.dtype == torch.int8 and state_W.dtype == torch.float32
-            and 4096 + 16 * (K // block) + M * K <= _FEW_ROWS_LDS):
+            and 4096 + 16 * (K // block + 128 // block) + M * K <= _FEW_ROWS_LDS):
         return None
     assert x.is_cuda and W_int8.is_cuda
     assert W_int8.shape[1] == K and tuple(state_W.shape) == (K // block, N), "incompatible dimensions"

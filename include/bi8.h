@@ -173,7 +173,7 @@ int bi8_gemm_nt_partials(const int8_t *A, const int8_t *W, int32_t *P,
  *   W     int8 [N,K], leading dimension ldw;  sW fp32 [K/block, N]   (the cached weights, block_linear.py:127-128)
  *   C     [M,N] of the same `dtype`, leading dimension ldc;  bias [N] of bias_dtype or NULL
  * The result is bit for bit that of bi8_quantize_rowwise followed by bi8_gemm_nt_dequant on the same operands.
- * Covers 1 <= M <= 4, block 64 or 128, K a positive multiple of 128 with 4096 + 16*K/block + M*K <= 65536 (the
+ * Covers 1 <= M <= 4, block 64 or 128, K a positive multiple of 128 with 4096 + 16*(K/block + 128/block) + M*K <= 65536 (the
  * quantized rows sit in LDS), x and W 16-byte aligned with ldx*sizeof(elem) and ldw multiples of 16; anything else
  * returns BI8_ERR_UNSUPPORTED and the caller uses the two separate entry points.
  */

@@ -5,7 +5,9 @@
  * (one correction for 16-bit inputs, two for binary32) and compares it with the C `/` operator
  *   - for EVERY pair of bf16 values and EVERY pair of f16 values with |v| <= s (all significands
  *     and every exponent difference that can still give a non-zero code), and
- *   - for a large number of random and adversarial binary32 pairs.
+ *   - for a large number of random and adversarial binary32 pairs, and
+ *   - for DIRECTED hard-to-round binary32 pairs: quotients that lie within 2^-48 (relative) of the midpoint between
+ *     two adjacent binary32 values, the closest a quotient of two 24-bit significands can come to one.
  * Prints the number of mismatching quotients; exit status 0 only if there are none.
  *
  * Build: gcc -O2 -ffp-contract=off -fopenmp recip_division_check.c -lm
@@ -15,6 +17,9 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 
 static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
 
@@ -84,7 +89,6 @@ int main(int argc, char **argv) {
     {
         uint64_t st = rng_state;
 #ifdef _OPENMP
-        extern int omp_get_thread_num(void);
         st += 0x1234567ull * (uint64_t)(omp_get_thread_num() + 1);
 #endif
 #pragma omp for schedule(static)
@@ -124,7 +128,42 @@ int main(int argc, char **argv) {
             }
         }
     }
+    /* Directed hard cases.  For significands S (of s) and V (of v), V / S rounds hardest when V * 2^25 = S * X - r with
+     * X odd (X / 2^25 is then the midpoint between two adjacent 24-bit quotients) and |r| as small as it can be: r odd,
+     * |r| = 1, 3, 5, 7.  For odd S, X = r * S^-1 mod 2^25 solves that; it is usable when it has 25 bits and V has 24. */
+    long badh = 0, nhard = 0;
+#pragma omp parallel reduction(+ : badh, nhard)
+    {
+        uint64_t st = 0xC0FFEEull;
+#ifdef _OPENMP
+        st += 0x7654321ull * (uint64_t)(omp_get_thread_num() + 1);
+#endif
+#pragma omp for schedule(static)
+        for (long i = 0; i < 6000000; ++i) {
+            uint32_t S = (uint32_t)(0x800000u | (rng(&st) & 0x7FFFFFu)) | 1u;      /* odd, 24 bits */
+            if (i < 64) S = 0xFFFFFFu - 2u * (uint32_t)i;                          /* significands close to all ones */
+            else if (i < 128) S = 0x800001u + 2u * (uint32_t)(i - 64);            /* and just above a power of two */
+            uint32_t inv = S;                                                      /* S * inv = 1 mod 2^32 (Newton) */
+            for (int k = 0; k < 5; ++k) inv *= 2u - S * inv;
+            for (int r = -7; r <= 7; r += 2) {
+                uint32_t X = ((uint32_t)r * inv) & 0x1FFFFFFu;
+                if (X < 0x1000000u) continue;                                      /* needs 25 bits: quotient in [1/2, 1) */
+                int64_t T = (int64_t)S * (int64_t)X - r;                           /* = V * 2^25 */
+                if (T & 0x1FFFFFF) { badh++; continue; }                           /* cannot happen */
+                int64_t V = T >> 25;
+                if (V < 0x800000 || V > 0xFFFFFF) continue;
+                for (int de = 0; de <= 8; de += 4) {                               /* the same significands, smaller quotients */
+                    float s = ldexpf((float)S, -23 + (int)(i % 50) - 20);
+                    float v = ldexpf((float)V, -24 + (int)(i % 50) - 20 - de);
+                    if (v > s) continue;
+                    badh += check_pair(v, s, 2);
+                    nhard++;
+                }
+            }
+        }
+    }
     printf("random binary32 pairs: %ld checked, %ld mismatches\n", n_random, bad32);
+    printf("directed hard-to-round binary32 pairs: %ld checked, %ld mismatches\n", nhard, badh);
     printf("near-tie binary32 pairs: %ld checked, %ld mismatches\n", ntie, badt);
-    return (bad || bad32 || badt) ? 1 : 0;
+    return (bad || bad32 || badt || badh || nhard < 1000000) ? 1 : 0;
 }

@@ -313,3 +313,55 @@ def test_headline_shape_8192(ops, block):
     dense = (x[rows].float() @ w.float().t())
     rel = (C[rows.to(DEV)].cpu().float() - dense).norm() / dense.norm()
     assert rel < 3e-2
+
+
+# (M, N, K, kernel family)
+NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (2048, 2304, 256, "gemm_tile_256x128"),
+                    (8, 256, 512, "gemm_gemv"), (24, 256, 512, "gemm_skinny"), (70, 90, 200, "gemm_generic")]
+
+
+@pytest.mark.parametrize("shape", NONFINITE_SHAPES, ids=lambda s: s[3])
+def test_infinite_and_nan_scales(ops, shape):
+    """A block that held an infinity has scale inf.  The reference's sw * (sx * (P * div)) (triton_functions.py:120)
+    then gives +-inf where the block partial P is not 0 and NaN where it is.  A ROW scale of inf or NaN gives exactly
+    that in every kernel.  A COLUMN scale of inf gives it in the few-row and general kernels; the tiled kernels
+    (M > 32), whose fold computes fma(1.5*2^23 + P, b, -1.5*2^23 * b), give NaN for the whole column instead of +-inf:
+    the one place where non-finite results differ from the reference's, pinned here.  Everything else stays finite."""
+    from blockwise_int8_linear_amd import _lib
+    M, N, K, family = shape
+    block = 128 if K % 128 == 0 else 64
+    assert _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, 0).decode() == family
+    g = torch.Generator().manual_seed(M + N)
+    A, W = _codes(g, M, K), _codes(g, N, K)
+    nblk = -(-K // block)
+    j = nblk - 1
+    A[5, j * block:] = 0                            # this row's partial of block j is 0 for every column
+    sa = torch.rand(nblk, M, generator=g) + 0.1
+    sw = torch.rand(nblk, N, generator=g) * 0.05 + 1e-3
+    with cfg_as(ops, block, torch.float32):
+        run = lambda sa_, sw_: ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa_.to(DEV), sw_.to(DEV)).cpu()
+        # row scales: inf on rows 3 and 5 (row 5 has P = 0), -inf on row 4, NaN on row 7
+        sa2 = sa.clone()
+        sa2[j, 3] = sa2[j, 5] = float("inf")
+        sa2[j, 4] = float("-inf")
+        sa2[j, 7] = float("nan")
+        ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa2, sw, block, None, torch.float32)
+        got = run(sa2, sw)
+        assert ref[5].isnan().all() and ref[7].isnan().all() and ref[3].isinf().sum() > N // 2
+        assert torch.equal(got.isnan(), ref.isnan()) and torch.equal(got.isinf(), ref.isinf())
+        assert torch.equal(got[ref.isinf()], ref[ref.isinf()])             # the signs of the infinities
+        fin = torch.isfinite(ref)
+        assert fin[8:].all() and ((got[fin] - ref[fin]).abs() <= 1e-3 * ref[fin].abs() + 1e-6).all()
+        # a column scale of inf
+        sw2 = sw.clone()
+        sw2[j, 2] = float("inf")
+        ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw2, block, None, torch.float32)
+        got = run(sa, sw2)
+        assert ref[5, 2].isnan() and ref[:, 2].isinf().sum() >= M - 3
+        if family in ("gemm_gemv", "gemm_skinny", "gemm_generic"):
+            assert torch.equal(got.isnan(), ref.isnan()) and torch.equal(got[ref.isinf()], ref[ref.isinf()])
+        else:
+            assert got[:, 2].isnan().all()
+        other = torch.ones(N, dtype=torch.bool)
+        other[2] = False
+        assert torch.isfinite(got[:, other]).all() and ((got[:, other] - ref[:, other]).abs() <= 1e-3 * ref[:, other].abs() + 1e-6).all()
