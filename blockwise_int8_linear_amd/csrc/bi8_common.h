@@ -13,6 +13,7 @@ typedef int bi8_v16i __attribute__((ext_vector_type(16)));
 typedef uint32_t bi8_v4u __attribute__((ext_vector_type(4)));
 typedef uint32_t bi8_v2u __attribute__((ext_vector_type(2)));
 typedef float bi8_v4f __attribute__((ext_vector_type(4)));
+typedef float bi8_v2f __attribute__((ext_vector_type(2)));
 
 // Multi-dword accesses at addresses that are only aligned to the element (rows of odd length, e.g. the GPT-2
 // vocabulary 50257): the amdhsa ABI runs with unaligned access enabled, so these are single instructions.

@@ -6,6 +6,7 @@
 //
 // NT GEMM, both operands K-contiguous.  Four kernels, chosen by shape in dispatch():
 //   gemm_wide    blocks 128 / 64, problems of >= 129 tiles of 256x256: v_mfma_i32_16x16x64_i8, 64x128 per wave;
+//   gemm_wide32  block 32, same problems and tile: v_mfma_i32_32x32x32_i8, 32x256 per wave;
 //   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x128 / 64x128 tiles, 64x64 per wave; also
 //                the int32 block partials;
 //   gemm_gemv    M <= 16, blocks 64/128 (decode): one pass over W, 16 columns per workgroup, K split over 4 waves,
@@ -982,6 +983,300 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     }
 }
 
+// ---- 256x256 tile on v_mfma_i32_32x32x32_i8 ---------------------------------------------------------------------------
+// Same workgroup tile, loader, stage buffers and single barrier per stage as gemm_wide; what differs is the shape of
+// the matrix instruction and with it the wave tile.  A 32x32x32 MFMA does twice the work of a 16x16x64 one for the
+// same hold on the issue port, so half as many of them are issued per K-block; the price is its accumulator layout
+// (16 rows per lane instead of 4), which makes a wave's row scales cost 16 registers per 32 rows.  The eight waves
+// therefore stack along M: one wave owns 32 rows x 256 columns = 8 subtiles of 32x32.  Per stage it keeps its 32 rows
+// of A (16 registers) and the K-block's row scales (16) in registers and streams the eight column subtiles of W
+// through ONE register buffer: the 16-byte chunk of W that MFMA k-step ks has just consumed is refilled with the same
+// chunk of the next subtile, which is needed four MFMAs later.  An item = one (K-block, column subtile): BLK/32
+// chained MFMAs, each followed by a slice of the fold of the item before (the chain is dependent, so the fold's
+// vector instructions fill the wait for the previous MFMA's result).
+// Used for block 32, where a K-block is exactly one such MFMA (8192^3: 1.23 ms against 1.47 ms on 128x128 tiles).
+// For blocks 128 and 64 it measured SLOWER than gemm_wide (0.65 against 0.53 ms, 0.81 against 0.71 ms at 8192^3): its
+// three 16-register tuples (two partials and the 1.5*2^23 start value, which the compiler then rebuilds with eight
+// moves per item rather than keep) and the 32x256 wave tile's extra LDS reads (48 against 36 per wave and stage) cost
+// more than the halved MFMA count gives back; a 64x128 wave tile with this instruction does not fit 256 registers.
+template <int NBS> struct Wide32Lds {
+    using W = WideLds<NBS>;
+    static constexpr int kOutPitch = 512 + 16;                                // a wave's 32 x 256 tile of 16-bit outputs
+    static constexpr int kOut = 8 * 32 * kOutPitch;                          // 132 KiB
+    static constexpr int kBytes = kOut > W::kStages ? kOut : W::kStages;
+};
+
+template <int BLK, int CDT>
+__global__ __launch_bounds__(512) void gemm_wide32(const GemmArgs g) {
+    static_assert(BLK == 128 || BLK == 64 || BLK == 32, "a K-block is 1, 2 or 4 MFMAs of 32 bytes of K");
+    constexpr int NBS = kStageK / BLK;             // K-blocks per stage
+    constexpr int KSB = BLK / 32;                  // MFMAs per K-block and subtile
+    constexpr int NJ = 8;                          // column subtiles of a wave
+    constexpr int NI = NBS * NJ;                   // items per stage
+    using L = WideLds<NBS>;
+    constexpr int BM = 256, BN = 256, NW = 8;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, h = lane >> 5;
+
+    int tile_m, tile_n;
+    tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int nstages = (int)(g.K / kStageK);
+
+    // ---- loader: exactly gemm_wide's (wave instruction i covers tile rows 8i .. 8i+7, chunk swizzle (row >> 1) & 7)
+    const int ld_row = lane >> 3;
+    const int ld_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+    const int64_t a_rows = (g.M - m0 < BM) ? (g.M - m0) : BM, w_rows = (g.N - n0 < BN) ? (g.N - n0) : BN;
+    const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
+    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
+    const uint32_t a_off = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_off = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
+    const uint32_t a_wave = (uint32_t)(wave * 8 * g.lda), w_wave = (uint32_t)(wave * 8 * g.ldw);
+    const uint32_t a_step = (uint32_t)(NW * 8 * g.lda), w_step = (uint32_t)(NW * 8 * g.ldw);
+    const int64_t nblk = g.K / BLK;
+    const bool s_is_a = wave < 4;
+    const int s_part = wave & 3;
+    const bi8_brsrc sa_brsrc = bi8_make_brsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
+    const bi8_brsrc sw_brsrc = bi8_make_brsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
+    const bi8_brsrc s_brsrc = s_is_a ? sa_brsrc : sw_brsrc;
+    const uint32_t s_off = (uint32_t)((s_part * 64 + lane) * 4);
+    const uint32_t s_inc = (uint32_t)((s_is_a ? g.M : g.N) * 4);
+    float s_raw[NBS];
+#pragma unroll
+    for (int kb = 0; kb < NBS; ++kb) s_raw[kb] = 0.0f;
+    // Column scales are stored prepared, as the pair (b, -1.5*2^23*b) with b rounded to 22 significant bits, in the
+    // order [column within its subtile][subtile][b, c]: a lane reads the pairs of two subtiles with one 16-byte read.
+    // The fetching lane holds tile column s_part * 64 + lane = subtile 2 * s_part + lane / 32, column lane % 32.
+    const int c_dst = L::kSWReg + ((lane & 31) * NJ + 2 * s_part + (lane >> 5)) * 8;
+    // (a row-scale lane's second store repeats its first: both kinds of lane run the same instructions)
+    int p_dst0 = s_is_a ? L::kSAReg + (s_part * 64 + lane) * 4 : c_dst;
+    const int p_second = s_is_a ? 0 : 4;           // wave-uniform
+    const int p_buf0 = s_is_a ? L::kSBuf : L::kCBuf, p_row0 = s_is_a ? L::kSRow : L::kCRow;
+    uint32_t s_pos = 0, k_pos = 0;
+    constexpr int kLoadsPerStage = 4 + 4 + NBS;
+    constexpr int kEarly = 3, kLateItems = (kLoadsPerStage - kEarly + 1) / 2;
+    static_assert(kLateItems <= NI - 1, "the late loads are issued before the last item of the stage before");
+
+    const uint32_t lds_base = bi8_lds_address(lds);
+    auto issue_one = [&](int buf, int idx) {
+        if (idx < 4) {
+            bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + idx * NW) * 1024, a_off, k_pos, a_wave + idx * a_step);
+        } else if (idx < 8) {
+            bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + (idx - 4) * NW) * 1024, w_off, k_pos, w_wave + (idx - 4) * w_step);
+        } else if (idx < kLoadsPerStage) {
+            s_raw[idx - 8] = bi8_buffer_load_f32(s_brsrc, (int)s_off, (int)s_pos);
+            s_pos += s_inc;
+            if (idx == kLoadsPerStage - 1) k_pos += kStageK;
+        }
+    };
+    auto publish_scales = [&](int buf) {           // buf is wave-uniform
+        const int dst = p_dst0 + buf * p_buf0;
+#pragma unroll
+        for (int kb = 0; kb < NBS; ++kb) {
+            const float b = bi8_u2f((bi8_f2u(s_raw[kb]) + 2u) & ~3u);     // 22 significant bits
+            *(float *)(lds + dst + kb * p_row0) = s_is_a ? s_raw[kb] : b;
+            *(float *)(lds + (dst + p_second) + kb * p_row0) = s_is_a ? s_raw[kb] : -BI8_MAGIC * b;   // exact
+        }
+    };
+
+    // ---- operand fragments of a 32x32x32 MFMA: lane -> row l32 of the subtile, 16-byte chunk 2*ks + h of the stage's
+    // eight, stored at chunk position (2*ks + h) ^ ((row >> 1) & 7): address(ks) = address(0) ^ (ks << 5)
+    const int frag_sw = ((h ^ ((l32 >> 1) & 7)) << 4);
+    // (W: one address register per ks, read 32 times a stage; A is read four times a stage and derives its addresses)
+    int a_addr0 = L::kAReg + (wave * 32 + l32) * kStageK + frag_sw, w_addr[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) w_addr[ks] = (L::kWReg + l32 * kStageK + frag_sw) ^ (ks << 5);
+    // outputs of a subtile: lane -> column l32, rows 8 * (r >> 2) + 4 * h + (r & 3) for accumulator register r
+    int sa_base = L::kSAReg + (wave * 32 + 4 * h) * 4;
+    int sw_base = L::kSWReg + l32 * NJ * 8;
+    asm volatile("" : "+v"(a_addr0), "+v"(w_addr[0]), "+v"(w_addr[1]), "+v"(w_addr[2]), "+v"(w_addr[3]), "+v"(sa_base), "+v"(sw_base), "+v"(p_dst0));
+
+    float acc[NJ][16];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] = 0.0f;
+
+    constexpr int kMagicBits = 0x4B400000;        // bit pattern of 1.5 * 2^23
+    const bi8_v16i magic = {kMagicBits, kMagicBits, kMagicBits, kMagicBits, kMagicBits, kMagicBits, kMagicBits, kMagicBits,
+                            kMagicBits, kMagicBits, kMagicBits, kMagicBits, kMagicBits, kMagicBits, kMagicBits, kMagicBits};
+    bi8_v4i A[4], Wf[4];                           // this stage's A chunks; the current subtile's W chunks
+    bi8_v4f sx[4];                                 // row scales of the K-block being folded: rows 8*g + 4*h + 0..3
+    bi8_v2f bc[2];                                 // (b, c) of a subtile, by parity of the item
+    bi8_v16i P[2];
+    P[0] = P[1] = magic;
+    bc[0] = bc[1] = bi8_v2f{0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sx[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto read_a = [&](int ks) {
+        int addr = a_addr0;
+        if (ks) asm volatile("v_xor_b32 %0, %1, %2" : "=v"(addr) : "v"(a_addr0), "v"(ks << 5));    // not hoisted out of the loop
+        A[ks] = *(const bi8_v4i *)(lds + addr);
+    };
+    auto read_w = [&](int ks, int j) { Wf[ks] = *(const bi8_v4i *)(lds + w_addr[ks] + j * 32 * kStageK); };
+    auto read_bc = [&](int kb, int j) { bc[j & 1] = *(const bi8_v2f *)(lds + sw_base + kb * L::kCRow + j * 8); };
+    auto read_sx = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) sx[i] = *(const bi8_v4f *)(lds + sa_base + kb * L::kSRow + i * 8 * 4);
+    };
+    // The read addresses above point into the stage buffer that the reads of the moment are for; they move to the other
+    // buffer right behind the barrier of a stage, after which every read is for the next stage.
+    auto switch_buffers = [&](int to) {            // to: wave-uniform, 0 or 1
+        const int d = to ? 1 : -1;
+        a_addr0 += d * L::kABuf;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) w_addr[ks] += d * L::kWBuf;
+        sa_base += d * L::kSBuf;
+        sw_base += d * L::kCBuf;
+    };
+    // elements [16 * q / KSB, 16 * (q + 1) / KSB) of a finished partial: fma(f, b, c) = fl(b * P) (the partial carries
+    // the 1.5*2^23 offset), then the row scale and the accumulation
+    auto fold_slice = [&](const bi8_v16i &pt, int j, int q) {
+        const float b = bc[j & 1][0], cm = bc[j & 1][1];
+#pragma unroll
+        for (int r = q * (16 / KSB); r < (q + 1) * (16 / KSB); ++r) {
+            const float u = __builtin_fmaf(bi8_u2f((uint32_t)pt[r]), b, cm);
+            acc[j][r] = __builtin_fmaf(u, sx[r >> 2][r & 3], acc[j][r]);
+        }
+    };
+    auto wait_vm = [&](auto pending_c) {
+        constexpr int kPending = decltype(pending_c)::value;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
+    };
+
+    // One stage, in stage buffer `cur` (wave-uniform; the loop below is not unrolled over the two buffers, so that the
+    // registers keep their roles from one stage to the next).  Item t = (K-block t / 8, subtile t % 8).  On entry A[]
+    // and Wf[] hold this stage's operands of item 0, and P[1], sx[], bc[1] the last item of the stage before, still to
+    // be folded.
+    auto stage = [&](int cur) {
+        const int nxt = 1 - cur;
+#pragma unroll
+        for (int t = 0; t < NI; ++t) {
+            const int kb = t / NJ, j = t % NJ;
+            const int tp = (t + NI - 1) % NI, jp = tp % NJ;             // the item before
+            if (t < kLateItems) issue_one(nxt, kEarly + 2 * t);
+            // this item's pair: first used by the fold one item on (the other register serves the fold below)
+            read_bc(kb, j);
+            if (t == NI - 1) {
+                // every operand of this stage is in registers or on its way: publish the next stage, release this one
+                __builtin_amdgcn_s_waitcnt(0xC07F);                    // lgkmcnt(0) only
+                wait_vm(std::integral_constant<int, 0>{});
+                publish_scales(nxt);
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                switch_buffers(nxt);
+#pragma unroll
+                for (int idx = 0; idx < kEarly - 1; ++idx) issue_one(cur, idx);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int q = 0; q < KSB; ++q) {
+                const int ks = kb * KSB + q;
+                P[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(A[ks], Wf[ks], q == 0 ? magic : P[t & 1], 0, 0, 0);
+                // the chunk just consumed is refilled: W with the next item's, A (after its last use) with the next stage's
+                if (t == NI - 1) {
+                    read_w(q, 0);
+                    // no A chunk is needed any more once this stage's last MFMA on it is issued: the next stage's
+#pragma unroll
+                    for (int kk = q; kk < 4; kk += KSB) read_a(kk);
+                } else {
+                    const int tn = t + 1;
+                    read_w((tn / NJ) * KSB + q, tn % NJ);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                fold_slice(P[tp & 1], jp, q);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (t == NI - 1) issue_one(cur, kEarly - 1);
+            // the fold above was the last of its K-block when the item before was a subtile 7: its row scales make way
+            // for those of the block whose first item has just been issued
+            if (j == 0) read_sx(kb);
+            if (t < kLateItems) issue_one(nxt, kEarly + 2 * t + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // prologue: the first stage's loads and the early part of the second's; wait for the first stage
+#pragma unroll
+    for (int idx = 0; idx < kLoadsPerStage; ++idx) issue_one(0, idx);
+#pragma unroll
+    for (int idx = 0; idx < kEarly; ++idx) issue_one(1, idx);
+    wait_vm(std::integral_constant<int, kEarly>{});
+    publish_scales(0);
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        read_a(ks);
+        if (ks < KSB) read_w(ks, 0);
+    }
+    // The trip count is rounded up to even and loads run two stages ahead: stages past the end of K read their
+    // scales through the buffers' range check as zeros, so they add exactly 0 to the accumulators.
+    {
+        const int trips = (nstages + 1) & ~1;
+        int cur = 0;
+#pragma nounroll
+        for (int s = 0; s < trips; ++s) {
+            stage(cur);
+            cur = 1 - cur;
+        }
+    }
+    wait_vm(std::integral_constant<int, 0>{});     // nothing may still be writing LDS when the wave ends
+#pragma unroll
+    for (int q = 0; q < KSB; ++q) fold_slice(P[(NI - 1) & 1], NJ - 1, q);   // the last item of the last (possibly padding) stage
+
+    const float div = (float)(1.0 / (127.0 * 127.0));
+    const bool has_bias = g.bias != nullptr;
+    if constexpr (CDT != BI8_F32) {
+        // 16-bit outputs leave through LDS: a row-major copy of the wave's 32 x 256 tile, stored as 512-byte row runs
+        __syncthreads();                           // every wave is done with the stage buffers
+        uint8_t *tile = lds + wave * (32 * Wide32Lds<NBS>::kOutPitch);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int64_t n = n0 + j * 32 + l32;
+            const float bias = (has_bias && n < g.N) ? bi8_round_to<CDT>(load_bias(g, n)) : 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float v = bi8_round_to<CDT>(acc[j][r] * div);          // acc.to(C.dtype), then + bias in C's dtype
+                if (has_bias) v = v + bias;
+                const uint32_t bits = (CDT == BI8_BF16) ? bi8_bf16_bits(v) : bi8_f16_bits(v);
+                *(uint16_t *)(tile + (8 * (r >> 2) + 4 * h + (r & 3)) * Wide32Lds<NBS>::kOutPitch + (j * 32 + l32) * 2) = (uint16_t)bits;
+            }
+        }
+        // lane -> row 2p + lane / 32 of the tile, 8 outputs (16 bytes) at column 8 * (lane % 32)
+        const int64_t n = n0 + l32 * 8;
+#pragma unroll
+        for (int p = 0; p < 16; ++p) {
+            const int row = 2 * p + h;
+            const int64_t m = m0 + wave * 32 + row;
+            const bi8_v4u v = *(const bi8_v4u *)(tile + row * Wide32Lds<NBS>::kOutPitch + l32 * 16);
+            if (m < g.M) {
+                uint16_t *dst = (uint16_t *)g.C + m * g.ldc + n;
+                if (n + 8 <= g.N) {
+                    *(bi8_v4u_unaligned *)dst = v;
+                } else {
+                    for (int e = 0; e < 8 && n + e < g.N; ++e) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+                }
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int64_t n = n0 + j * 32 + l32;
+        const bool n_ok = n < g.N;
+        const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int64_t m = m0 + wave * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[j][r] * div, has_bias, bias);
+        }
+    }
+}
+
 // Skinny GEMM (M <= 32), HBM-bound on W: the whole problem is one pass over the N*K bytes of weight codes.
 // One workgroup = 32 output columns, 8 waves that split K in interleaved 128-byte stages; every wave gathers its
 // MFMA operands straight from global memory in operand layout (16 bytes per lane; the four k-steps of a stage
@@ -1520,6 +1815,20 @@ template <int BLK, int CDT> int launch_wide(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
+template <int BLK, int CDT> int launch_wide32(GemmArgs g, hipStream_t st) {
+    using L = Wide32Lds<kStageK / BLK>;
+    const int64_t tm = (g.M + 255) / 256, tn = (g.N + 255) / 256;
+    if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+    g.tiles_m = (int)tm;
+    g.tiles_n = (int)tn;
+    auto kern = gemm_wide32<BLK, CDT>;
+    static LdsOptIn opted;                         // one per kernel instantiation
+    const int rc = opted.ensure((const void *)kern, L::kBytes);
+    if (rc != BI8_OK) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(512), L::kBytes, st, g);
+    return bi8_launch_rc();
+}
+
 template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipStream_t st) {
     const int64_t tm = (g.M + 63) / 64, tn = (g.N + 63) / 64;
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
@@ -1567,7 +1876,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             return p;
         }
         // 256x256 tiles when there is enough work to fill the 256 CUs with them
-        if ((block == 128 || block == 64) && ((M + 255) / 256) * ((N + 255) / 256) >= kWideMinTiles) {
+        if (((M + 255) / 256) * ((N + 255) / 256) >= kWideMinTiles) {
             p.kernel = kKWide;
             return p;
         }
@@ -1636,8 +1945,9 @@ template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, co
             break;
         case kKSkinny: return launch_skinny<BLK, CDT>(g, st);
         case kKWide:
-            if constexpr (BLK != 32) return launch_wide<BLK, CDT>(g, st);
-            break;
+            // blocks 128 and 64: 16x16x64 MFMAs, 64x128 per wave; block 32 (one MFMA per K-block): 32x32x32, 32x256 per wave
+            if constexpr (BLK == 32) return launch_wide32<BLK, CDT>(g, st);
+            else return launch_wide<BLK, CDT>(g, st);
         case kKSplit128x128:
         case kKSplit64x128: {
             GemmArgs gs = g;

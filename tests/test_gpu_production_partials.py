@@ -67,6 +67,8 @@ CASES = [
     (2944, 2900, 384, 128, "gemm_wide"),            # odd number of stages (the loop runs a padding stage), ragged N
     (2944, 2944, 512, 64, "gemm_wide"),             # two K-blocks per stage
     (2900, 2944, 384, 64, "gemm_wide"),
+    (2944, 2944, 256, 32, "gemm_wide"),             # block 32: the 32x32x32-MFMA form, four K-blocks per stage
+    (2900, 2944, 384, 32, "gemm_wide"),
     (2048, 2304, 512, 128, "gemm_tile_256x128"),    # the software-pipelined block-128 instantiation
     (2000, 2304, 384, 128, "gemm_tile_256x128"),
     (2048, 2304, 512, 64, "gemm_tile_256x128"),
@@ -122,7 +124,7 @@ def test_partials_of_the_shipping_kernels(ops, case, out):
             assert torch.equal(C.cpu()[exact], want[exact])
 
 
-@pytest.mark.parametrize("case", CASES[:2] + CASES[4:5], ids=lambda c: "x".join(map(str, c[:4])) + "-" + c[4])
+@pytest.mark.parametrize("case", CASES[:2] + CASES[4:7], ids=lambda c: "x".join(map(str, c[:4])) + "-" + c[4])
 def test_partials_of_the_f16_instantiations(ops, case):
     M, N, K, block, kernel = case
     g = torch.Generator().manual_seed(K + block)
