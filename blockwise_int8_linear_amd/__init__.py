@@ -16,6 +16,7 @@ from .ops import (
     int8_matmul_block_partials,
     linear_few_rows,
     quantize_block_dual,
+    quantize_block_dual_colsum,
     quantize_block_rowwise,
     quantize_block_transposed,
 )
@@ -25,5 +26,5 @@ __all__ = [
     "blockwise_int8_linear_Wint8", "quantize_weight_for_training", "replace_linear_with_blockwise_int8_recursive",
     "replace_linear_with_blockwise_int8", "quantize_block_rowwise", "quantize_block_transposed",
     "dequantize_block_rowwise", "int8_matmul_block64_rowwise_dequantize", "int8_matmul_block_partials",
-    "linear_few_rows", "quantize_block_dual",
+    "linear_few_rows", "quantize_block_dual", "quantize_block_dual_colsum",
 ]

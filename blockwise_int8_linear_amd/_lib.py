@@ -11,7 +11,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libbi8.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "bi8.h")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _i64, _vp, _ci = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int
 
@@ -22,6 +22,8 @@ SIGNATURES = {
     "bi8_quantize_rowwise": (_ci, [_vp, _ci, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_quantize_transposed": (_ci, [_vp, _ci, _vp, _vp, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_quantize_dual": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
+    "bi8_colsum_workspace_bytes": (_i64, [_i64, _i64]),
+    "bi8_quantize_dual_colsum": (_ci, [_vp, _ci, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_dequantize_rowwise": (_ci, [_vp, _vp, _vp, _ci, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_gemm_nt_dequant": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp]),
     "bi8_gemm_nt_dequant_ws": (_ci, [_vp, _vp, _vp, _vp, _vp, _ci, _vp, _ci, _i64, _i64, _i64, _i64, _i64, _i64, _ci, _vp, _i64, _vp]),

@@ -7,6 +7,8 @@ Differences from the reference that do not change results:
     quantizer, block_linear.py:93-94, :100-103) are never materialized, and each of X, W and G is read once for both
     of its quantization directions (X and W in the forward pass, whose transposed codes are what is saved for backward);
   * ``ctx.save_for_backward`` is called, not assigned over (block_linear.py:73);
+  * the bias gradient ``G.sum(dim=0)`` (block_linear.py:110) comes out of the kernel that quantizes G (same read of G;
+    fp32 sums in a fixed order);
   * switching the module back to training mode drops the cached int8 weights, so a later ``eval()``
     re-quantizes the current weights (the reference keeps serving the first cache, block_linear.py:138-139);
   * the eval path with at most 4 rows (token-by-token decode) quantizes and multiplies in one kernel
@@ -93,9 +95,14 @@ class blockwise_int8_linear(torch.autograd.Function):
         Xt_int8, Xt_state, Wt_store, Wt_state = ctx.saved_tensors
         need_gx, need_gw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         g_store = None
+        need_gb = ctx.needs_input_grad[2]
         if need_gx and need_gw:
-            # one read of G for both GEMMs; the row codes padded like the transposed W codes they are multiplied with
-            g_int8, g_state, gt_int8, gt_state, g_store, _ = _quantize_block_dual(G, block_linear_config.GROUP_SIZE, pad=True)
+            # one read of G for both GEMMs (the row codes padded like the transposed W codes they are multiplied with)
+            # and, if there is a bias, for its gradient G.sum(dim=0) (block_linear.py:110)
+            g_int8, g_state, gt_int8, gt_state, g_store, _, *rest = _quantize_block_dual(G, block_linear_config.GROUP_SIZE, pad=True,
+                                                                                         colsum=need_gb)
+            if need_gb:
+                grad_bias = rest[0]
         elif need_gx:
             g_int8, g_state = quantize_block_rowwise(G)
         elif need_gw:
@@ -108,7 +115,7 @@ class blockwise_int8_linear(torch.autograd.Function):
         if need_gw:
             # grad_W [N,K] = G.T [N,M] @ X [M,K]: contraction over the tokens, both quantized along M
             grad_W = int8_matmul_block64_rowwise_dequantize(gt_int8, Xt_int8.t(), gt_state, Xt_state)
-        if ctx.needs_input_grad[2]:
+        if need_gb and grad_bias is None:
             grad_bias = G.sum(dim=0)
         return grad_X, grad_W, grad_bias
 
@@ -155,8 +162,12 @@ class blockwise_int8_linear_Wint8(torch.autograd.Function):
         Xt_int8, Xt_state, Wt_int8, Wt_state, Wt_store = ctx.saved_tensors
         need_gx, need_gw = ctx.needs_input_grad[0], Xt_int8 is not None
         g_store = None
+        need_gb = ctx.needs_input_grad[3]
         if need_gx and need_gw:
-            g_int8, g_state, gt_int8, gt_state, g_store, _ = _quantize_block_dual(G, block_linear_config.GROUP_SIZE, pad=True)
+            g_int8, g_state, gt_int8, gt_state, g_store, _, *rest = _quantize_block_dual(G, block_linear_config.GROUP_SIZE, pad=True,
+                                                                                         colsum=need_gb)
+            if need_gb:
+                grad_bias = rest[0]
         elif need_gx:
             g_int8, g_state = quantize_block_rowwise(G)
         elif need_gw:
@@ -166,7 +177,7 @@ class blockwise_int8_linear_Wint8(torch.autograd.Function):
             grad_X = grad_X.view(*G_3D.size()[:-1], -1)
         if need_gw:
             grad_W = int8_matmul_block64_rowwise_dequantize(gt_int8, Xt_int8.t(), gt_state, Xt_state)
-        if ctx.needs_input_grad[3]:
+        if need_gb and grad_bias is None:
             grad_bias = G.sum(dim=0)
         # one entry per argument that apply() was given (the last two are optional)
         return (grad_X, None, None, grad_bias, None, None, grad_W, None)[:len(ctx.needs_input_grad)]

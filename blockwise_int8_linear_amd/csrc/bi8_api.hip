@@ -1,7 +1,7 @@
 // Version and error-string entry points of libbi8.
 #include "bi8_common.h"
 
-extern "C" int bi8_version(void) { return 4; }
+extern "C" int bi8_version(void) { return 5; }
 
 extern "C" const char *bi8_strerror(int code) {
     switch (code) {

@@ -9,8 +9,10 @@
 //   gemm_wide32  block 32, same problems and tile: v_mfma_i32_32x32x32_i8, 32x256 per wave;
 //   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x128 / 64x128 tiles, 64x64 per wave; also
 //                the int32 block partials;
-//   gemm_gemv    M <= 16, blocks 64/128 (decode): one pass over W, 16 columns per workgroup, K split over 4 waves,
-//                operands gathered from global memory through an 8-stage register ring;
+//   gemv_rows    M <= 2, blocks 64/128 (single-token decode; also bi8_linear_few_rows, which quantizes the activations in
+//                the same launch): one pass over W in 1 KiB runs of whole rows, v_dot4_i32_i8 on the vector unit;
+//   gemm_gemv    M <= 16, blocks 64/128 (small decode batches): one pass over W, 16 columns per workgroup, K split over
+//                4 waves, operands gathered from global memory through an 8-stage register ring;
 //   gemm_skinny  M <= 32 otherwise: the same idea with 32x32x32 MFMAs and one stage of lookahead;
 //   gemm_generic anything else (K not a multiple of 128, rows not 16-byte aligned, other block sizes): same
 //                MFMA, operands gathered straight from global memory with byte loads.
@@ -1478,183 +1480,231 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
     }
 }
 
-// Quantize + few-row GEMM in one launch (M <= 4: single-token decode).  The eval path of the reference quantizes the
-// activations and then multiplies (block_linear.py:141-144): two launches of which the first moves a few KiB.  Here
-// every workgroup first starts its W loads exactly as gemm_gemv does, then quantizes the whole of x [M,K] (read
-// through L2) into LDS -- int8 codes [M][K] and row scales [K-block][4] -- with the arithmetic of the row quantizer
-// (same helpers, same results), and runs the gemm_gemv loop with its A operands read from LDS.  The output is bit for
-// bit that of bi8_quantize_rowwise followed by bi8_gemm_nt_dequant.
-constexpr int kFewRowsMax = 4;
-constexpr size_t kFewRowsLdsMax = 64 * 1024;
-template <int BLK, int DT>
-__global__ __launch_bounds__(256) void linear_few_rows(const GemmArgs g, const void *__restrict__ x, int64_t ldx) {
-    constexpr int NW = 4, D = kGemvDepth;
-    constexpr int NBS = kStageK / BLK;
-    constexpr int VEC = Bi8Vec<DT>::kElems;
-    constexpr int L = BLK / VEC;                   // lanes that hold one K-block of one row
-    constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
-    constexpr int64_t ES = 16 / VEC;
-    constexpr int U = 4;                           // 16-byte loads of x in flight per lane
-    static_assert(BLK == 64 || BLK == 128, "one or two 64-byte MFMAs per K-block");
-    extern __shared__ __attribute__((aligned(16))) float gemv_lds[];
+// ---- one or two rows, weight rows read as whole runs -------------------------------------------------------------------
+// One or two rows of activations against all of W: single-token decode.  The problem is one pass over the N*K bytes of
+// weight codes and nothing else matters.  Gathering W in the operand layout of an MFMA (gemm_gemv: 16 rows x 64
+// bytes per load instruction) reads 64-byte pieces of sixteen rows at a time, which this chip's memory pipeline serves
+// at 3.8 - 4.5 TB/s; whole 1 KiB runs of one row per load instruction (lane -> 16 consecutive bytes) come in at 5.3 -
+// 6.2 TB/s (a read-only micro-benchmark of the two patterns on the same grid).  With so few rows the matrix pipe has
+// nothing to offer anyway (a 16-row MFMA would be 1/16 to 1/4 used), so the dot products are v_dot4_i32_i8 on the
+// vector unit: per 16 bytes of W and row of activations four of them, then an integer sum over the lanes of a K-block
+// (DPP), the conversion and the two scale products.  One workgroup = 16 output columns, a wave = four of them, each
+// walked along K in runs of 1 KiB with sixteen loads in flight per lane (four rows x four runs).  The activations'
+// codes [M][K] and row scales, and the 16 columns' scales, sit in LDS; with FUSED the codes are made here from the
+// un-quantized activations by the row quantizer's own arithmetic (BlockInt8Linear.infer, block_linear.py:141-144, as one
+// launch).  The fp32 sums run over the K-blocks in a fixed order (per lane group ascending, then a butterfly over the
+// groups): the same code and therefore the same bits with and without FUSED.
+constexpr int kRowsMax = 2;                        // rows of activations (with four the kernel needs more registers than three
+                                                   // workgroups per CU leave it, and the MFMA kernel is as fast)
+constexpr size_t kRowsLdsMax = 64 * 1024;
+// scale rows in LDS: the K-blocks of whole runs, plus one run of zeros for loop slots past the end of K, rounded up to
+// 16 rows (the rows are filled 64 floats at a time)
+template <int BLK> constexpr int rows_blocks_padded(int64_t K) { return ((int)((K + 1023) / 1024 + 1) * (1024 / BLK) + 15) & ~15; }
+// the kernel is compiled for 1 and for 2 rows
+static inline int rows_compiled_for(int64_t M) { return M <= 1 ? 1 : 2; }
+template <int BLK> static size_t rows_lds_bytes(int64_t M, int64_t K) {
+    return (size_t)rows_blocks_padded<BLK>(K) * (4 + 16) * sizeof(float) + (size_t)rows_compiled_for(M) * (size_t)K + 1024;
+}
+template <int CTRL> __device__ __forceinline__ int bi8_dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false); }
+
+template <int BLK, int DT, bool FUSED, int MM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void gemv_rows(const GemmArgs g, const void *__restrict__ x, int64_t ldx) {
+    static_assert(BLK == 64 || BLK == 128, "a K-block is 4 or 8 lanes of 16 bytes");
+    constexpr int LB = BLK / 16;                   // lanes per K-block
+    constexpr int BPC = 1024 / BLK;                // K-blocks per run of 1 KiB
+    constexpr int R = 4, CG = 4;                   // rows of W per wave; runs in flight per row
+    extern __shared__ __attribute__((aligned(16))) float rows_lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int r16 = lane & 15, q = lane >> 4;
     const int K = (int)g.K, M = (int)g.M;
-    const int nstages = K / kStageK;
-    const int nblk = nstages * NBS;
-    float(*red)[4][64] = (float(*)[4][64])gemv_lds;                 // [wave][register][lane]
-    float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][4 rows], plus one stage of zeros
-    int8_t *s_a = (int8_t *)(s_sx + (size_t)(nblk + NBS) * 4);       // [M][K], 16-byte aligned
+    const int nblk = K / BLK;
+    const int nrun = (K + 1023) / 1024;            // runs per row; the last one may be partial (K is a multiple of 128)
+    const int nblk_pad = rows_blocks_padded<BLK>(K);
+    float *s_sx = rows_lds;                        // [K-block][4 rows of activations], zeros past M and past K
+    float *s_sw = s_sx + (size_t)nblk_pad * 4;     // [K-block][16 columns], zeros past N and past K
+    int8_t *s_a = (int8_t *)(s_sw + (size_t)nblk_pad * 16);          // [M][K] codes (+ 1 KiB that partial runs may read)
     const int64_t n0 = (int64_t)blockIdx.x * 16;
-    const int64_t n = n0 + r16;
     const int64_t wrows = g.N - n0 < 16 ? g.N - n0 : 16;
     const bi8_brsrc rw = bi8_make_brsrc(g.W + n0 * g.ldw, (wrows - 1) * g.ldw + g.K);   // rows past N read as zeros
-    const bi8_brsrc rs = bi8_make_brsrc(g.sW, (int64_t)nblk * g.N * 4);
-    const int voff_w = r16 * (int)g.ldw + q * 16;
-    const int voff_s = (int)(n < g.N ? n : g.N - 1) * 4;           // clamped: never stored
-    const int srow = (int)g.N * 4;
 
-    bi8_v4i wf[D][2];
-    float swf[D][NBS];
-    // CHECKED loads: a stage past the end of K gets an offset beyond the buffers' ranges and returns zeros without
-    // touching memory
-    auto load_stage = [&](int t, bi8_v4i *w, float *sw, auto checked) {
-        const int s = wave + NW * t;
-        int kill = 0, sc = s;
-        if constexpr (decltype(checked)::value) {
-            kill = s < nstages ? 0 : kBufOut;                       // wave-uniform
-            sc = s < nstages ? s : nstages - 1;
+    // ---- Order of the memory traffic.  Loads complete in the order they are issued, so what the prologue needs goes
+    // out FIRST (a few KiB: the activations, their scales, the 16 columns' scales), then this wave's first sixteen runs
+    // of W; the prologue then waits for its own data only ("at most 16 loads still outstanding"), and the loop works
+    // on the runs of W as they arrive.  Scales (and, without FUSED, the codes) go global -> LDS directly, no registers.
+    // The workgroup barrier is a bare s_barrier behind an LDS wait: a fence would wait for the W loads as well.
+    const uint32_t lds0 = bi8_lds_address(rows_lds);
+    {
+        const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW, (int64_t)nblk * g.N * 4);
+        for (int i0 = wave * 64; i0 < nblk_pad * 16; i0 += 256) {
+            const int i = i0 + lane, jb = i >> 4, n = i & 15;
+            const uint32_t off = (jb < nblk && n < wrows) ? (uint32_t)(((int64_t)jb * g.N + n0 + n) * 4) : (uint32_t)kBufOut;
+            bi8_buffer_to_lds4(sw_rsrc, lds0 + (uint32_t)(nblk_pad * 4 + i0) * 4, off, 0);
         }
-        const int k0 = sc * kStageK;
+    }
+    constexpr int VEC = FUSED ? Bi8Vec<DT>::kElems : 16;
+    constexpr int U = 8;                           // 16-byte loads of x in flight per lane (FUSED)
+    const int cpr = K / VEC;                       // 16-byte chunks per row of activations
+    const int total = M * cpr;
+    bi8_v4u raw[U];
+    auto load_x = [&](int c0) {
+        if constexpr (FUSED) {
+            constexpr int64_t ES = 16 / VEC;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) w[kb] = bi8_buffer_load16(rw, voff_w + kill + kb * 64, k0, true);
-#pragma unroll
-        for (int b = 0; b < NBS; ++b) sw[b] = bi8_buffer_load_f32(rs, voff_s + kill, (sc * NBS + b) * srow);
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * 256 + tid;
+                raw[u] = bi8_v4u{0u, 0u, 0u, 0u};
+                if (c < total) raw[u] = *(const bi8_v4u *)((const char *)x + ((int64_t)(c / cpr) * ldx + (int64_t)(c % cpr) * VEC) * ES);
+            }
+        }
+    };
+    if constexpr (FUSED) {
+        load_x(0);
+    } else {
+        // codes [M][K] (rows are 16-byte aligned; LDS keeps them densely, so chunk c lands at byte 16 * c) and the row
+        // scales [K-block][M] into [K-block][4]
+        const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A, (int64_t)(M - 1) * g.lda + K);
+        for (int c0 = wave * 64; c0 < total; c0 += 256) {
+            const int c = c0 + lane;
+            const uint32_t off = c < total ? (uint32_t)((c / cpr) * (int)g.lda + (c % cpr) * 16) : (uint32_t)kBufOut;
+            bi8_buffer_to_lds16(a_rsrc, lds0 + (uint32_t)(nblk_pad * 20) * 4 + (uint32_t)c0 * 16, off, 0);
+        }
+        const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA, (int64_t)nblk * M * 4);
+        for (int i0 = wave * 64; i0 < nblk_pad * 4; i0 += 256) {
+            const int i = i0 + lane, jb = i >> 2, m = i & 3;
+            const uint32_t off = (jb < nblk && m < M) ? (uint32_t)((jb * M + m) * 4) : (uint32_t)kBufOut;
+            bi8_buffer_to_lds4(sa_rsrc, lds0 + (uint32_t)i0 * 4, off, 0);
+        }
+    }
+    // (the compiler must not move the loads of W, which it knows to be plain loads, above the ones before)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    bi8_v4i w[CG][R];
+    auto load_w = [&](int c, int cc, int r) {      // run c of row 4 * wave + r into slot (cc, r)
+        const int k = c * 1024 + lane * 16;
+        const int voff = (k < K ? (4 * wave + r) * (int)g.ldw + k : kBufOut);          // past K: no access, zeros
+        w[cc][r] = bi8_buffer_load16(rw, voff, 0, true);
     };
 #pragma unroll
-    for (int d = 0; d < D; ++d) load_stage(d, wf[d], swf[d], std::true_type{});
+    for (int cc = 0; cc < CG; ++cc)
+#pragma unroll
+        for (int r = 0; r < R; ++r) load_w(cc, cc, r);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 
-    // x -> codes and scales in LDS.  Chunk c = 16 bytes of x; K % 128 == 0 makes every aligned group of L chunks one
-    // K-block of one row, and a group is either all inside x or all past its end.
-    const char *xb = (const char *)x;
-    const int cpr = K / VEC;                       // chunks per row
-    const int total = M * cpr;
-    for (int c0 = 0; c0 < total; c0 += 256 * U) {
-        bi8_v4u raw[U];
+    if constexpr (FUSED) {
+        // x [M,K] of type DT -> codes and scales, with the row quantizer's helpers (same results).  Chunk c = 16 bytes of
+        // x; K % 128 == 0 makes every aligned group of L chunks one K-block of one row.
+        constexpr int L = BLK / VEC;
+        constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
+        for (int c0 = 0; c0 < total; c0 += 256 * U) {
+            if (c0) load_x(c0);                    // (more than 8 chunks per thread: these loads queue behind the runs of W)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int c = c0 + u * 256 + tid;
-            raw[u] = bi8_v4u{0u, 0u, 0u, 0u};
-            if (c < total) raw[u] = *(const bi8_v4u *)(xb + ((int64_t)(c / cpr) * ldx + (int64_t)(c % cpr) * VEC) * ES);
-        }
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * 256 + tid;
+                if (c0 + u * 256 + (tid & ~63) >= total) break;        // wave-uniform: nothing left for this wave
+                const int row = c / cpr, col = (c % cpr) * VEC;
+                float f[VEC];
+                bi8_unpack<DT>(raw[u], f);
+                float m = 0.0f;
+                bool special = false;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int c = c0 + u * 256 + tid;
-            if (c0 + u * 256 + (tid & ~63) >= total) break;        // wave-uniform: nothing left for this wave
-            const int row = c / cpr, col = (c % cpr) * VEC;
-            float f[VEC];
-            bi8_unpack<DT>(raw[u], f);
-            float m = 0.0f;
-            bool special = false;
+                for (int e = 0; e < VEC; ++e) {
+                    m = __builtin_fmaxf(m, __builtin_fabsf(f[e]));
+                    special |= (f[e] != f[e]);
+                }
+                m = bi8_group_max<L>(m);
+                special |= !bi8_scale_is_ordinary(m);
+                uint32_t code[VEC];
+                if (__builtin_expect(special, 0)) {
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                m = __builtin_fmaxf(m, __builtin_fabsf(f[e]));
-                special |= (f[e] != f[e]);
-            }
-            m = bi8_group_max<L>(m);
-            special |= !bi8_scale_is_ordinary(m);
-            uint32_t code[VEC];
-            if (__builtin_expect(special, 0)) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) code[e] = bi8_code_slow(f[e], m);
-            } else {
-                const float y = 1.0f / m;
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) code[e] = bi8_code_fast<NCORR>(f[e], m, y);
-            }
-            if (c < total) {
-                if ((lane & (L - 1)) == 0) s_sx[(col / BLK) * 4 + row] = m;
-                int8_t *dst = s_a + row * K + col;
-                if constexpr (VEC == 4) {
-                    *(uint32_t *)dst = bi8_pack4(code[0], code[1], code[2], code[3]);
+                    for (int e = 0; e < VEC; ++e) code[e] = bi8_code_slow(f[e], m);
                 } else {
-                    *(bi8_v2u *)dst = bi8_v2u{bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
+                    const float y = 1.0f / m;
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) code[e] = bi8_code_fast<NCORR>(f[e], m, y);
+                }
+                if (c < total) {
+                    if ((lane & (L - 1)) == 0) s_sx[(col / BLK) * 4 + row] = m;
+                    int8_t *dst = s_a + row * K + col;
+                    if constexpr (VEC == 4) {
+                        *(uint32_t *)dst = bi8_pack4(code[0], code[1], code[2], code[3]);
+                    } else {
+                        *(bi8_v2u *)dst = bi8_v2u{bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
+                    }
                 }
             }
         }
+        for (int i = tid; i < nblk_pad * 4; i += 256)
+            if (i >= nblk * 4 || (i & 3) >= M) s_sx[i] = 0.0f;
     }
-    for (int i = tid; i < (nblk + NBS) * 4; i += 256)
-        if (i >= nblk * 4 || (i & 3) >= M) s_sx[i] = 0.0f;
-    __syncthreads();
+    // the direct-to-LDS loads were all issued before the sixteen runs of W
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (16 & 15) | ((16 >> 4) << 14));                   // vmcnt(16)
+    __builtin_amdgcn_s_waitcnt(0xC07F);                                                     // lgkmcnt(0): this wave's LDS writes
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
 
-    // the A operands follow the W ring one slot behind its refill: read from LDS a whole ring ahead of their use
-    // (MFMA lanes of rows >= M read row 0: an output row depends on its own A row only, and those rows are not stored)
-    const int8_t *arow = s_a + (r16 < M ? r16 : 0) * K + q * 16;
-    bi8_v4i af[D][2];
-    auto read_a = [&](int t, bi8_v4i *a) {
-        const int s = wave + NW * t;
-        const int sc = s < nstages ? s : nstages - 1;              // stages past the end fold with column scale 0
-        a[0] = *(const bi8_v4i *)(arow + sc * kStageK);
-        a[1] = *(const bi8_v4i *)(arow + sc * kStageK + 64);
-    };
+    float acc[R][MM];
 #pragma unroll
-    for (int d = 0; d < D; ++d) read_a(d, af[d]);
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    const int mine = (nstages - wave + NW - 1) / NW;
-    // D stages from the ring; REFILL 2: every slot refilled (those stages exist), 1: refilled with checked loads,
-    // 0: not refilled (the last group)
-    auto group = [&](int base, auto refill) {
-        constexpr int REFILL = decltype(refill)::value;
+    for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const int t = base + d;
-            const int s = wave + NW * t;
-            const int sb = (s < nstages ? s : nstages) * NBS;        // past the end: the stage of zero row scales
-            const bi8_v4i zero = {0, 0, 0, 0};
-            bi8_v4i p[NBS];
-            if constexpr (NBS == 1) {
-                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][0], wf[d][0], zero, 0, 0, 0);
-                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][1], wf[d][1], p[0], 0, 0, 0);
-            } else {
-                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][0], wf[d][0], zero, 0, 0, 0);
-                p[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][1], wf[d][1], zero, 0, 0, 0);
-            }
-            float swv[NBS];
+        for (int m = 0; m < MM; ++m) acc[r][m] = 0.0f;
+    const int8_t *a_lane = s_a + lane * 16;
+    const int grp = lane / LB;                     // this lane's K-block inside a run
+    // one group of CG runs: every slot is consumed (run, then row) and, with REFILL, loaded again with the run CG on
+    auto group = [&](int c0, auto refill) {
+        constexpr bool REFILL = decltype(refill)::value;
 #pragma unroll
-            for (int b = 0; b < NBS; ++b) swv[b] = swf[d][b];
-            if constexpr (REFILL == 2) load_stage(t + D, wf[d], swf[d], std::false_type{});
-            if constexpr (REFILL == 1) load_stage(t + D, wf[d], swf[d], std::true_type{});
-            if constexpr (REFILL != 0) read_a(t + D, af[d]);
+        for (int cc = 0; cc < CG; ++cc) {
+            const int c = c0 + cc;
+            const int kc = (c < nrun ? c : nrun - 1) * 1024;           // runs past the end: zero W against any codes ...
+            const int jb = (c < nrun ? c : nrun) * BPC + grp;          // ... and zero scales
+            bi8_v4i xa[MM];                                            // (rows past M: whatever the LDS holds, against zero scales)
 #pragma unroll
-            for (int b = 0; b < NBS; ++b) {
-                const bi8_v4f sx = *(const bi8_v4f *)(s_sx + (sb + b) * 4);
+            for (int m = 0; m < MM; ++m) xa[m] = *(const bi8_v4i *)(a_lane + m * K + kc);
+            const bi8_v4f sxv = *(const bi8_v4f *)(s_sx + jb * 4);
+            const bi8_v4f swv = *(const bi8_v4f *)(s_sw + jb * 16 + 4 * wave);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf((float)p[b][r] * sx[r], swv[b], acc[r]);
+            for (int r = 0; r < R; ++r) {
+                const bi8_v4i wv = w[cc][r];
+                if constexpr (REFILL) load_w(c + CG, cc, r);
+                const float swr = swv[r];
+#pragma unroll
+                for (int m = 0; m < MM; ++m) {
+                    int p = __builtin_amdgcn_sdot4(wv[0], xa[m][0], 0, false);
+                    p = __builtin_amdgcn_sdot4(wv[1], xa[m][1], p, false);
+                    p = __builtin_amdgcn_sdot4(wv[2], xa[m][2], p, false);
+                    p = __builtin_amdgcn_sdot4(wv[3], xa[m][3], p, false);
+                    p += bi8_dpp_i<0xB1>(p);                           // lanes ^1
+                    p += bi8_dpp_i<0x4E>(p);                           // lanes ^2
+                    if constexpr (LB == 8) p += bi8_dpp_i<0x141>(p);       // the other quad of the K-block (half-row mirror)
+                    acc[r][m] = __builtin_fmaf((float)p * sxv[m], swr, acc[r][m]);
+                }
             }
         }
     };
-    int base = 0;
-    for (; base + 2 * D <= mine; base += D) group(base, std::integral_constant<int, 2>{});
-    if (base + D < mine) {
-        group(base, std::integral_constant<int, 1>{});
-        base += D;
-    }
-    group(base, std::integral_constant<int, 0>{});
+    int c0 = 0;
+    for (; c0 + CG < nrun; c0 += CG) group(c0, std::true_type{});
+    group(c0, std::false_type{});
+
+    // every lane of a K-block's group holds the same sums: add up the groups (butterfly over the lane bits above a group)
+    const float div = (float)(1.0 / (127.0 * 127.0));
+    const bool has_bias = g.bias != nullptr;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
-    __syncthreads();
-    if (wave == 0 && q == 0) {                     // rows 0..3 live in lanes 0..15
-        const float div = (float)(1.0 / (127.0 * 127.0));
-        const bool has_bias = g.bias != nullptr;
+    for (int r = 0; r < R; ++r) {
+        const int64_t n = n0 + 4 * wave + r;
         const float bias = (has_bias && n < g.N) ? load_bias(g, n) : 0.0f;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float v = red[0][r][lane];
-#pragma unroll
-            for (int w = 1; w < NW; ++w) v += red[w][r][lane];
-            if (r < M && n < g.N) store_c<DT>(g.C, (int64_t)r * g.ldc + n, v * div, has_bias, bias);
+        for (int m = 0; m < MM; ++m) {
+            if (m < M) {
+                float v = acc[r][m];
+                if constexpr (LB == 4) v += bi8_dpp<0x141>(v);         // groups ^1 (lanes ^4: half-row mirror across the quads)
+                v += bi8_dpp<0x140>(v);                                // lanes ^8 (row mirror across the halves of a row)
+                v += __shfl_xor(v, 16, 64);
+                v += __shfl_xor(v, 32, 64);
+                if (lane == 0 && n < g.N) store_c<DT>(g.C, (int64_t)m * g.ldc + n, v * div, has_bias, bias);
+            }
         }
     }
 }
@@ -1842,10 +1892,10 @@ constexpr int kGemvMaxBlocks = 512;                // gemm_gemv keeps the row sc
 
 // ---- which kernel runs a problem ------------------------------------------------------------------------------------
 // One rule, used by the launcher, by bi8_gemm_workspace_bytes and by bi8_gemm_kernel_name.
-enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128 };
+enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows };
 static const char *const kGemmKernelNames[] = {"gemm_generic", "gemm_gemv", "gemm_skinny", "gemm_wide", "gemm_tile_256x128",
                                                 "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk",
-                                                "gemm_tile_64x128_splitk"};
+                                                "gemm_tile_64x128_splitk", "gemv_rows"};
 struct GemmPlan {
     int kernel;
     int splits, split_stages;      // of the split kernels: workgroups per tile along K and 128-byte stages of K per split
@@ -1867,6 +1917,11 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                          (block == 32 || block == 64 || block == 128);
     if (!tile_ok) return p;
     if (!partials) {
+        if (M <= kRowsMax && (block == 64 || block == 128) &&
+            (block == 64 ? rows_lds_bytes<64>(M, K) : rows_lds_bytes<128>(M, K)) <= kRowsLdsMax && (K / block + 16) * N * 4 < 0x7fffffffLL) {
+            p.kernel = kKRows;
+            return p;
+        }
         if (M <= 16 && (block == 64 || block == 128) && K / block <= kGemvMaxBlocks) {
             p.kernel = kKGemv;
             return p;
@@ -1927,6 +1982,15 @@ template <int BLK, int CDT> int launch_gemv(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
+template <int BLK, int CDT> int launch_rows(const GemmArgs &g, hipStream_t st) {
+    const int64_t tn = (g.N + 15) / 16;
+    if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
+    const size_t lds = rows_lds_bytes<BLK>(g.M, g.K);
+    if (rows_compiled_for(g.M) == 1) hipLaunchKernelGGL((gemv_rows<BLK, CDT, false, 1>), dim3((unsigned)tn), dim3(256), lds, st, g, nullptr, 0);
+    else hipLaunchKernelGGL((gemv_rows<BLK, CDT, false, 2>), dim3((unsigned)tn), dim3(256), lds, st, g, nullptr, 0);
+    return bi8_launch_rc();
+}
+
 template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, const GemmPlan &p, hipStream_t st) {
     constexpr int kRing = 3;                       // stage buffers of the tile kernels that are not software-pipelined
     switch (p.kernel) {
@@ -1940,6 +2004,9 @@ template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, co
     }
     if constexpr (!PARTIALS) {
         switch (p.kernel) {
+        case kKRows:
+            if constexpr (BLK != 32) return launch_rows<BLK, CDT>(g, st);
+            break;
         case kKGemv:
             if constexpr (BLK != 32) return launch_gemv<BLK, CDT>(g, st);
             break;
@@ -2067,8 +2134,14 @@ extern "C" const char *bi8_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int
 
 template <int DT> int launch_few_rows(const GemmArgs &g, const void *x, int64_t ldx, int block, size_t lds, hipStream_t st) {
     const unsigned tn = (unsigned)((g.N + 15) / 16);
-    if (block == 64) hipLaunchKernelGGL((linear_few_rows<64, DT>), dim3(tn), dim3(256), lds, st, g, x, ldx);
-    else hipLaunchKernelGGL((linear_few_rows<128, DT>), dim3(tn), dim3(256), lds, st, g, x, ldx);
+    const int mm = rows_compiled_for(g.M);
+    if (block == 64) {
+        if (mm == 1) hipLaunchKernelGGL((gemv_rows<64, DT, true, 1>), dim3(tn), dim3(256), lds, st, g, x, ldx);
+        else hipLaunchKernelGGL((gemv_rows<64, DT, true, 2>), dim3(tn), dim3(256), lds, st, g, x, ldx);
+    } else {
+        if (mm == 1) hipLaunchKernelGGL((gemv_rows<128, DT, true, 1>), dim3(tn), dim3(256), lds, st, g, x, ldx);
+        else hipLaunchKernelGGL((gemv_rows<128, DT, true, 2>), dim3(tn), dim3(256), lds, st, g, x, ldx);
+    }
     return bi8_launch_rc();
 }
 
@@ -2080,12 +2153,12 @@ extern "C" int bi8_linear_few_rows(const void *x, int dtype, const int8_t *W, co
     if (M < 0 || N < 0 || K < 0 || ldx < K || ldw < K || ldc < N) return BI8_ERR_BAD_SHAPE;
     if (!x || !W || !sW || !C) return BI8_ERR_NULL_POINTER;
     const int64_t vec = dtype == BI8_F32 ? 4 : 8;
-    if (M < 1 || M > kFewRowsMax || N < 1 || (block != 64 && block != 128) || K < kStageK || K % kStageK != 0 || ldx % vec != 0 ||
+    if (M < 1 || M > kRowsMax || N < 1 || (block != 64 && block != 128) || K < kStageK || K % kStageK != 0 || ldx % vec != 0 ||
         ldw % 16 != 0 || ldw >= (1 << 22) || (K / block) * N * 4 >= 0x7fffffffLL || !bi8_aligned(x, 16) || !bi8_aligned(W, 16) ||
         !bi8_aligned(sW, 4) || (N + 15) / 16 > 0x7fffffffLL)
         return BI8_ERR_UNSUPPORTED;
-    const size_t lds = (4 * 4 * 64 + (size_t)(K / block + kStageK / block) * 4) * sizeof(float) + (size_t)M * (size_t)K;
-    if (lds > kFewRowsLdsMax) return BI8_ERR_UNSUPPORTED;
+    const size_t lds = block == 64 ? rows_lds_bytes<64>(M, K) : rows_lds_bytes<128>(M, K);
+    if (lds > kRowsLdsMax) return BI8_ERR_UNSUPPORTED;
     GemmArgs g{nullptr, W, nullptr, sW, bias, C, nullptr, M, N, K, 0, ldw, ldc, 0, 0, bias_dtype};
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {

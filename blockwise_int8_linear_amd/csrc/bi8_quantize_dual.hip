@@ -9,6 +9,11 @@
 // registers: the lanes of one row reduce their absmax with DPP, quantize and store their codes.  The column direction
 // runs half by half through LDS exactly as in bi8_quantize_transposed (tile kept in its own type, 16-byte LDS accesses).  Both outputs are bit for bit those of the
 // two separate entry points.
+//
+// bi8_quantize_dual_colsum also returns the column sums of x (the bias gradient G.sum(dim=0) of block_linear.py:110,
+// when x is the output gradient G): the column walk has every element in a register anyway, so each thread adds up its
+// rows, the tile's row groups are added in ascending order, the tiles' sums go to a workspace [tile row][column] and a
+// second, tiny kernel adds them in ascending order (fp32 sums in a fixed order: deterministic) and casts.
 #include "bi8_common.h"
 
 namespace {
@@ -37,11 +42,12 @@ constexpr int kQPitch = kTR + 16;  // code tile pitch in bytes: rows stay 16-byt
 // ALIGNED: rows of x start on 16-byte boundaries and C is a multiple of the elements per 16 bytes, rows of q on 8-byte
 // boundaries.  Otherwise whole 16-byte chunks move with unaligned accesses and the last, partial chunk of a row
 // element by element.
-template <int DT, int B, bool ALIGNED>
+template <int DT, int B, bool ALIGNED, bool SUM>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == BI8_F32 ? 2 : 3))) void quantize_dual_tile(const void *__restrict__ x, int8_t *__restrict__ q,
                                                                float *__restrict__ scales, int8_t *__restrict__ qT,
-                                                               float *__restrict__ scalesT, int64_t R, int64_t C, int64_t ldx,
-                                                               int64_t ldq, int64_t ldqt, int64_t tiles_c, int64_t ntiles) {
+                                                               float *__restrict__ scalesT, float *__restrict__ colsum_part, int64_t R,
+                                                               int64_t C, int64_t ldx, int64_t ldq, int64_t ldqt, int64_t tiles_c,
+                                                               int64_t ntiles) {
     constexpr int VEC = Bi8Vec<DT>::kElems;
     constexpr int64_t ES = 16 / VEC;
     constexpr int LPR = kTC / VEC;                 // lanes per half row: 8 (16-bit) or 16 (fp32)
@@ -58,6 +64,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
     static_assert(B == 32 || B == 64 || B == 128, "tile = one or more whole blocks in both directions");
     __shared__ __attribute__((aligned(16))) uint8_t s_x[kTR * kXPitch];
     __shared__ float s_max[G][kTC];
+    __shared__ float s_sum[SUM ? G : 1][kTC];
     __shared__ __attribute__((aligned(16))) uint8_t s_q[kTC * kQPitch];
 
     const int tid = threadIdx.x;
@@ -201,10 +208,33 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
                     special |= (v[k][i] != v[k][i]);
                 }
             }
-            if constexpr (GPW > 1) {
+            if constexpr (SUM) {
+                // this thread's rows of its columns, top to bottom (rows past R were loaded as zeros)
+#pragma unroll
+                for (int k = 0; k < CPT; ++k) {
+                    float t = v[k][0];
+#pragma unroll
+                    for (int i = 1; i < RPT; ++i) t += v[k][i];
+                    s_sum[g][cw * CPT + k] = t;
+                }
+            }
+            if constexpr (GPW > 1 || SUM) {
 #pragma unroll
                 for (int k = 0; k < CPT; ++k) s_max[g][cw * CPT + k] = m[k];
                 __syncthreads();
+                if constexpr (SUM) {
+                    // the tile's row groups in ascending order; read before the barrier that follows phase 3, written
+                    // again after the one that follows the next phase 1
+                    if (g == 0) {
+#pragma unroll
+                        for (int k = 0; k < CPT; ++k) {
+                            float t = s_sum[0][cw * CPT + k];
+#pragma unroll
+                            for (int qg = 1; qg < G; ++qg) t += s_sum[qg][cw * CPT + k];
+                            if (c0 + cw * CPT + k < C) colsum_part[tr * C + c0 + cw * CPT + k] = t;
+                        }
+                    }
+                }
                 const int gb = g & ~(GPW - 1);
 #pragma unroll
                 for (int qg = 0; qg < GPW; ++qg)
@@ -265,8 +295,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
 }
 
 template <int DT, int B, bool ALIGNED>
-int launch_dual(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq,
-                int64_t ldqt, hipStream_t st) {
+int launch_dual(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, float *colsum_part, int64_t R, int64_t C, int64_t ldx,
+                int64_t ldq, int64_t ldqt, hipStream_t st) {
     const int64_t tiles_c = (C + 2 * kTC - 1) / (2 * kTC);
     const int64_t tiles_r = (R + kTR - 1) / kTR;
     const int64_t ntiles = tiles_c * tiles_r;
@@ -274,25 +304,72 @@ int launch_dual(const void *x, int8_t *q, float *scales, int8_t *qT, float *scal
     // bf16 [8192,8192]), three with fp32 (42 KiB)
     const int64_t resident = (DT == BI8_F32 ? 3 : 4) * 256;
     const int64_t grid = ntiles < resident ? ntiles : resident;
-    hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT, R, C,
-                       ldx, ldq, ldqt, tiles_c, ntiles);
+    if (colsum_part)
+        hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED, true>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT,
+                           colsum_part, R, C, ldx, ldq, ldqt, tiles_c, ntiles);
+    else
+        hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED, false>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT,
+                           colsum_part, R, C, ldx, ldq, ldqt, tiles_c, ntiles);
     return bi8_launch_rc();
 }
 
 template <int DT, bool ALIGNED>
-int dispatch(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C, int64_t ldx, int64_t ldq,
-             int64_t ldqt, int block, hipStream_t st) {
+int dispatch(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, float *colsum_part, int64_t R, int64_t C, int64_t ldx,
+             int64_t ldq, int64_t ldqt, int block, hipStream_t st) {
     switch (block) {
-    case 32: return launch_dual<DT, 32, ALIGNED>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
-    case 64: return launch_dual<DT, 64, ALIGNED>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
-    default: return launch_dual<DT, 128, ALIGNED>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, st);
+    case 32: return launch_dual<DT, 32, ALIGNED>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, st);
+    case 64: return launch_dual<DT, 64, ALIGNED>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, st);
+    default: return launch_dual<DT, 128, ALIGNED>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, st);
     }
+}
+
+// Column sums without the quantizer (the shapes that the one-pass kernel does not take): the same grouping of the
+// rows -- groups of kTR / G rows top to bottom, the groups of a 128-row tile in ascending order -- so that the sums
+// do not depend on which kernel made them.  One thread per column.
+template <int DT>
+__global__ __launch_bounds__(256) void colsum_tiles(const void *__restrict__ x, float *__restrict__ part, int64_t R, int64_t C, int64_t ldx) {
+    constexpr int RPT = (DT == BI8_F32) ? 32 : 16;
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t tr = blockIdx.y;
+    if (c >= C) return;
+    float total = 0.0f;
+    for (int g = 0; g < kTR / RPT; ++g) {
+        float t = 0.0f;
+        for (int i = 0; i < RPT; ++i) {
+            const int64_t r = tr * kTR + g * RPT + i;
+            const float v = r < R ? bi8_load_elem<DT>(x, r * ldx + c) : 0.0f;
+            t = i == 0 ? v : t + v;
+        }
+        total = g == 0 ? t : total + t;
+    }
+    part[tr * C + c] = total;
+}
+
+// out[c] = cast(sum over the row tiles, ascending)
+template <int DT>
+__global__ __launch_bounds__(256) void colsum_finish(const float *__restrict__ part, void *__restrict__ out, int64_t tiles_r, int64_t C) {
+    const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    float t = tiles_r > 0 ? part[c] : 0.0f;
+    for (int64_t tr = 1; tr < tiles_r; ++tr) t += part[tr * C + c];
+    bi8_store_elem<DT>(out, c, t);
+}
+
+template <int DT> int launch_colsum_finish(const float *part, void *out, int64_t tiles_r, int64_t C, hipStream_t st) {
+    hipLaunchKernelGGL((colsum_finish<DT>), dim3((unsigned)((C + 255) / 256)), dim3(256), 0, st, part, out, tiles_r, C);
+    return bi8_launch_rc();
+}
+template <int DT> int launch_colsum_tiles(const void *x, float *part, int64_t R, int64_t C, int64_t ldx, hipStream_t st) {
+    const int64_t tiles_r = (R + kTR - 1) / kTR;
+    if (tiles_r > 65535) return BI8_ERR_TOO_LARGE;
+    hipLaunchKernelGGL((colsum_tiles<DT>), dim3((unsigned)((C + 255) / 256), (unsigned)tiles_r), dim3(256), 0, st, x, part, R, C, ldx);
+    return bi8_launch_rc();
 }
 
 }  // namespace
 
-extern "C" int bi8_quantize_dual(const void *x, int x_dtype, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C,
-                                 int64_t ldx, int64_t ldq, int64_t ldqt, int block, void *stream) {
+static int quantize_dual(const void *x, int x_dtype, int8_t *q, float *scales, int8_t *qT, float *scalesT, float *colsum_part, int64_t R,
+                         int64_t C, int64_t ldx, int64_t ldq, int64_t ldqt, int block, void *stream) {
     if (x_dtype < 0 || x_dtype > 2) return BI8_ERR_BAD_DTYPE;
     if (block < 1 || block > (1 << 20)) return BI8_ERR_BAD_BLOCK;
     if (R < 0 || C < 0 || ldx < C || ldq < C || ldqt < R) return BI8_ERR_BAD_SHAPE;
@@ -304,22 +381,64 @@ extern "C" int bi8_quantize_dual(const void *x, int x_dtype, int8_t *q, float *s
     const bool one_pass = (block == 32 || block == 64 || block == 128) && bi8_aligned(x, esize) && ldqt % 16 == 0 && bi8_aligned(qT, 16);
     if (!one_pass) {
         // other block sizes, transposed rows of odd length: the two single-direction entry points, same results
-        const int rc = bi8_quantize_rowwise(x, x_dtype, q, scales, R, C, ldx, ldq, block, stream);
+        int rc = bi8_quantize_rowwise(x, x_dtype, q, scales, R, C, ldx, ldq, block, stream);
         if (rc != BI8_OK) return rc;
-        return bi8_quantize_transposed(x, x_dtype, qT, scalesT, R, C, ldx, ldqt, block, stream);
+        rc = bi8_quantize_transposed(x, x_dtype, qT, scalesT, R, C, ldx, ldqt, block, stream);
+        if (rc != BI8_OK || !colsum_part) return rc;
+        switch (x_dtype) {
+        case BI8_F32: return launch_colsum_tiles<BI8_F32>(x, colsum_part, R, C, ldx, (hipStream_t)stream);
+        case BI8_BF16: return launch_colsum_tiles<BI8_BF16>(x, colsum_part, R, C, ldx, (hipStream_t)stream);
+        default: return launch_colsum_tiles<BI8_F16>(x, colsum_part, R, C, ldx, (hipStream_t)stream);
+        }
     }
     const bool aligned = C % vec == 0 && ldx % vec == 0 && bi8_aligned(x, 16) && ldq % 8 == 0 && bi8_aligned(q, 8);
     hipStream_t st = (hipStream_t)stream;
     if (aligned) {
         switch (x_dtype) {
-        case BI8_F32: return dispatch<BI8_F32, true>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
-        case BI8_BF16: return dispatch<BI8_BF16, true>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
-        default: return dispatch<BI8_F16, true>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+        case BI8_F32: return dispatch<BI8_F32, true>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, block, st);
+        case BI8_BF16: return dispatch<BI8_BF16, true>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, block, st);
+        default: return dispatch<BI8_F16, true>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, block, st);
         }
     }
     switch (x_dtype) {
-    case BI8_F32: return dispatch<BI8_F32, false>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
-    case BI8_BF16: return dispatch<BI8_BF16, false>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
-    default: return dispatch<BI8_F16, false>(x, q, scales, qT, scalesT, R, C, ldx, ldq, ldqt, block, st);
+    case BI8_F32: return dispatch<BI8_F32, false>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, block, st);
+    case BI8_BF16: return dispatch<BI8_BF16, false>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, block, st);
+    default: return dispatch<BI8_F16, false>(x, q, scales, qT, scalesT, colsum_part, R, C, ldx, ldq, ldqt, block, st);
+    }
+}
+
+extern "C" int bi8_quantize_dual(const void *x, int x_dtype, int8_t *q, float *scales, int8_t *qT, float *scalesT, int64_t R, int64_t C,
+                                 int64_t ldx, int64_t ldq, int64_t ldqt, int block, void *stream) {
+    return quantize_dual(x, x_dtype, q, scales, qT, scalesT, nullptr, R, C, ldx, ldq, ldqt, block, stream);
+}
+
+extern "C" int64_t bi8_colsum_workspace_bytes(int64_t R, int64_t C) {
+    if (R <= 0 || C <= 0) return 0;
+    return ((R + kTR - 1) / kTR) * C * (int64_t)sizeof(float);
+}
+
+extern "C" int bi8_quantize_dual_colsum(const void *x, int x_dtype, int8_t *q, float *scales, int8_t *qT, float *scalesT, void *colsum,
+                                        void *workspace, int64_t workspace_bytes, int64_t R, int64_t C, int64_t ldx, int64_t ldq,
+                                        int64_t ldqt, int block, void *stream) {
+    if (x_dtype < 0 || x_dtype > 2) return BI8_ERR_BAD_DTYPE;
+    if (R < 0 || C < 0) return BI8_ERR_BAD_SHAPE;
+    if (C == 0) return BI8_OK;
+    if (!colsum) return BI8_ERR_NULL_POINTER;
+    if (R == 0) {                                  // an empty sum: zeros, written by the finishing kernel (no tiles to add)
+        switch (x_dtype) {
+        case BI8_F32: return launch_colsum_finish<BI8_F32>(nullptr, colsum, 0, C, (hipStream_t)stream);
+        case BI8_BF16: return launch_colsum_finish<BI8_BF16>(nullptr, colsum, 0, C, (hipStream_t)stream);
+        default: return launch_colsum_finish<BI8_F16>(nullptr, colsum, 0, C, (hipStream_t)stream);
+        }
+    }
+    if (!workspace || !bi8_aligned(workspace, 4)) return BI8_ERR_NULL_POINTER;
+    if (workspace_bytes < bi8_colsum_workspace_bytes(R, C)) return BI8_ERR_BAD_SHAPE;
+    const int rc = quantize_dual(x, x_dtype, q, scales, qT, scalesT, (float *)workspace, R, C, ldx, ldq, ldqt, block, stream);
+    if (rc != BI8_OK) return rc;
+    const int64_t tiles_r = (R + kTR - 1) / kTR;
+    switch (x_dtype) {
+    case BI8_F32: return launch_colsum_finish<BI8_F32>((const float *)workspace, colsum, tiles_r, C, (hipStream_t)stream);
+    case BI8_BF16: return launch_colsum_finish<BI8_BF16>((const float *)workspace, colsum, tiles_r, C, (hipStream_t)stream);
+    default: return launch_colsum_finish<BI8_F16>((const float *)workspace, colsum, tiles_r, C, (hipStream_t)stream);
     }
 }

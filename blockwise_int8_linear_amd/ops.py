@@ -123,7 +123,7 @@ def _code_buffer(rows: int, cols: int, device, pad: bool):
     return t, t
 
 
-def _quantize_block_dual(x: torch.Tensor, fblock_size, pad: bool):
+def _quantize_block_dual(x: torch.Tensor, fblock_size, pad: bool, colsum: bool = False):
     r, c = x.shape
     assert x.is_cuda
     x = _rows(_float_operand(x))
@@ -132,11 +132,30 @@ def _quantize_block_dual(x: torch.Tensor, fblock_size, pad: bool):
     qt, qt_store = _code_buffer(c, r, x.device, pad)
     s = torch.empty((ceil_div(c, fblock_size), r), device=x.device, dtype=torch.float32)
     st = torch.empty((ceil_div(r, fblock_size), c), device=x.device, dtype=torch.float32)
+    lib = _lib.load()
+    if colsum:
+        # the column sums of x from the same read (the bias gradient when x is the output gradient)
+        sums = torch.empty((c,), device=x.device, dtype=x.dtype)
+        ws = torch.empty((ceil_div(r, 128) * c,), device=x.device, dtype=torch.float32)
+        with _on_device(x):
+            rc = lib.bi8_quantize_dual_colsum(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), qt.data_ptr(), st.data_ptr(),
+                                              sums.data_ptr(), ws.data_ptr(), ws.numel() * 4, r, c, _ld(x), max(q_store.shape[1], 1),
+                                              max(qt_store.shape[1], 1), fblock_size, _stream(x))
+        _lib.check(rc, "bi8_quantize_dual_colsum")
+        return q, _scales_out(s), qt, _scales_out(st), q_store, qt_store, sums
     with _on_device(x):
-        rc = _lib.load().bi8_quantize_dual(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), qt.data_ptr(), st.data_ptr(),
-                                           r, c, _ld(x), max(q_store.shape[1], 1), max(qt_store.shape[1], 1), fblock_size, _stream(x))
+        rc = lib.bi8_quantize_dual(x.data_ptr(), _DT[x.dtype], q.data_ptr(), s.data_ptr(), qt.data_ptr(), st.data_ptr(),
+                                   r, c, _ld(x), max(q_store.shape[1], 1), max(qt_store.shape[1], 1), fblock_size, _stream(x))
     _lib.check(rc, "bi8_quantize_dual")
     return q, _scales_out(s), qt, _scales_out(st), q_store, qt_store
+
+
+def quantize_block_dual_colsum(x: torch.Tensor, fblock_size=None):
+    """``quantize_block_dual(x)`` plus ``x.sum(dim=0)`` (fp32 accumulation, result in x's dtype) from the same pass
+    over x: the output gradient's two quantizations and the bias gradient of block_linear.py:92, :101-103, :110.
+    Returns (q, scales, qT, scalesT, column sums)."""
+    out = _quantize_block_dual(x, fblock_size or block_linear_config.GROUP_SIZE, pad=False, colsum=True)
+    return out[0], out[1], out[2], out[3], out[6]
 
 
 def quantize_block_dual(x: torch.Tensor, fblock_size=None):
@@ -247,14 +266,20 @@ def _int8_matmul(a, b, state_x, state_w, bias=None, a_store=None, w_store=None):
     return c
 
 
-_FEW_ROWS = 4
+_FEW_ROWS = 2
 _FEW_ROWS_LDS = 64 * 1024
+
+
+def _few_rows_lds(M: int, K: int, block: int) -> int:
+    """LDS bytes of the few-row kernel: scales of the K-blocks (whole 1 KiB runs of K plus one) for 4 + 16 rows, the
+    activations' codes, 1 KiB of slack"""
+    return ceil_div((ceil_div(K, 1024) + 1) * (1024 // block), 16) * 16 * 80 + (1 if M <= 1 else 2) * K + 1024
 
 
 def linear_few_rows(x, W_int8, state_W, bias=None):
     """``quantize_block_rowwise(x)`` followed by ``int8_matmul_block64_rowwise_dequantize(x_int8, W_int8.t(),
     state_x, state_W, bias)`` (BlockInt8Linear.infer, block_linear.py:141-144) as ONE kernel, for the few-row case of
-    token-by-token decode: x [M,K] float with 1 <= M <= 4, W_int8 [N,K] and state_W [K/B, N] the cached weights.
+    token-by-token decode: x [M,K] float with 1 <= M <= 2, W_int8 [N,K] and state_W [K/B, N] the cached weights.
     Returns the same bits as the two launchers, or None when the operands are outside what the fused kernel covers
     (the caller then runs the two launchers)."""
     block = block_linear_config.GROUP_SIZE
@@ -263,7 +288,7 @@ def linear_few_rows(x, W_int8, state_W, bias=None):
     N = W_int8.shape[0]
     if not (1 <= M <= _FEW_ROWS and block in (64, 128) and K > 0 and K % 128 == 0 and N > 0 and x.dtype == dtype
             and x.dtype in _DT and W_int8.dtype == torch.int8 and state_W.dtype == torch.float32
-            and 4096 + 16 * (K // block + 128 // block) + M * K <= _FEW_ROWS_LDS):
+            and _few_rows_lds(M, K, block) <= _FEW_ROWS_LDS):
         return None
     assert x.is_cuda and W_int8.is_cuda
     assert W_int8.shape[1] == K and tuple(state_W.shape) == (K // block, N), "incompatible dimensions"

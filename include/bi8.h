@@ -87,6 +87,19 @@ int bi8_quantize_dual(const void *x, int x_dtype, int8_t *q, float *scales, int8
                       int64_t R, int64_t C, int64_t ldx, int64_t ldq, int64_t ldqt, int block, void *stream);
 
 /*
+ * bi8_quantize_dual that also returns the column sums of x: colsum[c] = cast(sum over r of x[r,c]), in x's type.
+ * With x = the output gradient G this is the backward pass's bias gradient, `grad_bias = G.sum(dim=0)`
+ * (block_linear.py:110), taken from the same read of G that quantizes it for the two gradient GEMMs (:92, :101-103).
+ * fp32 sums in a fixed order (rows top to bottom in groups, groups and 128-row tiles ascending): deterministic, and
+ * equal to torch's sum up to fp32 summation order.  `workspace`: bi8_colsum_workspace_bytes(R, C) bytes of scratch
+ * memory (ceil(R/128) * C floats), 4-byte aligned, used only by the kernels of this call.
+ */
+int64_t bi8_colsum_workspace_bytes(int64_t R, int64_t C);
+int bi8_quantize_dual_colsum(const void *x, int x_dtype, int8_t *q, float *scales, int8_t *qT, float *scalesT,
+                             void *colsum, void *workspace, int64_t workspace_bytes,
+                             int64_t R, int64_t C, int64_t ldx, int64_t ldq, int64_t ldqt, int block, void *stream);
+
+/*
  * Block dequantize.  Replaces dequantize_block_rowwise / _dequantize_block_rowwise
  * (triton_functions.py:492-500 / :468-490):  out = (scale * float(q)) * fp32(1/127), cast to out_dtype.
  */
@@ -166,15 +179,17 @@ int bi8_gemm_nt_partials(const int8_t *A, const int8_t *W, int32_t *P,
                          int block, void *stream);
 
 /*
- * Quantize + GEMM of the eval path in ONE launch for at most 4 rows (single-token decode).  Replaces the pair
+ * Quantize + GEMM of the eval path in ONE launch for one or two rows (single-token decode).  Replaces the pair
  * `quantize_block_rowwise(X)` + `int8_matmul_block64_rowwise_dequantize(X_int8, W_int8.t(), state_X, state_W, bias)`
- * of BlockInt8Linear.infer (block_linear.py:141-144) when X has 1..4 rows.
+ * of BlockInt8Linear.infer (block_linear.py:141-144) when X has 1 or 2 rows.
  *   x     [M,K] of `dtype`, leading dimension ldx   (activations, not yet quantized)
  *   W     int8 [N,K], leading dimension ldw;  sW fp32 [K/block, N]   (the cached weights, block_linear.py:127-128)
  *   C     [M,N] of the same `dtype`, leading dimension ldc;  bias [N] of bias_dtype or NULL
  * The result is bit for bit that of bi8_quantize_rowwise followed by bi8_gemm_nt_dequant on the same operands.
- * Covers 1 <= M <= 4, block 64 or 128, K a positive multiple of 128 with 4096 + 16*(K/block + 128/block) + M*K <= 65536 (the
- * quantized rows sit in LDS), x and W 16-byte aligned with ldx*sizeof(elem) and ldw multiples of 16; anything else
+ * Covers 1 <= M <= 2, block 64 or 128, K a positive multiple of 128 with
+ * 80 * roundup16((ceil(K/1024) + 1) * (1024/block)) + M*K + 1024 <= 65536 (the quantized rows and
+ * the scales sit in LDS), x and W
+ * 16-byte aligned with ldx*sizeof(elem) and ldw multiples of 16; anything else
  * returns BI8_ERR_UNSUPPORTED and the caller uses the two separate entry points.
  */
 int bi8_linear_few_rows(const void *x, int dtype, const int8_t *W, const float *sW,

@@ -33,7 +33,7 @@ def test_library_exports_every_declared_symbol():
                           "bi8_dequantize_rowwise", "bi8_gemm_nt_dequant", "bi8_gemm_nt_partials",
                           "bi8_linear_few_rows", "bi8_quantize_dual", "bi8_gemm_nt_dequant_ws",
                           "bi8_gemm_workspace_bytes", "bi8_gemm_kernel_name", "bi8_static_scratch_bytes",
-                          "bi8_gemm_nt_dequant_static"}
+                          "bi8_gemm_nt_dequant_static", "bi8_colsum_workspace_bytes", "bi8_quantize_dual_colsum"}
     lib = _lib.load()
     for name in decls:
         assert hasattr(lib, name), f"{name} not exported"
@@ -60,7 +60,7 @@ def test_ctypes_signatures_match_header():
 
 def test_version_and_error_strings():
     lib = _lib.load()
-    assert lib.bi8_version() == _lib.ABI_VERSION == 4
+    assert lib.bi8_version() == _lib.ABI_VERSION == 5
     assert lib.bi8_strerror(0) == b"success"
     assert b"block" in lib.bi8_strerror(3)
     with pytest.raises(_lib.Bi8Error, match="leading dimension"):
@@ -216,7 +216,9 @@ def test_kernel_choice_by_shape():
     assert name(2048, 4096, 4096, 128) == "gemm_tile_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
     assert name(2048, 2304, 512, 64) == "gemm_tile_256x128"
     assert name(300, 500, 512, 128) == "gemm_tile_128x128" and name(48, 700, 640, 128) == "gemm_tile_64x128"
-    assert name(1, 4096, 4096, 128) == "gemm_gemv" and name(16, 11008, 4096, 64) == "gemm_gemv"
+    assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
+    assert name(3, 4096, 4096, 128) == "gemm_gemv" and name(16, 11008, 4096, 64) == "gemm_gemv"
+    assert name(2, 4096, 32768, 128) == "gemm_gemv"                  # 2 x 32768 codes do not fit the few-row kernel's LDS
     assert name(16, 4096, 4096, 32) == "gemm_skinny" and name(24, 4096, 4096, 128) == "gemm_skinny"
     assert name(1, 128, 128 * 1024, 128) == "gemm_skinny"            # more K-blocks than the few-row kernel keeps scales for
     assert name(128, 4096, 4096, 128) == "gemm_tile_128x128"         # no scratch memory: one pass

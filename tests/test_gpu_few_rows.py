@@ -1,4 +1,4 @@
-"""The one-kernel quantize + GEMM of the eval path for 1..4 rows (bi8_linear_few_rows) against the two launchers it
+"""The one-kernel quantize + GEMM of the eval path for one or two rows (bi8_linear_few_rows) against the two launchers it
 replaces -- same bits -- and against the CPU checker; the cases it does not cover hand back to the two launchers."""
 import pytest
 import torch
@@ -39,8 +39,8 @@ def _weights(pkg, N, K, dtype, seed):
 
 @pytest.mark.parametrize("dtype", ["bf16", "f16", "f32"])
 @pytest.mark.parametrize("block", [64, 128])
-@pytest.mark.parametrize("M,K,N", [(1, 128, 16), (1, 4096, 4096), (2, 1024, 50), (3, 640, 1000), (4, 11008, 300),
-                                   (1, 11008, 4096), (4, 256, 17)])
+@pytest.mark.parametrize("M,K,N", [(1, 128, 16), (1, 4096, 4096), (2, 1024, 50), (2, 640, 1000), (2, 11008, 300),
+                                   (1, 11008, 4096), (2, 256, 17), (1, 5120, 33)])
 def test_same_bits_as_the_two_launchers(pkg, M, K, N, block, dtype):
     dt = DTYPES[dtype]
     with cfg_as(pkg, block, dt):
@@ -65,7 +65,7 @@ def test_same_bits_as_the_two_launchers(pkg, M, K, N, block, dtype):
 def test_special_blocks(pkg):
     """zero blocks, a NaN element, an inf element, subnormal and huge magnitudes: same codes and scales as the row
     quantizer, so the same output bits (NaN compares through the bit pattern)"""
-    M, K, N, block, dt = 3, 512, 64, 128, torch.float32
+    M, K, N, block, dt = 2, 768, 64, 128, torch.float32
     with cfg_as(pkg, block, dt):
         _, Wq, Ws = _weights(pkg, N, K, dt, seed=1)
         x = torch.randn(M, K, generator=torch.Generator().manual_seed(2))
@@ -73,7 +73,7 @@ def test_special_blocks(pkg):
         x[0, 130] = float("nan")
         x[1, 260] = float("inf")
         x[1, 384:512] *= 1e-42
-        x[2, 0:128] *= 1e35
+        x[0, 512:640] *= 1e35
         x = x.to(DEV)
         xq, xs = pkg.quantize_block_rowwise(x)
         two = pkg.int8_matmul_block64_rowwise_dequantize(xq, Wq.t(), xs, Ws)
@@ -101,7 +101,7 @@ def test_uncovered_cases_return_none(pkg):
     with cfg_as(pkg, 128, dt):
         _, Wq, Ws = _weights(pkg, 32, 256, dt, seed=6)
         x5 = torch.randn(5, 256).to(dt).to(DEV)
-        assert pkg.linear_few_rows(x5, Wq, Ws) is None                            # five rows
+        assert pkg.linear_few_rows(x5, Wq, Ws) is None and pkg.linear_few_rows(x5[:3], Wq, Ws) is None   # five rows, three rows
         assert pkg.linear_few_rows(x5[:1].float(), Wq, Ws) is None                # x not of the configured type
         xodd = torch.randn(1, 257).to(dt).to(DEV)[:, 1:]                          # rows not 16-byte aligned
         assert pkg.linear_few_rows(xodd, Wq, Ws) is None
@@ -109,7 +109,7 @@ def test_uncovered_cases_return_none(pkg):
         assert pkg.linear_few_rows(x5[:1], Wq, torch.ones(8, 32, device=DEV)) is None   # block 32
     with cfg_as(pkg, 128, dt):
         _, Wq, Ws = _weights(pkg, 16, 32768, dt, seed=7)
-        assert pkg.linear_few_rows(torch.randn(4, 32768).to(dt).to(DEV), Wq, Ws) is None   # 4 rows of 32 KiB exceed the LDS budget
+        assert pkg.linear_few_rows(torch.randn(2, 32768).to(dt).to(DEV), Wq, Ws) is None   # 2 rows of 32 KiB exceed the LDS budget
         one = pkg.linear_few_rows(torch.randn(1, 32768).to(dt).to(DEV), Wq, Ws)
         assert one is not None and torch.isfinite(one.float()).all()
 

@@ -315,9 +315,40 @@ def test_headline_shape_8192(ops, block):
     assert rel < 3e-2
 
 
+def _run_nonfinite_few_rows(ops, A, W, block, g):
+    """the same for the kernel of one or two rows: row 0 has an infinite scale in the last block and a NaN scale in
+    the first, row 1 an infinite scale on a block whose codes are all zero; then a column scale of inf"""
+    M, K = A.shape
+    N = W.shape[0]
+    nblk = K // block
+    j = nblk - 1
+    A[1, j * block:] = 0
+    sa = torch.rand(nblk, M, generator=g) + 0.1
+    sw = torch.rand(nblk, N, generator=g) * 0.05 + 1e-3
+    with cfg_as(ops, block, torch.float32):
+        run = lambda sa_, sw_: ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa_.to(DEV), sw_.to(DEV)).cpu()
+        sa2 = sa.clone()
+        sa2[j, 0] = sa2[j, 1] = float("inf")
+        ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa2, sw, block, None, torch.float32)
+        got = run(sa2, sw)
+        assert ref[1].isnan().all() and ref[0].isinf().sum() > N // 2
+        assert torch.equal(got.isnan(), ref.isnan()) and torch.equal(got[ref.isinf()], ref[ref.isinf()])
+        sa2[0, 0] = float("nan")
+        assert run(sa2, sw).isnan().all()
+        sw2 = sw.clone()
+        sw2[j, 2] = float("inf")
+        ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw2, block, None, torch.float32)
+        got = run(sa, sw2)
+        assert ref[1, 2].isnan() and ref[0, 2].isinf()
+        assert torch.equal(got.isnan(), ref.isnan()) and torch.equal(got[ref.isinf()], ref[ref.isinf()])
+        fin = torch.isfinite(ref)
+        assert ((got[fin] - ref[fin]).abs() <= 1e-3 * ref[fin].abs() + 1e-6).all()
+
+
 # (M, N, K, kernel family)
 NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (2048, 2304, 256, "gemm_tile_256x128"),
-                    (8, 256, 512, "gemm_gemv"), (24, 256, 512, "gemm_skinny"), (70, 90, 200, "gemm_generic")]
+                    (8, 256, 512, "gemm_gemv"), (24, 256, 512, "gemm_skinny"), (70, 90, 200, "gemm_generic"), (8, 256, 2560, "gemm_gemv_long"),
+                    (2, 256, 1536, "gemv_rows")]
 
 
 @pytest.mark.parametrize("shape", NONFINITE_SHAPES, ids=lambda s: s[3])
@@ -330,11 +361,14 @@ def test_infinite_and_nan_scales(ops, shape):
     from blockwise_int8_linear_amd import _lib
     M, N, K, family = shape
     block = 128 if K % 128 == 0 else 64
-    assert _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, 0).decode() == family
+    assert _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, 0).decode() == family.replace("_long", "")
     g = torch.Generator().manual_seed(M + N)
     A, W = _codes(g, M, K), _codes(g, N, K)
     nblk = -(-K // block)
     j = nblk - 1
+    if M <= 2:
+        _run_nonfinite_few_rows(ops, A, W, block, g)
+        return
     A[5, j * block:] = 0                            # this row's partial of block j is 0 for every column
     sa = torch.rand(nblk, M, generator=g) + 0.1
     sw = torch.rand(nblk, N, generator=g) * 0.05 + 1e-3
@@ -358,7 +392,7 @@ def test_infinite_and_nan_scales(ops, shape):
         ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw2, block, None, torch.float32)
         got = run(sa, sw2)
         assert ref[5, 2].isnan() and ref[:, 2].isinf().sum() >= M - 3
-        if family in ("gemm_gemv", "gemm_skinny", "gemm_generic"):
+        if family in ("gemm_gemv", "gemm_gemv_long", "gemm_skinny", "gemm_generic"):
             assert torch.equal(got.isnan(), ref.isnan()) and torch.equal(got[ref.isinf()], ref[ref.isinf()])
         else:
             assert got[:, 2].isnan().all()

@@ -96,3 +96,48 @@ def test_dual_empty(ops):
     e = torch.empty(0, 128, device=DEV, dtype=torch.bfloat16)
     q, s, qt, st = ops.quantize_block_dual(e, 128)
     assert q.shape == (0, 128) and s.shape == (1, 0) and qt.shape == (128, 0) and st.shape == (0, 128)
+
+
+def _colsum_bound(x_cpu, out_dtype):
+    """what a different fp32 summation order and the final cast can change: 2^-22 of the column's sum of magnitudes,
+    plus one unit in the last place of the output type"""
+    ulp = {torch.float32: 2.0 ** -23, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[out_dtype]
+    mag = x_cpu.double().abs().sum(0)
+    return 2.0 ** -22 * mag + ulp * x_cpu.double().sum(0).abs() + 1e-30
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("block", [32, 64, 128])
+def test_dual_with_column_sums(ops, dtype, block):
+    """bi8_quantize_dual_colsum: the same four outputs as bi8_quantize_dual bit for bit, and the column sums of x (the
+    bias gradient G.sum(dim=0), block_linear.py:110) in x's type; shapes of the one-pass kernel and of the fallbacks"""
+    for (R, C) in [(256, 256), (300, 1000), (1000, 72), (129, 64), (5, 8), (1, 4096), (8192, 768), (2181, 2115), (90, 77), (384, 1001)]:
+        x_cpu = torch.randn(R, C, generator=torch.Generator().manual_seed(R + C + block)).to(DTYPES[dtype])
+        x = x_cpu.to(DEV)
+        q, s, qt, st, sums = ops.quantize_block_dual_colsum(x, block)
+        q0, s0, qt0, st0 = ops.quantize_block_dual(x, block)
+        assert torch.equal(q, q0) and _same(s, s0) and torch.equal(qt, qt0) and _same(st, st0)
+        assert sums.shape == (C,) and sums.dtype == x.dtype
+        ref = x_cpu.sum(dim=0)                                   # the reference's expression, on the CPU
+        assert ((sums.cpu().double() - ref.double()).abs() <= _colsum_bound(x_cpu, x.dtype)).all()
+        # the sums do not depend on the block size or on which kernel made them (block 16 runs the fallback kernels)
+        assert _same(sums.float(), ops.quantize_block_dual_colsum(x, 16)[4].float())
+        # small integers add up exactly in any order
+        xi = torch.randint(-8, 9, (R, C), generator=torch.Generator().manual_seed(C)).to(DTYPES[dtype])
+        got = ops.quantize_block_dual_colsum(xi.to(DEV), block)[4]
+        assert torch.equal(got.cpu(), xi.double().sum(0).to(DTYPES[dtype]))
+
+
+def test_dual_with_column_sums_special_and_empty(ops):
+    x = torch.randn(300, 200, generator=torch.Generator().manual_seed(4))
+    x[7, 3] = float("inf")
+    x[9, 4] = float("nan")
+    x[11, 5] = float("inf"); x[200, 5] = float("-inf")
+    sums = ops.quantize_block_dual_colsum(x.to(DEV), 64)[4].cpu()
+    ref = x.sum(0)
+    assert sums[3] == float("inf") and sums[4].isnan() and sums[5].isnan()
+    ok = torch.isfinite(ref)
+    assert torch.equal(torch.isfinite(sums), ok) and ((sums[ok] - ref[ok]).abs() <= 1e-4).all()
+    e = torch.empty(0, 128, device=DEV, dtype=torch.bfloat16)
+    out = ops.quantize_block_dual_colsum(e, 128)
+    assert out[0].shape == (0, 128) and out[4].shape == (128,) and (out[4] == 0).all()
