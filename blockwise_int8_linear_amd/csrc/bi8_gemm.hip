@@ -1502,8 +1502,10 @@ constexpr size_t kRowsLdsMax = 64 * 1024;
 template <int BLK> constexpr int rows_blocks_padded(int64_t K) { return ((int)((K + 1023) / 1024 + 1) * (1024 / BLK) + 15) & ~15; }
 // the kernel is compiled for 1 and for 2 rows
 static inline int rows_compiled_for(int64_t M) { return M <= 1 ? 1 : 2; }
-template <int BLK> static size_t rows_lds_bytes(int64_t M, int64_t K) {
-    return (size_t)rows_blocks_padded<BLK>(K) * (4 + 16) * sizeof(float) + (size_t)rows_compiled_for(M) * (size_t)K + 1024;
+// x_bytes: size of an element of the un-quantized activations that the fused form stages in LDS (0: codes are given)
+template <int BLK> static size_t rows_lds_bytes(int64_t M, int64_t K, int64_t x_bytes) {
+    return (size_t)rows_blocks_padded<BLK>(K) * (4 + 16) * sizeof(float) + (size_t)rows_compiled_for(M) * (size_t)K + 1024 +
+           (size_t)M * (size_t)K * (size_t)x_bytes;
 }
 template <int CTRL> __device__ __forceinline__ int bi8_dpp_i(int v) { return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false); }
 
@@ -1543,23 +1545,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void g
         }
     }
     constexpr int VEC = FUSED ? Bi8Vec<DT>::kElems : 16;
-    constexpr int U = 8;                           // 16-byte loads of x in flight per lane (FUSED)
     const int cpr = K / VEC;                       // 16-byte chunks per row of activations
     const int total = M * cpr;
-    bi8_v4u raw[U];
-    auto load_x = [&](int c0) {
-        if constexpr (FUSED) {
-            constexpr int64_t ES = 16 / VEC;
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int c = c0 + u * 256 + tid;
-                raw[u] = bi8_v4u{0u, 0u, 0u, 0u};
-                if (c < total) raw[u] = *(const bi8_v4u *)((const char *)x + ((int64_t)(c / cpr) * ldx + (int64_t)(c % cpr) * VEC) * ES);
-            }
-        }
-    };
+    // FUSED: the un-quantized activations are staged in LDS behind the codes, chunk c at byte 16 * c
+    const uint32_t stage0 = lds0 + (uint32_t)(nblk_pad * 20) * 4 + (uint32_t)(MM * K + 1024);
     if constexpr (FUSED) {
-        load_x(0);
+        constexpr int ES = 16 / VEC;
+        const bi8_rsrc x_rsrc = bi8_make_rsrc(x, ((int64_t)(M - 1) * ldx + K) * ES);
+        for (int c0 = wave * 64; c0 < total; c0 += 256) {
+            const int c = c0 + lane;
+            const uint32_t off = c < total ? (uint32_t)(((c / cpr) * (int)ldx + (c % cpr) * VEC) * ES) : (uint32_t)kBufOut;
+            bi8_buffer_to_lds16(x_rsrc, stage0 + (uint32_t)c0 * 16, off, 0);
+        }
     } else {
         // codes [M][K] (rows are 16-byte aligned; LDS keeps them densely, so chunk c lands at byte 16 * c) and the row
         // scales [K-block][M] into [K-block][4]
@@ -1593,45 +1590,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void g
     __builtin_amdgcn_sched_barrier(0);
 
     if constexpr (FUSED) {
-        // x [M,K] of type DT -> codes and scales, with the row quantizer's helpers (same results).  Chunk c = 16 bytes of
-        // x; K % 128 == 0 makes every aligned group of L chunks one K-block of one row.
+        // x [M,K] of type DT -> codes and scales, with the row quantizer's helpers (same results).  Every wave works on
+        // the chunks that it fetched itself (they have landed once at most the sixteen runs of W are outstanding);
+        // K % 128 == 0 makes every aligned group of L chunks one K-block of one row.
         constexpr int L = BLK / VEC;
         constexpr int NCORR = (DT == BI8_F32) ? 2 : 1;
-        for (int c0 = 0; c0 < total; c0 += 256 * U) {
-            if (c0) load_x(c0);                    // (more than 8 chunks per thread: these loads queue behind the runs of W)
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (16 & 15) | ((16 >> 4) << 14));               // vmcnt(16)
+        const uint8_t *stage = (const uint8_t *)s_a + (size_t)MM * K + 1024;
+        for (int c0 = wave * 64; c0 < total; c0 += 256) {
+            const int c = c0 + lane;                                   // (total is a multiple of L: whole groups are in or out)
+            const bi8_v4u raw = c < total ? *(const bi8_v4u *)(stage + (size_t)c * 16) : bi8_v4u{0u, 0u, 0u, 0u};
+            const int row = c / cpr, col = (c % cpr) * VEC;
+            float f[VEC];
+            bi8_unpack<DT>(raw, f);
+            float m = 0.0f;
+            bool special = false;
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int c = c0 + u * 256 + tid;
-                if (c0 + u * 256 + (tid & ~63) >= total) break;        // wave-uniform: nothing left for this wave
-                const int row = c / cpr, col = (c % cpr) * VEC;
-                float f[VEC];
-                bi8_unpack<DT>(raw[u], f);
-                float m = 0.0f;
-                bool special = false;
+            for (int e = 0; e < VEC; ++e) {
+                m = __builtin_fmaxf(m, __builtin_fabsf(f[e]));
+                special |= (f[e] != f[e]);
+            }
+            m = bi8_group_max<L>(m);
+            special |= !bi8_scale_is_ordinary(m);
+            uint32_t code[VEC];
+            if (__builtin_expect(special, 0)) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    m = __builtin_fmaxf(m, __builtin_fabsf(f[e]));
-                    special |= (f[e] != f[e]);
-                }
-                m = bi8_group_max<L>(m);
-                special |= !bi8_scale_is_ordinary(m);
-                uint32_t code[VEC];
-                if (__builtin_expect(special, 0)) {
+                for (int e = 0; e < VEC; ++e) code[e] = bi8_code_slow(f[e], m);
+            } else {
+                const float y = 1.0f / m;
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) code[e] = bi8_code_slow(f[e], m);
+                for (int e = 0; e < VEC; ++e) code[e] = bi8_code_fast<NCORR>(f[e], m, y);
+            }
+            if (c < total) {
+                if ((lane & (L - 1)) == 0) s_sx[(col / BLK) * 4 + row] = m;
+                int8_t *dst = s_a + row * K + col;
+                if constexpr (VEC == 4) {
+                    *(uint32_t *)dst = bi8_pack4(code[0], code[1], code[2], code[3]);
                 } else {
-                    const float y = 1.0f / m;
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) code[e] = bi8_code_fast<NCORR>(f[e], m, y);
-                }
-                if (c < total) {
-                    if ((lane & (L - 1)) == 0) s_sx[(col / BLK) * 4 + row] = m;
-                    int8_t *dst = s_a + row * K + col;
-                    if constexpr (VEC == 4) {
-                        *(uint32_t *)dst = bi8_pack4(code[0], code[1], code[2], code[3]);
-                    } else {
-                        *(bi8_v2u *)dst = bi8_v2u{bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
-                    }
+                    *(bi8_v2u *)dst = bi8_v2u{bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
                 }
             }
         }
@@ -1918,7 +1914,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     if (!tile_ok) return p;
     if (!partials) {
         if (M <= kRowsMax && (block == 64 || block == 128) &&
-            (block == 64 ? rows_lds_bytes<64>(M, K) : rows_lds_bytes<128>(M, K)) <= kRowsLdsMax && (K / block + 16) * N * 4 < 0x7fffffffLL) {
+            (block == 64 ? rows_lds_bytes<64>(M, K, 0) : rows_lds_bytes<128>(M, K, 0)) <= kRowsLdsMax && (K / block + 16) * N * 4 < 0x7fffffffLL) {
             p.kernel = kKRows;
             return p;
         }
@@ -1985,7 +1981,7 @@ template <int BLK, int CDT> int launch_gemv(GemmArgs g, hipStream_t st) {
 template <int BLK, int CDT> int launch_rows(const GemmArgs &g, hipStream_t st) {
     const int64_t tn = (g.N + 15) / 16;
     if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-    const size_t lds = rows_lds_bytes<BLK>(g.M, g.K);
+    const size_t lds = rows_lds_bytes<BLK>(g.M, g.K, 0);
     if (rows_compiled_for(g.M) == 1) hipLaunchKernelGGL((gemv_rows<BLK, CDT, false, 1>), dim3((unsigned)tn), dim3(256), lds, st, g, nullptr, 0);
     else hipLaunchKernelGGL((gemv_rows<BLK, CDT, false, 2>), dim3((unsigned)tn), dim3(256), lds, st, g, nullptr, 0);
     return bi8_launch_rc();
@@ -2157,7 +2153,7 @@ extern "C" int bi8_linear_few_rows(const void *x, int dtype, const int8_t *W, co
         ldw % 16 != 0 || ldw >= (1 << 22) || (K / block) * N * 4 >= 0x7fffffffLL || !bi8_aligned(x, 16) || !bi8_aligned(W, 16) ||
         !bi8_aligned(sW, 4) || (N + 15) / 16 > 0x7fffffffLL)
         return BI8_ERR_UNSUPPORTED;
-    const size_t lds = block == 64 ? rows_lds_bytes<64>(M, K) : rows_lds_bytes<128>(M, K);
+    const size_t lds = block == 64 ? rows_lds_bytes<64>(M, K, bi8_dtype_size(dtype)) : rows_lds_bytes<128>(M, K, bi8_dtype_size(dtype));
     if (lds > kRowsLdsMax) return BI8_ERR_UNSUPPORTED;
     GemmArgs g{nullptr, W, nullptr, sW, bias, C, nullptr, M, N, K, 0, ldw, ldc, 0, 0, bias_dtype};
     hipStream_t st = (hipStream_t)stream;

@@ -270,10 +270,10 @@ _FEW_ROWS = 2
 _FEW_ROWS_LDS = 64 * 1024
 
 
-def _few_rows_lds(M: int, K: int, block: int) -> int:
-    """LDS bytes of the few-row kernel: scales of the K-blocks (whole 1 KiB runs of K plus one) for 4 + 16 rows, the
-    activations' codes, 1 KiB of slack"""
-    return ceil_div((ceil_div(K, 1024) + 1) * (1024 // block), 16) * 16 * 80 + (1 if M <= 1 else 2) * K + 1024
+def _few_rows_lds(M: int, K: int, block: int, elem_bytes: int) -> int:
+    """LDS bytes of the one-launch few-row kernel: scales of the K-blocks (whole 1 KiB runs of K plus one, in multiples
+    of 16) for 4 + 16 rows, the activations' codes, 1 KiB of slack, the un-quantized activations"""
+    return ceil_div((ceil_div(K, 1024) + 1) * (1024 // block), 16) * 16 * 80 + (1 if M <= 1 else 2) * K + 1024 + M * K * elem_bytes
 
 
 def linear_few_rows(x, W_int8, state_W, bias=None):
@@ -288,7 +288,7 @@ def linear_few_rows(x, W_int8, state_W, bias=None):
     N = W_int8.shape[0]
     if not (1 <= M <= _FEW_ROWS and block in (64, 128) and K > 0 and K % 128 == 0 and N > 0 and x.dtype == dtype
             and x.dtype in _DT and W_int8.dtype == torch.int8 and state_W.dtype == torch.float32
-            and _few_rows_lds(M, K, block) <= _FEW_ROWS_LDS):
+            and _few_rows_lds(M, K, block, x.element_size()) <= _FEW_ROWS_LDS):
         return None
     assert x.is_cuda and W_int8.is_cuda
     assert W_int8.shape[1] == K and tuple(state_W.shape) == (K // block, N), "incompatible dimensions"

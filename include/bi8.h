@@ -187,8 +187,8 @@ int bi8_gemm_nt_partials(const int8_t *A, const int8_t *W, int32_t *P,
  *   C     [M,N] of the same `dtype`, leading dimension ldc;  bias [N] of bias_dtype or NULL
  * The result is bit for bit that of bi8_quantize_rowwise followed by bi8_gemm_nt_dequant on the same operands.
  * Covers 1 <= M <= 2, block 64 or 128, K a positive multiple of 128 with
- * 80 * roundup16((ceil(K/1024) + 1) * (1024/block)) + M*K + 1024 <= 65536 (the quantized rows and
- * the scales sit in LDS), x and W
+ * 80 * roundup16((ceil(K/1024) + 1) * (1024/block)) + M*K*(1 + sizeof(elem)) + 1024 <= 65536 (x, its codes and the
+ * scales sit in LDS), x and W
  * 16-byte aligned with ldx*sizeof(elem) and ldw multiples of 16; anything else
  * returns BI8_ERR_UNSUPPORTED and the caller uses the two separate entry points.
  */

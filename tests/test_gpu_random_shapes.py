@@ -163,7 +163,7 @@ def test_few_rows_random(ops, seed):
         cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = old
     if one is None:
         from blockwise_int8_linear_amd.ops import _few_rows_lds
-        assert M > 2 or _few_rows_lds(M, K, block) > 65536, (M, K, N, block, dtype)
+        assert M > 2 or _few_rows_lds(M, K, block, x.element_size()) > 65536, (M, K, N, block, dtype)
     else:
         view = torch.int32 if dtype == "f32" else torch.int16
         assert torch.equal(one.view(view), two.view(view)), (M, K, N, block, dtype)
