@@ -80,6 +80,13 @@ __device__ __forceinline__ void bi8_buffer_to_lds16_sum(bi8_rsrc r, uint32_t lds
                  : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff_a), "s"(soff_b)
                  : "memory", "m0", "scc", "vcc");
 }
+// 64 lanes x one 16-bit element, each zero-extended into its own dword of LDS
+__device__ __forceinline__ void bi8_buffer_to_lds2(bi8_rsrc r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ushort %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(r), "s"(soff)
+                 : "memory", "m0", "vcc");
+}
 __device__ __forceinline__ void bi8_buffer_to_lds4(bi8_rsrc r, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :
@@ -105,6 +112,27 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tile
     tn = in / rows;
 }
 
+// The same order for a kernel that walks several tiles: pid is wave-uniform and every step stays on the scalar unit
+// (no division: band_magic = floor(2^32 / (kGroupM * tiles_n)) comes from the host).
+__device__ __forceinline__ void tile_of_workgroup_scalar(int pid, int tiles_m, int tiles_n, uint32_t band_magic, int &tm, int &tn) {
+    const int total = tiles_m * tiles_n;
+    const int per = total >> 3;
+    const int idx = pid < per * kXcds ? (pid & (kXcds - 1)) * per + (pid >> 3) : pid;
+    const int band = kGroupM * tiles_n;
+    int b = (int)__umulhi((uint32_t)idx, band_magic);          // floor(idx / band) or one less
+    int in = idx - b * band;
+    if (in >= band) {
+        in -= band;
+        ++b;
+    }
+    const int left = tiles_m - b * kGroupM;
+    const int rows = left < kGroupM ? left : kGroupM;          // 1 .. 4
+    static_assert(kGroupM == 4 && kXcds == 8, "the shifts below");
+    const int q = rows == 4 ? in >> 2 : rows == 3 ? (int)__umulhi((uint32_t)in, 0x55555556u) : rows == 2 ? in >> 1 : in;
+    tm = b * kGroupM + (in - q * rows);
+    tn = q;
+}
+
 template <int CDT> __device__ __forceinline__ void store_c(void *C, int64_t idx, float acc, bool has_bias, float bias) {
     float c = bi8_round_to<CDT>(acc);                      // acc.to(C.dtype)             triton_functions.py:127
     if (has_bias) c = c + bi8_round_to<CDT>(bias);         // + bias.to(C.dtype), in C's dtype   :129-131
@@ -125,6 +153,7 @@ struct GemmArgs {
     float *ws;
     int64_t ws_bytes;
     int splits, split_stages;
+    uint32_t band_magic;            // gemm_wide: floor(2^32 / (kGroupM * tiles_n))
 };
 
 __device__ __forceinline__ float load_bias(const GemmArgs &g, int64_t n) {
@@ -625,6 +654,10 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // and releases this stage's buffer to the loads of the stage after next.
 // Measured on MI355X: a SIMD issues about one instruction of any kind per 4 cycles, so the kernel is bound by its
 // instruction count; two fold instructions per output per K-block are 2/3 of it.
+// The grid is persistent, one workgroup per CU (the LDS admits no second one): a workgroup walks tiles b, b + grid, ...
+// of the XCD-aware order and never drains its pipeline between them, so a tile's outputs leave (through a small
+// wave-private LDS strip) while the next tile's first stages land.  Measured against one workgroup per tile:
+// 8192^3 -1.5 %, 8192 x 50257 x 768 -13 %.
 template <int NBS> struct WideLds {                 // NBS = K-blocks per stage
     static constexpr int kABuf = 256 * kStageK, kWBuf = 256 * kStageK;       // 32 KiB per operand per stage
     static constexpr int kSRow = 256 * 4;                                    // one row-scale row of the tile
@@ -640,8 +673,16 @@ template <int NBS> struct WideLds {                 // NBS = K-blocks per stage
     // after the K loop the same memory holds each wave's 64x128 tile of 16-bit outputs, row-major; the pitch
     // (256 + 16 bytes) puts the four row groups of one accumulator register into different banks
     static constexpr int kOutPitch = 272;
-    static constexpr int kDummy = kSWReg + 2 * kCBuf;                        // 1 KiB written and never read
+    static constexpr int kDummy = kSWReg + 2 * kCBuf;                        // gemm_wide32: 1 KiB written and never read
+    static constexpr int kBiasReg = kDummy;                                  // gemm_wide: the tile's bias, 256 x 4 bytes
     static constexpr int kStages = kDummy + 1024;                            // 135 / 141 KiB
+    // gemm_wide: next to the stage buffers every wave owns a strip of 16 rows x 64 columns of 16-bit outputs, through
+    // which its accumulators leave as row-major runs while the next tile's first stages are already landing in the
+    // stage buffers; the pitch (128 + 16 bytes) puts the four row groups of one accumulator register into different banks
+    static constexpr int kStripPitch = 144;
+    static constexpr int kStripBytes = 16 * kStripPitch;
+    static constexpr int kStrips = kStages;
+    static constexpr int kBytesPersistent = kStages + 8 * kStripBytes;       // 153 / 159 KiB of the CU's 160
     static constexpr int kOut = 8 * 64 * kOutPitch;                          // 136 KiB
     static constexpr int kBytes = kOut > kStages ? kOut : kStages;           // of the CU's 160 KiB
 };
@@ -660,18 +701,29 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     const int wm = wave >> 1, wn = wave & 1;
     const int r16 = lane & 15, q = lane >> 4;
 
-    int tile_m, tile_n;
-    tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
-    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    // The grid is persistent: workgroup b computes tiles b, b + gridDim.x, ... of the XCD-aware tile order, and the
+    // stage pipeline runs on across tile boundaries: while a tile's last two stages are computed the loader already
+    // fetches the first two stages of the workgroup's next tile, and they land while the accumulators leave.
+    const int ntiles = g.tiles_m * g.tiles_n;
     const int nstages = (int)(g.K / kStageK);
+    const int npairs = (nstages + 1) >> 1;         // the trip count is rounded up to even (see below)
+    int pid = blockIdx.x;                          // the tile being computed
+    int m0, n0;
+    {
+        int tile_m, tile_n;
+        tile_of_workgroup_scalar(pid, g.tiles_m, g.tiles_n, g.band_magic, tile_m, tile_n);
+        m0 = tile_m * BM;
+        n0 = tile_n * BN;
+    }
 
     // ---- loader (same scheme as gemm_tile): wave instruction i covers tile rows 8i .. 8i+7, lane -> row
     // 8i + lane/8, LDS chunk lane%8, which holds source chunk (lane%8) ^ ((row >> 1) & 7); i = wave + 8*it.
+    // One buffer per operand over the whole matrix (the host checks that each is below 2 GiB); the tile and the K
+    // position are scalar offsets.  Rows past the end of a matrix are past the end of its buffer and read as zeros.
     const int ld_row = lane >> 3;
     const int ld_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
-    const int64_t a_rows = (g.M - m0 < BM) ? (g.M - m0) : BM, w_rows = (g.N - n0 < BN) ? (g.N - n0) : BN;
-    const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
-    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
+    const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A, (g.M - 1) * g.lda + g.K);
+    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W, (g.N - 1) * g.ldw + g.K);
     const uint32_t a_off = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_off = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
     const uint32_t a_wave = (uint32_t)(wave * 8 * g.lda), w_wave = (uint32_t)(wave * 8 * g.ldw);
     const uint32_t a_step = (uint32_t)(NW * 8 * g.lda), w_step = (uint32_t)(NW * 8 * g.ldw);
@@ -679,9 +731,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     const int64_t nblk = g.K / BLK;
     const bool s_is_a = wave < 4;
     const int s_part = wave & 3;
-    const bi8_brsrc sa_brsrc = bi8_make_brsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
-    const bi8_brsrc sw_brsrc = bi8_make_brsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
-    const bi8_brsrc s_brsrc = s_is_a ? sa_brsrc : sw_brsrc;
+    const bi8_brsrc s_brsrc = s_is_a ? bi8_make_brsrc(g.sA, nblk * g.M * 4) : bi8_make_brsrc(g.sW, nblk * g.N * 4);
     const uint32_t s_off = (uint32_t)((s_part * 64 + lane) * 4);
     const uint32_t s_inc = (uint32_t)((s_is_a ? g.M : g.N) * 4);
     // The scales come into a register of the fetching lane, which stores them to LDS just before the barrier that
@@ -695,27 +745,45 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     for (int kb = 0; kb < NBS; ++kb) s_raw[kb] = 0.0f;
     const int c_dst = L::kSWReg + (s_part >> 1) * 1024 + (((2 * (s_part & 1) + (lane >> 5)) * 16 + (lane & 15)) * 2 + ((lane >> 4) & 1)) * 8;
     int p_dst0 = s_is_a ? L::kSAReg + (s_part * 64 + lane) * 4 : c_dst;
-    int p_dst1 = s_is_a ? L::kDummy + (s_part * 64 + lane) * 4 : c_dst + 4;
+    int p_dst1 = s_is_a ? L::kStrips + wave * L::kStripBytes + lane * 4 : c_dst + 4;     // the wave's strip is idle during the K loop
     const int p_buf0 = s_is_a ? L::kSBuf : L::kCBuf, p_row0 = s_is_a ? L::kSRow : L::kCRow;
     const int p_buf1 = s_is_a ? 0 : L::kCBuf, p_row1 = s_is_a ? 0 : L::kCRow;
-    uint32_t s_pos = 0, k_pos = 0;                 // scale-row and K position of the next stage to load
+    // The loader walks the stream of stages (this tile's, then the next tile's) at two positions one stage apart:
+    // E, where a stage gets its first kEarly loads (rows of A), and L, where it gets the others.  A position is the
+    // byte offset of (tile, K position) in each operand; all of them are wave-uniform.
+    uint32_t ao_E = (uint32_t)(m0 * g.lda), ao_L = ao_E, wo_L = (uint32_t)(n0 * g.ldw);
+    uint32_t so_L = (uint32_t)((s_is_a ? m0 : n0) * 4);
+    uint32_t ao_nxt = 0, wo_nxt = 0, so_nxt = 0;   // the workgroup's next tile
+    int m0_nxt = 0, n0_nxt = 0;
+    auto aim_next = [&](int p) {
+        int tile_m, tile_n;
+        // past the last tile: tile 0 once more, a stage or two loaded and never used
+        tile_of_workgroup_scalar(p < ntiles ? p : 0, g.tiles_m, g.tiles_n, g.band_magic, tile_m, tile_n);
+        m0_nxt = tile_m * BM;
+        n0_nxt = tile_n * BN;
+        ao_nxt = (uint32_t)(m0_nxt * g.lda);
+        wo_nxt = (uint32_t)(n0_nxt * g.ldw);
+        so_nxt = (uint32_t)((s_is_a ? m0_nxt : n0_nxt) * 4);
+    };
     constexpr int kLoadsPerStage = 4 + 4 + NBS;
     // A wave's nine or ten load instructions of a stage are spread out so that the texture path never sees all of
     // the workgroup's at once: the first kEarly right after the barrier that releases their buffer (last column
     // step of the stage two before), the others two per step during the first steps of the stage before.
     constexpr int kEarly = 3, kLateCols = (kLoadsPerStage - kEarly + 1) / 2;
+    static_assert(kEarly <= 4, "the early loads are rows of A");
+    // The stage in buffer F gives the stage after it (buffer G) its late loads, at L, and the stage after that
+    // (buffer F again) its early loads, at E.
 
     const uint32_t lds_base = bi8_lds_address(lds);
     // load instruction idx of a stage: 0-3 = A rows, 4-7 = W rows, 8.. = scale rows; the K position advances after the last
     auto issue_one = [&](int buf, int idx) {
         if (idx < 4) {
-            bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + idx * NW) * 1024, a_off, k_pos, a_wave + idx * a_step);
+            bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + idx * NW) * 1024, a_off, idx < kEarly ? ao_E : ao_L, a_wave + idx * a_step);
         } else if (idx < 8) {
-            bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + (idx - 4) * NW) * 1024, w_off, k_pos, w_wave + (idx - 4) * w_step);
+            bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + (idx - 4) * NW) * 1024, w_off, wo_L, w_wave + (idx - 4) * w_step);
         } else if (idx < kLoadsPerStage) {
-            s_raw[idx - 8] = bi8_buffer_load_f32(s_brsrc, (int)s_off, (int)s_pos);
-            s_pos += s_inc;
-            if (idx == kLoadsPerStage - 1) k_pos += kStageK;
+            s_raw[idx - 8] = bi8_buffer_load_f32(s_brsrc, (int)s_off, (int)so_L);
+            so_L += s_inc;
         }
     };
 
@@ -897,11 +965,27 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         }
     };
 
+    // 16-bit outputs: the bias of the tile's 256 columns waits in LDS for the tile's end, one dword per column (a
+    // 16-bit element zero-extended), fetched by waves 4-7, 64 columns each.  The waits and barriers of the stages
+    // that follow complete and publish it; columns past N read as zeros.
+    const bi8_rsrc bias_rsrc = bi8_make_rsrc(g.bias, g.bias ? g.N * (g.bias_dtype == BI8_F32 ? 4 : 2) : 0);
+    auto fetch_bias = [&]() {
+        if (wave >= 4) {
+            const uint32_t dst = lds_base + L::kBiasReg + (wave - 4) * 256, col = (uint32_t)(n0 + (wave - 4) * 64);
+            if (g.bias_dtype == BI8_F32) bi8_buffer_to_lds4(bias_rsrc, dst, (uint32_t)(lane * 4), col * 4);
+            else bi8_buffer_to_lds2(bias_rsrc, dst, (uint32_t)(lane * 2), col * 2);
+        }
+    };
+    if (CDT != BI8_F32 && g.bias != nullptr) fetch_bias();
+
     // prologue: the first stage's loads and the early part of the second's; wait for the first stage
 #pragma unroll
     for (int idx = 0; idx < kLoadsPerStage; ++idx) issue_one(0, idx);
+    ao_E += kStageK;
 #pragma unroll
     for (int idx = 0; idx < kEarly; ++idx) issue_one(1, idx);
+    ao_L = ao_E;
+    wo_L += kStageK;
     wait_vm(std::integral_constant<int, kEarly>{});
     publish_scales(0);
     __syncthreads();
@@ -913,76 +997,134 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     else read_bh(Bh[0], 0, 0);
     // The trip count is rounded up to even and loads run two stages ahead: stages past the end of K read their
     // scales through the buffers' range check as zeros, so they add exactly 0 to the accumulators.
-    for (int s = 0; s < nstages; s += 2) {
-        if constexpr (BLK == 128) {
-            stage(std::integral_constant<int, 0>{});
-            stage(std::integral_constant<int, 1>{});
-        } else {
-            stage64(std::integral_constant<int, 0>{});
-            stage64(std::integral_constant<int, 1>{});
-        }
-    }
-    wait_vm(std::integral_constant<int, 0>{});     // nothing may still be writing LDS when the wave ends
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {                  // the last column of the last (possibly padding) stage
-        fold2(cB[1][i], 0, sx[i], 7, acc[i][7]);
-        fold2(cB[1][i], 2, sx[i], 7, acc[i][7]);
-    }
-
     const float div = (float)(1.0 / (127.0 * 127.0));
     const bool has_bias = g.bias != nullptr;
-    if constexpr (CDT != BI8_F32) {
-        // 16-bit outputs leave through LDS: in the accumulator layout a store instruction would write 32-byte
-        // runs of four rows; from a row-major copy of the wave's 64x128 tile it writes 256-byte runs.
-        {
-            __syncthreads();                       // every wave is done with the stage buffers
-            uint8_t *tile = lds + wave * (64 * L::kOutPitch);
+    for (;;) {
+        aim_next(pid + (int)gridDim.x);
+        for (int pi = 0; pi < npairs; ++pi) {
+            // Stages 2pi (buffer 0) and 2pi + 1 (buffer 1).  In the tile's last pair E is in the next tile from the
+            // start, and L follows it there after the first of the two stages.
+            const bool last = pi == npairs - 1;
+            ao_E = last ? ao_nxt : ao_L + kStageK;
+            if constexpr (BLK == 128) stage(std::integral_constant<int, 0>{});
+            else stage64(std::integral_constant<int, 0>{});
+            ao_L = ao_E;
+            wo_L = last ? wo_nxt : wo_L + kStageK;
+            so_L = last ? so_nxt : so_L;
+            ao_E += kStageK;
+            if constexpr (BLK == 128) stage(std::integral_constant<int, 1>{});
+            else stage64(std::integral_constant<int, 1>{});
+            ao_L = ao_E;
+            wo_L += kStageK;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {              // the last column of the last (possibly padding) stage
+            fold2(cB[1][i], 0, sx[i], 7, acc[i][7]);
+            fold2(cB[1][i], 2, sx[i], 7, acc[i][7]);
+        }
+
+        if constexpr (CDT != BI8_F32) {
+            // 16-bit outputs leave through the wave's LDS strip, 16 rows x 64 columns at a time: in the accumulator
+            // layout a store instruction would write 32-byte runs of four rows; from the row-major strip it writes
+            // 128-byte runs.  The strip is the wave's own, so no barrier: LDS serves a wave's instructions in order.
+            // Nothing here waits for memory (the bias comes from LDS, addresses are rebuilt from the lane number
+            // rather than kept in registers across the K loop): the next tile's loads and this tile's stores stay in flight.
+            int lane_e = lane;
+            asm volatile("" : "+v"(lane_e));
+            const int er16 = lane_e & 15, eq = lane_e >> 4;
+            uint8_t *strip = lds + L::kStrips + wave * L::kStripBytes;
+            uint8_t *strip_w = strip + 4 * eq * L::kStripPitch + er16 * 2;
+            const uint8_t *strip_r = strip + (lane_e >> 3) * L::kStripPitch + (lane_e & 7) * 16;
+            const int row_e = lane_e >> 3, col_e = (lane_e & 7) * 8;        // of the strip, as read back
+            const int m_left = (int)(g.M - m0) - wm * 64 - row_e;             // rows 16i + 8p below this are inside C
+            const int n_e = n0 + wn * 128 + col_e;
+            uint8_t *c_tile = (uint8_t *)g.C + ((int64_t)(m0 + wm * 64) * g.ldc + n0 + wn * 128) * 2;
+            const uint32_t c_lane = (uint32_t)((row_e * g.ldc + col_e) * 2);
+            const uint8_t *bias_lds = lds + L::kBiasReg + (wn * 128 + er16) * 4;
+            auto leave = [&](auto with_bias_c) {
+                constexpr bool kBias = decltype(with_bias_c)::value;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int jh = 0; jh < 2; ++jh) {
+#pragma unroll
+                        for (int jj = 0; jj < 4; ++jj) {
+                            float bias = 0.0f;
+                            if constexpr (kBias) {
+                                const int j = 4 * jh + jj;
+                                const uint32_t raw = *(const uint32_t *)(bias_lds + j * 64);
+                                bias = g.bias_dtype == BI8_F32 ? bi8_u2f(raw) : g.bias_dtype == BI8_BF16 ? bi8_from_bf16_bits(raw) : bi8_from_f16_bits(raw);
+                                bias = bi8_round_to<CDT>(bias);
+                            }
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) {
+                                float v = bi8_round_to<CDT>(acc[i][4 * jh + jj][r] * div);    // acc.to(C.dtype), then + bias in C's dtype
+                                if constexpr (kBias) v = v + bias;
+                                const uint32_t bits = (CDT == BI8_BF16) ? bi8_bf16_bits(v) : bi8_f16_bits(v);
+                                *(uint16_t *)(strip_w + r * L::kStripPitch + jj * 32) = (uint16_t)bits;
+                            }
+                        }
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                        // lane -> row 8p + lane/8 of the strip, 8 outputs (16 bytes) at column 8 * (lane % 8)
+#pragma unroll
+                        for (int p = 0; p < 2; ++p) {
+                            const bi8_v4u v = *(const bi8_v4u *)(strip_r + 8 * p * L::kStripPitch);
+                            if (16 * i + 8 * p < m_left) {
+                                uint8_t *dst = c_tile + ((int64_t)(16 * i + 8 * p) * g.ldc + jh * 64) * 2 + c_lane;
+                                if (n_e + jh * 64 + 8 <= g.N) {
+                                    *(bi8_v4u_unaligned *)dst = v;          // rows of odd length start on 2-byte boundaries
+                                } else {
+#pragma nounroll
+                                    for (int e = 0; e < 8 && n_e + jh * 64 + e < g.N; ++e) ((uint16_t *)dst)[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+                                }
+                            }
+                        }
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                    }
+            };
+            if (has_bias) leave(std::true_type{});
+            else leave(std::false_type{});
+        } else {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const int64_t n = n0 + wn * 128 + j * 16 + r16;
-                const float bias = (has_bias && n < g.N) ? bi8_round_to<CDT>(load_bias(g, n)) : 0.0f;
+                const int64_t n = (int64_t)n0 + wn * 128 + j * 16 + r16;
+                const bool n_ok = n < g.N;
+                const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        float v = bi8_round_to<CDT>(acc[i][j][r] * div);      // acc.to(C.dtype), then + bias in C's dtype
-                        if (has_bias) v = v + bias;
-                        const uint32_t bits = (CDT == BI8_BF16) ? bi8_bf16_bits(v) : bi8_f16_bits(v);
-                        *(uint16_t *)(tile + (i * 16 + 4 * q + r) * L::kOutPitch + (j * 16 + r16) * 2) = (uint16_t)bits;
+                        const int64_t m = (int64_t)m0 + wm * 64 + i * 16 + 4 * q + r;
+                        if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[i][j][r] * div, has_bias, bias);
                     }
             }
-            // lane -> row 4p + lane/16 of the tile, 8 outputs (16 bytes) at column 8 * (lane % 16)
-            const int64_t n = n0 + wn * 128 + (lane & 15) * 8;
-#pragma unroll
-            for (int p = 0; p < 16; ++p) {
-                const int row = 4 * p + (lane >> 4);
-                const int64_t m = m0 + wm * 64 + row;
-                const bi8_v4u v = *(const bi8_v4u *)(tile + row * L::kOutPitch + (lane & 15) * 16);
-                if (m < g.M) {
-                    uint16_t *dst = (uint16_t *)g.C + m * g.ldc + n;
-                    if (n + 8 <= g.N) {
-                        *(bi8_v4u_unaligned *)dst = v;          // rows of odd length start on 2-byte boundaries
-                    } else {
-                        for (int e = 0; e < 8 && n + e < g.N; ++e) dst[e] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
-                    }
-                }
-            }
-            return;
         }
+
+        pid += (int)gridDim.x;
+        if (pid >= ntiles) break;
+        // The next tile: its first stage is published, its operands of column 0 are in A and Bf[0].  The first step
+        // folds "the column before" from an empty partial with zero scales, as at the start of the kernel.
+        m0 = m0_nxt;
+        n0 = n0_nxt;
+        if (CDT != BI8_F32 && has_bias) {
+            __syncthreads();                       // every wave has read the tile's bias
+            fetch_bias();
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            cB[1][i] = magic;
+            sx[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+        }
+        bc[1] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
     }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int64_t n = n0 + wn * 128 + j * 16 + r16;
-        const bool n_ok = n < g.N;
-        const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int64_t m = m0 + wm * 64 + i * 16 + 4 * q + r;
-                if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[i][j][r] * div, has_bias, bias);
-            }
-    }
+    wait_vm(std::integral_constant<int, 0>{});     // nothing may still be writing LDS when the wave ends
 }
 
 // ---- 256x256 tile on v_mfma_i32_32x32x32_i8 ---------------------------------------------------------------------------
@@ -1829,6 +1971,30 @@ struct LdsOptIn {
     }
 };
 
+// Compute units of the current device, rounded down to whole rounds over the XCDs so that a workgroup of a persistent
+// grid keeps to its own XCD's share of the tile order (looked up once per device).
+static int compute_units(int *out) {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return bi8_hip_rc(e);
+    int n = (dev >= 0 && dev < 64) ? cached[dev].load(std::memory_order_acquire) : 0;
+    if (n <= 0) {
+        e = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return bi8_hip_rc(e);
+        n = n >= kXcds ? n - n % kXcds : kXcds;
+        if (dev >= 0 && dev < 64) cached[dev].store(n, std::memory_order_release);
+    }
+    *out = n;
+    return BI8_OK;
+}
+
+// gemm_wide addresses each operand through one buffer with 32-bit offsets
+static bool wide_addressable(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block) {
+    const int64_t lim = 0x7fffffffLL, nblk = K / block;
+    return (M - 1) * lda + K <= lim && (N - 1) * ldw + K <= lim && nblk * M * 4 <= lim && nblk * N * 4 <= lim && M + 256 <= lim && N + 256 <= lim;
+}
+
 template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
 int launch_tile(GemmArgs g, hipStream_t st) {
     constexpr int kLds = TileLds<BM, BN, BLK, NBUF>::kBytes;
@@ -1853,11 +2019,17 @@ template <int BLK, int CDT> int launch_wide(GemmArgs g, hipStream_t st) {
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     g.tiles_m = (int)tm;
     g.tiles_n = (int)tn;
+    if (!wide_addressable(g.M, g.N, g.K, g.lda, g.ldw, BLK)) return BI8_ERR_TOO_LARGE;       // the plan does not send such a problem here
+    g.band_magic = (uint32_t)((1ull << 32) / (uint64_t)(kGroupM * tn));
     auto kern = gemm_wide<BLK, CDT>;
     static LdsOptIn opted;                         // one per kernel instantiation
-    const int rc = opted.ensure((const void *)kern, L::kBytes);
+    const int rc = opted.ensure((const void *)kern, L::kBytesPersistent);
     if (rc != BI8_OK) return rc;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn)), dim3(512), L::kBytes, st, g);
+    int cus = 0;
+    const int rc_cus = compute_units(&cus);
+    if (rc_cus != BI8_OK) return rc_cus;
+    const int64_t grid = tm * tn < cus ? tm * tn : cus;        // the kernel's LDS leaves room for one workgroup per CU
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), L::kBytesPersistent, st, g);
     return bi8_launch_rc();
 }
 
@@ -1927,7 +2099,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             return p;
         }
         // 256x256 tiles when there is enough work to fill the 256 CUs with them
-        if (((M + 255) / 256) * ((N + 255) / 256) >= kWideMinTiles) {
+        if (((M + 255) / 256) * ((N + 255) / 256) >= kWideMinTiles && (block == 32 || wide_addressable(M, N, K, lda, ldw, block))) {
             p.kernel = kKWide;
             return p;
         }

@@ -78,7 +78,8 @@ def test_gemm_golden(ops):
 # and with a single stage
 SHAPES = [(253, 257, 234), (129, 266, 75), (389, 138, 45), (256, 512, 512), (1, 384, 256), (16, 1000, 1024),
           (64, 128, 128), (48, 700, 640), (100, 300, 384), (300, 500, 512), (1024, 512, 512), (3584, 3584, 256), (3500, 3700, 384),
-          (2304, 4500, 1152), (2560, 4096, 128)]
+          (2304, 4500, 1152), (2560, 4096, 128),
+          (4400, 4501, 384)]       # 324 tiles of 256x256: more than one per workgroup of the persistent grid, ragged edges
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -346,7 +347,7 @@ def _run_nonfinite_few_rows(ops, A, W, block, g):
 
 
 # (M, N, K, kernel family)
-NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (2048, 2304, 256, "gemm_tile_256x128"),
+NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (4400, 4500, 256, "gemm_wide"), (2048, 2304, 256, "gemm_tile_256x128"),
                     (8, 256, 512, "gemm_gemv"), (24, 256, 512, "gemm_skinny"), (70, 90, 200, "gemm_generic"), (8, 256, 2560, "gemm_gemv_long"),
                     (2, 256, 1536, "gemv_rows")]
 

@@ -67,6 +67,8 @@ CASES = [
     (2944, 2900, 384, 128, "gemm_wide"),            # odd number of stages (the loop runs a padding stage), ragged N
     (2944, 2944, 512, 64, "gemm_wide"),             # two K-blocks per stage
     (2900, 2944, 384, 64, "gemm_wide"),
+    (4400, 4500, 384, 128, "gemm_wide"),            # 324 tiles: workgroups of the persistent grid walk on to a second tile
+    (4500, 4400, 256, 64, "gemm_wide"),
     (2944, 2944, 256, 32, "gemm_wide"),             # block 32: the 32x32x32-MFMA form, four K-blocks per stage
     (2900, 2944, 384, 32, "gemm_wide"),
     (2048, 2304, 512, 128, "gemm_tile_256x128"),    # the software-pipelined block-128 instantiation
