@@ -73,7 +73,10 @@ CASES = [
     (2900, 2944, 384, 32, "gemm_wide"),
     (2048, 2304, 512, 128, "gemm_tile_256x128"),    # the software-pipelined block-128 instantiation
     (2000, 2304, 384, 128, "gemm_tile_256x128"),
-    (2048, 2304, 512, 64, "gemm_tile_256x128"),
+    (2048, 4096, 512, 64, "gemm_tile_256x128"),
+    (2048, 2304, 512, 64, "gemm_tile_128x192"),     # 192 tiles of 128x192 against 144 of 256x128
+    (8192, 768, 256, 64, "gemm_tile_128x192"),      # 256 tiles of 128x192 where 256x128 tiles would be 192
+    (8100, 760, 384, 64, "gemm_tile_128x192"),
     (300, 500, 512, 128, "gemm_tile_128x128"),
     (300, 500, 512, 32, "gemm_tile_128x128"),
     (2304, 2304, 256, 32, "gemm_tile_128x128"),
