@@ -215,7 +215,7 @@ def test_kernel_choice_by_shape():
     assert name(2944, 2944, 512, 128) == "gemm_wide"                 # 12 x 12 = 144 tiles of 256x256
     assert name(8192, 768, 3072, 64) == "gemm_tile_128x192" and name(8192, 768, 3072, 128) == "gemm_tile_256x128"
     assert name(2048, 4096, 4096, 128) == "gemm_tile_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
-    assert name(2048, 2304, 512, 64) == "gemm_tile_256x128"
+    assert name(2048, 4096, 512, 64) == "gemm_tile_256x128" and name(2048, 2304, 512, 64) == "gemm_tile_128x192"
     assert name(300, 500, 512, 128) == "gemm_tile_128x128" and name(48, 700, 640, 128) == "gemm_tile_64x128"
     assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
     assert name(3, 4096, 4096, 128) == "gemm_gemv" and name(16, 11008, 4096, 64) == "gemm_gemv"
