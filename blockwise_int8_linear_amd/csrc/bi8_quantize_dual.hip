@@ -42,7 +42,9 @@ constexpr int kQPitch = kTR + 16;  // code tile pitch in bytes: rows stay 16-byt
 // ALIGNED: rows of x start on 16-byte boundaries and C is a multiple of the elements per 16 bytes, rows of q on 8-byte
 // boundaries.  Otherwise whole 16-byte chunks move with unaligned accesses and the last, partial chunk of a row
 // element by element.
-template <int DT, int B, bool ALIGNED, bool SUM>
+// NH: halves per tile.  2 is the tile described above; 1 (a 128 x 64 tile, blocks of at most 64) doubles the number of
+// workgroups for inputs too small to occupy the chip with full tiles.
+template <int DT, int B, bool ALIGNED, bool SUM, int NH>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == BI8_F32 ? 2 : 3))) void quantize_dual_tile(const void *__restrict__ x, int8_t *__restrict__ q,
                                                                float *__restrict__ scales, int8_t *__restrict__ qT,
                                                                float *__restrict__ scalesT, float *__restrict__ colsum_part, int64_t R,
@@ -62,6 +64,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
     constexpr int kXPitch = kTC * ESZ + (ESZ == 4 ? 0 : 16);   // bytes, 16-byte aligned (as in bi8_quantize_transposed)
     constexpr int LB = (B < kTC ? B : kTC) / VEC;  // lanes of one half row that share a row block
     static_assert(B == 32 || B == 64 || B == 128, "tile = one or more whole blocks in both directions");
+    static_assert(NH == 2 || (NH == 1 && B <= kTC), "a row block lies inside the tile");
     __shared__ __attribute__((aligned(16))) uint8_t s_x[kTR * kXPitch];
     __shared__ float s_max[G][kTC];
     __shared__ float s_sum[SUM ? G : 1][kTC];
@@ -77,7 +80,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
         int64_t tr = 0, tc = 0;
         if (tile < ntiles) tile_coords(tile, tiles_r, tiles_c, tr, tc);
         const int64_t r0 = tr * kTR;
-        const int64_t c0 = tc * (2 * kTC) + h * kTC;
+        const int64_t c0 = tc * (NH * kTC) + h * kTC;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             const int r = p * RPP + lr;
@@ -101,24 +104,24 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
         }
     };
 
-    bi8_v4u raw[2][NP];
-    load_half(blockIdx.x, 0, raw[0]);
-    load_half(blockIdx.x, 1, raw[1]);
+    bi8_v4u raw[NH][NP];
+#pragma unroll
+    for (int h = 0; h < NH; ++h) load_half(blockIdx.x, h, raw[h]);
     for (int64_t tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {
         int64_t tr, tc;
         tile_coords(tile, tiles_r, tiles_c, tr, tc);
         const int64_t r0 = tr * kTR;
-        const int64_t cbase = tc * (2 * kTC);
+        const int64_t cbase = tc * (NH * kTC);
 
         // ---- along the rows, from the registers ----------------------------------------------------------------
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             const int64_t row = r0 + p * RPP + lr;
-            float f[2][VEC];
-            float m[2];
-            bool special[2];
+            float f[NH][VEC];
+            float m[NH];
+            bool special[NH];
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int h = 0; h < NH; ++h) {
                 bi8_unpack<DT>(raw[h][p], f[h]);
                 m[h] = 0.0f;
                 special[h] = false;
@@ -129,13 +132,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
                 }
             }
             if constexpr (B == 2 * kTC) {
-                m[0] = m[1] = bi8_group_max<LPR>(__builtin_fmaxf(m[0], m[1]));
+                m[0] = m[NH - 1] = bi8_group_max<LPR>(__builtin_fmaxf(m[0], m[NH - 1]));
             } else {
-                m[0] = bi8_group_max<LB>(m[0]);
-                m[1] = bi8_group_max<LB>(m[1]);
+#pragma unroll
+                for (int h = 0; h < NH; ++h) m[h] = bi8_group_max<LB>(m[h]);
             }
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int h = 0; h < NH; ++h) {
                 const int64_t col = cbase + h * kTC + cc;
                 const bool live = row < R && col < C;
                 if (live && (tid % LB) == 0 && (B != 2 * kTC || h == 0)) scales[(col / B) * R + row] = m[h];
@@ -172,7 +175,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
 
         // ---- down the columns, one half at a time through LDS --------------------------------------------------
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
+        for (int h = 0; h < NH; ++h) {
             const int64_t c0 = cbase + h * kTC;
             // phase 1: this half -> LDS as it is (the previous half's column reads ended before the barrier that
             // precedes its phase 4); then start the next tile's loads of this half
@@ -297,18 +300,32 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
 template <int DT, int B, bool ALIGNED>
 int launch_dual(const void *x, int8_t *q, float *scales, int8_t *qT, float *scalesT, float *colsum_part, int64_t R, int64_t C, int64_t ldx,
                 int64_t ldq, int64_t ldqt, hipStream_t st) {
-    const int64_t tiles_c = (C + 2 * kTC - 1) / (2 * kTC);
     const int64_t tiles_r = (R + kTR - 1) / kTR;
-    const int64_t ntiles = tiles_c * tiles_r;
     // workgroups per CU: four with 16-bit inputs (29 KiB of LDS, under 128 registers: 62.7 us against 65.9 with three at
     // bf16 [8192,8192]), three with fp32 (42 KiB)
     const int64_t resident = (DT == BI8_F32 ? 3 : 4) * 256;
+    if constexpr (B <= kTC) {
+        // an input of fewer full tiles than the chip holds workgroups: half tiles, twice as many workgroups
+        const int64_t tiles_c1 = (C + kTC - 1) / kTC;
+        if (((C + 2 * kTC - 1) / (2 * kTC)) * tiles_r < resident) {
+            const int64_t ntiles = tiles_c1 * tiles_r, grid = ntiles < resident ? ntiles : resident;
+            if (colsum_part)
+                hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED, true, 1>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT,
+                                   scalesT, colsum_part, R, C, ldx, ldq, ldqt, tiles_c1, ntiles);
+            else
+                hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED, false, 1>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT,
+                                   scalesT, colsum_part, R, C, ldx, ldq, ldqt, tiles_c1, ntiles);
+            return bi8_launch_rc();
+        }
+    }
+    const int64_t tiles_c = (C + 2 * kTC - 1) / (2 * kTC);
+    const int64_t ntiles = tiles_c * tiles_r;
     const int64_t grid = ntiles < resident ? ntiles : resident;
     if (colsum_part)
-        hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED, true>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT,
+        hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED, true, 2>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT,
                            colsum_part, R, C, ldx, ldq, ldqt, tiles_c, ntiles);
     else
-        hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED, false>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT,
+        hipLaunchKernelGGL((quantize_dual_tile<DT, B, ALIGNED, false, 2>), dim3((unsigned)grid), dim3(kThreads), 0, st, x, q, scales, qT, scalesT,
                            colsum_part, R, C, ldx, ldq, ldqt, tiles_c, ntiles);
     return bi8_launch_rc();
 }
@@ -350,8 +367,16 @@ template <int DT>
 __global__ __launch_bounds__(256) void colsum_finish(const float *__restrict__ part, void *__restrict__ out, int64_t tiles_r, int64_t C) {
     const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
-    float t = tiles_r > 0 ? part[c] : 0.0f;
-    for (int64_t tr = 1; tr < tiles_r; ++tr) t += part[tr * C + c];
+    // sixteen independent loads at a time (a chain of dependent ones costs a memory latency each), added in order
+    float t = 0.0f;
+    for (int64_t t0 = 0; t0 < tiles_r; t0 += 16) {
+        float v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = t0 + i < tiles_r ? part[(t0 + i) * C + c] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            if (t0 + i < tiles_r) t = (t0 + i == 0) ? v[i] : t + v[i];
+    }
     bi8_store_elem<DT>(out, c, t);
 }
 

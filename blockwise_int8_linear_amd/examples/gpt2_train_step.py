@@ -2,7 +2,7 @@
 12 heads, MLP 3072, vocabulary 50257, context 1024, batch 8 x 1024 uniform-random tokens, AdamW on fp32 master
 weights (the model computes in bf16 copies refreshed from the masters every step).
 
-    python -m blockwise_int8_linear_amd.examples.gpt2_train_step [--steps 5]
+    python -m blockwise_int8_linear_amd.examples.gpt2_train_step [--steps 5] [--only int8|dense]
 
 Random-init weights (seed 0), synthetic tokens: this measures forward + backward (int8 grad-input and grad-weight
 GEMMs with transposed-block requantization, including the 50257-wide output layer) + optimizer, nothing about
@@ -111,13 +111,16 @@ def main():
     ap.add_argument("--ctx", type=int, default=1024)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--only", choices=["both", "dense", "int8"], default="both", help="which of the two models to run (profiling)")
     args = ap.parse_args()
     bi8.block_linear_config.GROUP_SIZE = 64
     bi8.block_linear_config.INPUT_OUTPUT_TORCH_TYPE = torch.bfloat16
     res = {"config": {k: getattr(args, k) for k in ("layers", "d_model", "heads", "vocab", "ctx", "batch")}, "block": 64,
            "dtype": "bf16 compute, fp32 master weights", "data": "synthetic"}
-    res["dense_bf16"] = run(False, args)
-    res["blockwise_int8"] = run(True, args)
+    if args.only != "int8":
+        res["dense_bf16"] = run(False, args)
+    if args.only != "dense":
+        res["blockwise_int8"] = run(True, args)
     print(json.dumps(res))
 
 
