@@ -11,8 +11,8 @@
 //                the int32 block partials;
 //   gemv_rows    M <= 2, blocks 64/128 (single-token decode; also bi8_linear_few_rows, which quantizes the activations in
 //                the same launch): one pass over W in 1 KiB runs of whole rows, v_dot4_i32_i8 on the vector unit;
-//   gemm_gemv    M <= 16, blocks 64/128 (small decode batches): one pass over W, 16 columns per workgroup, K split over
-//                4 waves, operands gathered from global memory through an 8-stage register ring;
+//   gemv_staged  M <= 16, blocks 64/128 (small decode batches): one pass over W, 16 columns per workgroup, K split over
+//                4 or 8 waves that each stream whole cache lines of W through a private LDS ring into 16x16x64 MFMAs;
 //   gemm_skinny  M <= 32 otherwise: the same idea with 32x32x32 MFMAs and one stage of lookahead;
 //   gemm_generic anything else (K not a multiple of 128, rows not 16-byte aligned, other block sizes): same
 //                MFMA, operands gathered straight from global memory with byte loads.
@@ -1498,112 +1498,133 @@ __global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
     }
 }
 
-// Few-row GEMM (M <= 16, blocks 64 and 128): decode.  HBM-bound on W; everything is arranged to keep many bytes of
-// W in flight.  One workgroup = 16 output columns, 4 waves that split K in interleaved 128-byte stages; a wave
-// gathers its operands straight from global memory in the layout of v_mfma_i32_16x16x64_i8 (16 bytes per lane:
-// 16 rows x 64 contiguous bytes per load instruction) through a ring of kDepth stages of registers, i.e. up to
-// kDepth * 2 KiB of W outstanding per wave.  The row scales of the whole problem (at most 16 rows) sit in LDS,
-// zero for rows >= M; the four partial accumulators are summed through LDS in wave order (deterministic).
-// Stages past the end of K load nothing and fold with column scale 0.
-constexpr int kGemvDepth = 8;                      // 4 and 6 measured the same
-template <int BLK, int CDT>
-__global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
-    constexpr int NW = 4, D = kGemvDepth;
-    constexpr int NBS = kStageK / BLK;             // K-blocks per stage: one MFMA (64 bytes of K) each when BLK = 64
+// ---- up to 16 rows, weight rows read as whole cache lines through LDS ----------------------------------------------------
+// Few-row GEMM (M <= 16, blocks 64 and 128): decode.  HBM-bound on W: one pass over the weight codes.  A load in MFMA
+// operand layout would fetch 64 bytes of 16 rows (half a cache line per row and instruction); here a wave's load
+// instruction fetches whole 128-byte lines (8 rows x 128 bytes, straight into LDS), and the operands are read back from
+// LDS in operand layout.  One workgroup = 16 output columns; its NW waves split K in interleaved 128-byte chunks and
+// never wait for one another: every wave owns a ring of kLdsGemvSlotsW stages of W (16 rows x 128 bytes each) with the
+// scales of their K-blocks, and a ring of two stages of A (all 16 rows, zeros past M).  The partial accumulators of
+// the waves are summed through LDS in wave order (deterministic).  Stages past the end of K load zeros (codes and
+// scales).  Measured at M = 16, block 128, against the same kernel with operands gathered from global memory in operand
+// layout through an 8-stage register ring: 4096 -> 11008 16.0 -> 12.8 us, 11008 -> 4096 17.1 -> 14.4 us.
+constexpr int kLdsGemvSlotsW = 4, kLdsGemvSlotsA = 2;
+constexpr int kLdsGemvSlot = 16 * 128;             // bytes of one stage of one operand
+constexpr int kLdsGemvScales = 256;                // bytes of one stage's scales: [K-block][16] column scales, then row scales
+constexpr size_t kLdsGemvWaveBytes = (size_t)(kLdsGemvSlotsW + kLdsGemvSlotsA) * kLdsGemvSlot + kLdsGemvSlotsW * kLdsGemvScales;
+template <int BLK, int CDT, int NW>
+__global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
+    constexpr int KW = 128;                        // bytes of K per wave and stage
+    constexpr int NSW = kLdsGemvSlotsW, NSA = kLdsGemvSlotsA;
+    constexpr int BPS = KW / BLK;                  // K-blocks per stage of a wave
+    constexpr int kSlot = kLdsGemvSlot;
     static_assert(BLK == 64 || BLK == 128, "one or two 64-byte MFMAs per K-block");
-    extern __shared__ __attribute__((aligned(16))) float gemv_lds[];
-    float(*red)[4][64] = (float(*)[4][64])gemv_lds;                 // [wave][register][lane]
-    float *s_sx = gemv_lds + NW * 4 * 64;                            // [K-block][16 rows], plus one stage of zeros
+    static_assert(NSW == 4 && NSA == 2, "the K loop is unrolled over the period of both rings");
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r16 = lane & 15, q = lane >> 4;
     const int64_t n0 = (int64_t)blockIdx.x * 16;
     const int64_t n = n0 + r16;
-    const int nstages = (int)(g.K / kStageK);
-    const int nblk = nstages * NBS;
-    // Buffer addressing: one VGPR offset per operand (this lane's row and 16-byte chunk), the stage's K offset in an
-    // SGPR, the half-stage as an immediate.  Rows past N and past M lie beyond the range and read as zeros.
-    const int64_t wrows = g.N - n0 < 16 ? g.N - n0 : 16;
-    const bi8_brsrc rw = bi8_make_brsrc(g.W + n0 * g.ldw, (wrows - 1) * g.ldw + g.K);
-    const bi8_brsrc ra = bi8_make_brsrc(g.A, (g.M - 1) * g.lda + g.K);
-    const bi8_brsrc rs = bi8_make_brsrc(g.sW, (int64_t)nblk * g.N * 4);
-    const int voff_w = r16 * (int)g.ldw + q * 16;
-    const int voff_a = r16 * (int)g.lda + q * 16;
-    const int voff_s = (int)(n < g.N ? n : g.N - 1) * 4;           // clamped: never stored
-    const int srow = (int)g.N * 4;
+    const int nchunks = (int)(g.K / KW);
+    const int nst = (((nchunks + NW - 1) / NW) + 3) & ~3;           // stages of every wave; those past the end of K load zeros
+    const int nblk = (int)(g.K / BLK);
+    constexpr int wave_bytes = (int)kLdsGemvWaveBytes;
+    uint8_t *mine = lds + wave * wave_bytes;
+    const uint32_t mine_addr = bi8_lds_address(lds) + (uint32_t)(wave * wave_bytes);
+    constexpr int kAReg = NSW * kSlot, kScReg = (NSW + NSA) * kSlot;
 
-    // stage t of this wave = global stage wave + NW * t; stages past the end are clamped and get column scale 0
-    bi8_v4i wf[D][2], af[D][2];
-    float swf[D][NBS];
-    // CHECKED loads give a stage past the end of K an offset beyond every buffer's range instead of a branch around
-    // them: they return zeros without touching memory (codes 0, column scale 0).
-    auto load_stage = [&](int t, bi8_v4i *w, bi8_v4i *a, float *sw, auto checked) {
-        const int s = wave + NW * t;
-        int kill = 0, sc = s;
-        if constexpr (decltype(checked)::value) {
-            kill = s < nstages ? 0 : kBufOut;                       // wave-uniform
-            sc = s < nstages ? s : nstages - 1;
-        }
-        const int k0 = sc * kStageK;
+    const int64_t wrows = g.N - n0 < 16 ? g.N - n0 : 16;
+    const bi8_rsrc rw = bi8_make_rsrc(g.W + n0 * g.ldw, (wrows - 1) * g.ldw + g.K);
+    const bi8_rsrc ra = bi8_make_rsrc(g.A, (g.M - 1) * g.lda + g.K);
+    const bi8_rsrc rsw = bi8_make_rsrc(g.sW, (int64_t)nblk * g.N * 4);
+    const bi8_rsrc rsa = bi8_make_rsrc(g.sA, (int64_t)nblk * g.M * 4);
+    // scales of a stage: lane -> K-block lane/16 of the stage's BPS, column (or row) lane%16; rows past M read as zeros
+    const uint32_t vsw = (uint32_t)((q * (int)g.N + (int)(n < g.N ? n : g.N - 1)) * 4);
+    const uint32_t vsa = r16 < g.M ? (uint32_t)((q * (int)g.M + r16) * 4) : (uint32_t)kBufOut;
+
+    // ---- loader: instruction i of a stage covers rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which
+    // holds source chunk (lane%8) ^ ((row >> 1) & 7) = (lane%8) ^ (lane/16) ^ 4i
+    const int ld_row = lane >> 3;
+    const int ld_chunk = (lane & 7) ^ ((lane >> 4) & 3);
+    uint32_t vw[2], va[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            w[kb] = bi8_buffer_load16(rw, voff_w + kill + kb * 64, k0, true);
-            a[kb] = bi8_buffer_load16(ra, voff_a + kill + kb * 64, k0, false);
-        }
+    for (int i = 0; i < 2; ++i) {
+        vw[i] = (uint32_t)((8 * i + ld_row) * (int)g.ldw + 16 * (ld_chunk ^ (4 * i)));
+        va[i] = (uint32_t)((8 * i + ld_row) * (int)g.lda + 16 * (ld_chunk ^ (4 * i)));
+    }
+    auto issue_w = [&](int s, int slot) {          // s, slot: wave-uniform; four load instructions
+        const int c = s * NW + wave;
+        const bool live = c < nchunks;
+        const uint32_t k0 = live ? (uint32_t)(c * KW) : (uint32_t)kBufOut;
 #pragma unroll
-        for (int b = 0; b < NBS; ++b) sw[b] = bi8_buffer_load_f32(rs, voff_s + kill, (sc * NBS + b) * srow);
+        for (int i = 0; i < 2; ++i) bi8_buffer_to_lds16(rw, mine_addr + slot * kSlot + i * 1024, vw[i], k0);
+        if (lane < 16 * BPS) {                     // (the loads write LDS for the active lanes only)
+            bi8_buffer_to_lds4(rsw, mine_addr + kScReg + slot * kLdsGemvScales, vsw, live ? (uint32_t)(c * BPS * (int)g.N * 4) : (uint32_t)kBufOut);
+            bi8_buffer_to_lds4(rsa, mine_addr + kScReg + slot * kLdsGemvScales + 128, vsa, live ? (uint32_t)(c * BPS * (int)g.M * 4) : (uint32_t)kBufOut);
+        }
     };
+    auto issue_a = [&](int s, int slot) {
+        const int c = s * NW + wave;
+        const uint32_t k0 = c < nchunks ? (uint32_t)(c * KW) : (uint32_t)kBufOut;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) bi8_buffer_to_lds16(ra, mine_addr + kAReg + slot * kSlot + i * 1024, va[i], k0);
+    };
+    // operand fragments: lane -> row r16, chunk 4j + q of the stage's eight, stored at (4j + q) ^ ((r16 >> 1) & 7)
+    const int frag = r16 * KW + ((q ^ ((r16 >> 1) & 7)) << 4);
+
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    const int mine = (nstages - wave + NW - 1) / NW;                // stages of this wave (wave < NW <= nstages not required)
+    // in flight at the top of stage s, oldest first: ..., A(s), W(s + NSW - 2)
 #pragma unroll
-    for (int d = 0; d < D; ++d) load_stage(d, wf[d], af[d], swf[d], std::true_type{});
-    // the row scales go to LDS while the first stages are on their way; one more stage of zeros behind them for the
-    // ring slots past the end of K (zero codes times a zero scale: a row scale of inf must not meet them)
-    for (int i = tid; i < (nblk + NBS) * 16; i += 256) {
-        const int jb = i >> 4, m = i & 15;
-        s_sx[i] = (jb < nblk && m < g.M) ? g.sA[(int64_t)jb * g.M + m] : 0.0f;
-    }
-    __syncthreads();
-    // D stages from the ring; REFILL 2: every slot is refilled (all of those stages exist), 1: refilled with checked
-    // loads, 0: not refilled (the last group).  Straight-line code in each form: a branch around single loads costs
-    // the register allocator dozens of copies.
-    auto group = [&](int base, auto refill) {
-        constexpr int REFILL = decltype(refill)::value;
+    for (int d = 0; d < NSW - 2; ++d) issue_w(d, d);
+    issue_a(0, 0);
+    issue_w(NSW - 2, NSW - 2);
+    auto stage = [&](int s, auto slot_c) {
+        constexpr int SW = decltype(slot_c)::value, SA = SW & 1;
+        issue_a(s + 1, SA ^ 1);
+        issue_w(s + NSW - 1, (SW + NSW - 1) % NSW);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | 10);   // vmcnt(10): everything up to A(s) has landed
+        const bi8_v4i zero = {0, 0, 0, 0};
+        bi8_v4i wf[2], af[2];
 #pragma unroll
-        for (int d = 0; d < D; ++d) {
-            const int t = base + d;
-            const int s = wave + NW * t;
-            const int sb = (s < nstages ? s : nstages) * NBS;        // past the end: the stage of zero row scales
-            const bi8_v4i zero = {0, 0, 0, 0};
-            bi8_v4i p[NBS];
-            if constexpr (NBS == 1) {
-                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][0], wf[d][0], zero, 0, 0, 0);
-                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][1], wf[d][1], p[0], 0, 0, 0);
-            } else {
-                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][0], wf[d][0], zero, 0, 0, 0);
-                p[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[d][1], wf[d][1], zero, 0, 0, 0);
-            }
-            float swv[NBS];
+        for (int j = 0; j < 2; ++j) {
+            wf[j] = *(const bi8_v4i *)(mine + SW * kSlot + (frag ^ (j << 6)));
+            af[j] = *(const bi8_v4i *)(mine + kAReg + SA * kSlot + (frag ^ (j << 6)));
+        }
+        bi8_v4i p[BPS];
+        if constexpr (BPS == 1) {
+            p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[0], wf[0], zero, 0, 0, 0);
+            p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[1], wf[1], p[0], 0, 0, 0);
+        } else {
+            p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[0], wf[0], zero, 0, 0, 0);
+            p[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[1], wf[1], zero, 0, 0, 0);
+        }
 #pragma unroll
-            for (int b = 0; b < NBS; ++b) swv[b] = swf[d][b];
-            if constexpr (REFILL == 2) load_stage(t + D, wf[d], af[d], swf[d], std::false_type{});
-            if constexpr (REFILL == 1) load_stage(t + D, wf[d], af[d], swf[d], std::true_type{});
+        for (int b = 0; b < BPS; ++b) {
+            const float sw = *(const float *)(mine + kScReg + SW * kLdsGemvScales + b * 64 + r16 * 4);
+            const bi8_v4f sx = *(const bi8_v4f *)(mine + kScReg + SW * kLdsGemvScales + 128 + b * 64 + q * 16);
 #pragma unroll
-            for (int b = 0; b < NBS; ++b) {
-                const bi8_v4f sx = *(const bi8_v4f *)(s_sx + (sb + b) * 16 + 4 * q);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf((float)p[b][r] * sx[r], swv[b], acc[r]);
-            }
+            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf((float)p[b][r] * sx[r], sw, acc[r]);
         }
     };
-    int base = 0;
-    for (; base + 2 * D <= mine; base += D) group(base, std::integral_constant<int, 2>{});
-    if (base + D < mine) {
-        group(base, std::integral_constant<int, 1>{});
-        base += D;
+    for (int s = 0; s < nst; s += NSW) {
+        stage(s, std::integral_constant<int, 0>{});
+        stage(s + 1, std::integral_constant<int, 1>{});
+        stage(s + 2, std::integral_constant<int, 2>{});
+        stage(s + 3, std::integral_constant<int, 3>{});
+        if constexpr (NSW > 4) {
+            stage(s + 4, std::integral_constant<int, 4>{});
+            stage(s + 5, std::integral_constant<int, 5>{});
+        }
+        if constexpr (NSW > 6) {
+            stage(s + 6, std::integral_constant<int, 6>{});
+            stage(s + 7, std::integral_constant<int, 7>{});
+        }
     }
-    group(base, std::integral_constant<int, 0>{});
+    __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): nothing may still be writing LDS when the rings are reused
+    __syncthreads();
+    float(*red)[4][64] = (float(*)[4][64])lds;     // [wave][register][lane], over the rings
 #pragma unroll
     for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
     __syncthreads();
@@ -1624,7 +1645,7 @@ __global__ __launch_bounds__(256) void gemm_gemv(const GemmArgs g) {
 
 // ---- one or two rows, weight rows read as whole runs -------------------------------------------------------------------
 // One or two rows of activations against all of W: single-token decode.  The problem is one pass over the N*K bytes of
-// weight codes and nothing else matters.  Gathering W in the operand layout of an MFMA (gemm_gemv: 16 rows x 64
+// weight codes and nothing else matters.  Gathering W in the operand layout of an MFMA (16 rows x 64
 // bytes per load instruction) reads 64-byte pieces of sixteen rows at a time, which this chip's memory pipeline serves
 // at 3.8 - 4.5 TB/s; whole 1 KiB runs of one row per load instruction (lane -> 16 consecutive bytes) come in at 5.3 -
 // 6.2 TB/s (a read-only micro-benchmark of the two patterns on the same grid).  With so few rows the matrix pipe has
@@ -2056,12 +2077,11 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
     return bi8_launch_rc();
 }
 
-constexpr int kGemvMaxBlocks = 512;                // gemm_gemv keeps the row scales in LDS: 64 bytes per K-block, 32 KiB at most
 
 // ---- which kernel runs a problem ------------------------------------------------------------------------------------
 // One rule, used by the launcher, by bi8_gemm_workspace_bytes and by bi8_gemm_kernel_name.
 enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKTile128x192 };
-static const char *const kGemmKernelNames[] = {"gemm_generic", "gemm_gemv", "gemm_skinny", "gemm_wide", "gemm_tile_256x128",
+static const char *const kGemmKernelNames[] = {"gemm_generic", "gemv_staged", "gemm_skinny", "gemm_wide", "gemm_tile_256x128",
                                                 "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk",
                                                 "gemm_tile_64x128_splitk", "gemv_rows", "gemm_tile_128x192"};
 struct GemmPlan {
@@ -2091,7 +2111,8 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             p.kernel = kKRows;
             return p;
         }
-        if (M <= 16 && (block == 64 || block == 128) && K / block <= kGemvMaxBlocks) {
+        if (M <= 16 && (block == 64 || block == 128) && (K / block + 16) * N * 4 < 0x3fffffffLL && 16 * ldw + K < 0x3fffffffLL &&
+            16 * lda + K < 0x3fffffffLL) {         // (gemv_staged addresses its buffers with 32-bit offsets)
             p.kernel = kKGemv;
             return p;
         }
@@ -2148,11 +2169,20 @@ template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-template <int BLK, int CDT> int launch_gemv(GemmArgs g, hipStream_t st) {
+template <int BLK, int CDT> int launch_staged(GemmArgs g, hipStream_t st) {
     const int64_t tn = (g.N + 15) / 16;
     if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-    const size_t lds = (4 * 4 * 64 + (size_t)(g.K / BLK + kStageK / BLK) * 16) * sizeof(float);
-    hipLaunchKernelGGL((gemm_gemv<BLK, CDT>), dim3((unsigned)tn), dim3(256), lds, st, g);
+    // eight waves per workgroup where four would leave CUs with a single workgroup's loads in flight
+    if (tn <= 384) {
+        constexpr size_t lds = 8 * kLdsGemvWaveBytes;
+        auto kern = gemv_staged<BLK, CDT, 8>;
+        static LdsOptIn opted;
+        const int rc = opted.ensure((const void *)kern, (int)lds);
+        if (rc != BI8_OK) return rc;
+        hipLaunchKernelGGL(kern, dim3((unsigned)tn), dim3(512), lds, st, g);
+    } else {
+        hipLaunchKernelGGL((gemv_staged<BLK, CDT, 4>), dim3((unsigned)tn), dim3(256), 4 * kLdsGemvWaveBytes, st, g);
+    }
     return bi8_launch_rc();
 }
 
@@ -2185,7 +2215,7 @@ template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, co
             if constexpr (BLK != 32) return launch_rows<BLK, CDT>(g, st);
             break;
         case kKGemv:
-            if constexpr (BLK != 32) return launch_gemv<BLK, CDT>(g, st);
+            if constexpr (BLK != 32) return launch_staged<BLK, CDT>(g, st);
             break;
         case kKSkinny: return launch_skinny<BLK, CDT>(g, st);
         case kKWide:

@@ -218,8 +218,8 @@ def test_kernel_choice_by_shape():
     assert name(2048, 4096, 512, 64) == "gemm_tile_256x128" and name(2048, 2304, 512, 64) == "gemm_tile_128x192"
     assert name(300, 500, 512, 128) == "gemm_tile_128x128" and name(48, 700, 640, 128) == "gemm_tile_64x128"
     assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
-    assert name(3, 4096, 4096, 128) == "gemm_gemv" and name(16, 11008, 4096, 64) == "gemm_gemv"
-    assert name(2, 4096, 32768, 128) == "gemm_gemv"                  # 2 x 32768 codes do not fit the few-row kernel's LDS
+    assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 11008, 4096, 64) == "gemv_staged"
+    assert name(2, 4096, 32768, 128) == "gemv_staged"                  # 2 x 32768 codes do not fit the few-row kernel's LDS
     assert name(16, 4096, 4096, 32) == "gemm_skinny" and name(24, 4096, 4096, 128) == "gemm_skinny"
     assert name(1, 128, 128 * 1024, 128) == "gemm_skinny"            # more K-blocks than the few-row kernel keeps scales for
     assert name(128, 4096, 4096, 128) == "gemm_tile_128x128"         # no scratch memory: one pass

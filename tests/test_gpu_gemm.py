@@ -348,7 +348,7 @@ def _run_nonfinite_few_rows(ops, A, W, block, g):
 
 # (M, N, K, kernel family)
 NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (4400, 4500, 256, "gemm_wide"), (2048, 2304, 256, "gemm_tile_256x128"),
-                    (8, 256, 512, "gemm_gemv"), (24, 256, 512, "gemm_skinny"), (70, 90, 200, "gemm_generic"), (8, 256, 2560, "gemm_gemv_long"),
+                    (8, 256, 512, "gemv_staged"), (24, 256, 512, "gemm_skinny"), (70, 90, 200, "gemm_generic"), (8, 256, 2560, "gemv_staged_long"),
                     (2, 256, 1536, "gemv_rows")]
 
 
@@ -393,7 +393,7 @@ def test_infinite_and_nan_scales(ops, shape):
         ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw2, block, None, torch.float32)
         got = run(sa, sw2)
         assert ref[5, 2].isnan() and ref[:, 2].isinf().sum() >= M - 3
-        if family in ("gemm_gemv", "gemm_gemv_long", "gemm_skinny", "gemm_generic"):
+        if family in ("gemv_staged", "gemv_staged_long", "gemm_skinny", "gemm_generic"):
             assert torch.equal(got.isnan(), ref.isnan()) and torch.equal(got[ref.isinf()], ref[ref.isinf()])
         else:
             assert got[:, 2].isnan().all()

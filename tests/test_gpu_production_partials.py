@@ -1,7 +1,7 @@
 """The int32 block partials of the kernels that produce the shipped outputs, recovered bit for bit.
 
 bi8_gemm_nt_partials runs its own kernel instantiations; the kernels behind bi8_gemm_nt_dequant (gemm_wide, the
-software-pipelined gemm_tile, gemm_gemv, gemm_skinny, the split of K) and bi8_linear_few_rows fold every partial
+software-pipelined gemm_tile, gemv_staged, gemm_skinny, the split of K) and bi8_linear_few_rows fold every partial
 into an fp32 accumulator straight away and never store it.  Here each of them is made to hand a partial back through
 its output: column scales all 1, row scales 1 for ONE K-block j and 0 for every other block, so that
 
@@ -84,9 +84,9 @@ CASES = [
     (1, 384, 512, 128, "gemv_rows"),
     (2, 1000, 4096 + 384, 128, "gemv_rows"),        # more than four runs of 1 KiB per row, the last one partial
     (2, 700, 2048 + 128, 64, "gemv_rows"),
-    (3, 384, 512, 128, "gemm_gemv"),
-    (16, 1000, 4096, 128, "gemm_gemv"),             # longer than the few-row kernel's register ring
-    (7, 1000, 1152, 64, "gemm_gemv"),
+    (3, 384, 512, 128, "gemv_staged"),
+    (16, 1000, 4096, 128, "gemv_staged"),           # eight stages per wave
+    (7, 1000, 1152, 64, "gemv_staged"),
     (24, 500, 2048, 128, "gemm_skinny"),
     (16, 300, 1024, 32, "gemm_skinny"),
     (128, 1024, 4096, 128, "gemm_tile_64x128_splitk"),
