@@ -79,7 +79,8 @@ def test_gemm_golden(ops):
 SHAPES = [(253, 257, 234), (129, 266, 75), (389, 138, 45), (256, 512, 512), (1, 384, 256), (16, 1000, 1024),
           (64, 128, 128), (48, 700, 640), (100, 300, 384), (300, 500, 512), (1024, 512, 512), (3584, 3584, 256), (3500, 3700, 384),
           (2304, 4500, 1152), (2560, 4096, 128),
-          (4400, 4501, 384)]       # 324 tiles of 256x256: more than one per workgroup of the persistent grid, ragged edges
+          (4400, 4501, 384),       # 324 tiles of 256x256: more than one per workgroup of the persistent grid, ragged edges
+          (5, 130, 66048)]         # a long contraction for the few-row kernel: 516 stages
 
 
 @pytest.mark.parametrize("shape", SHAPES)
