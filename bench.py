@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0          # HBM3E, 8 TB/s
 # WRITE_SIZE of rocprofv3 --pmc runs of this file, scaled by what the same counters read for a 256 MiB copy
 # (x2.0 and x1.0); the runs and figures are in profiles/gemm_wide_8192x8192x8192_block128.md.  Counters cannot be read
 # from inside the process, so this is a constant from those runs, labelled as such in the output ("traffic_source").
-GEMM_8192_TRAFFIC_BYTES = 980817527
+GEMM_8192_TRAFFIC_BYTES = 965859463
 GEMM_8192_TRAFFIC_SOURCE = ("profiles/gemm_wide_8192x8192x8192_block128.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
                             "command, scaled by a 256 MiB copy; a constant, not measured in this run")
 PREROLL_MAX = 400              # launches
@@ -242,6 +242,21 @@ def bench_extras(pkg, torch):
     nbytes = M * K * 4 + 8 * M * K // 128
     out["quantize_dual_bf16_8192"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
                                       "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
+
+    # Context, not part of the path: what a plain device-to-device copy of the same 128 MiB (the dual quantizer's input;
+    # it writes as many bytes again) reaches on this chip, three buffer pairs in rotation.  A kernel that reads and
+    # writes equal amounts has this, not the 8 TB/s of the data sheet, as its practical ceiling.
+    ds = [torch.empty_like(x) for x in xs]
+
+    def cp():
+        i = turn[0] = (turn[0] + 1) % 3
+        ds[i].copy_(xs[i])
+    for _ in range(6):
+        cp()
+    t = min(event_ms(cp, 30) for _ in range(2))
+    nbytes = 2 * xs[0].numel() * xs[0].element_size()
+    out["context_device_copy_128MiB"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
+                                         "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4), "what": "torch dst.copy_(src), read + write"}
     return out
 
 

@@ -69,6 +69,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
     __shared__ float s_max[G][kTC];
     __shared__ float s_sum[SUM ? G : 1][kTC];
     __shared__ __attribute__((aligned(16))) uint8_t s_q[kTC * kQPitch];
+    // the tile's row-direction scales, [block along the row][tile row]: stored from here as runs of kTR consecutive rows
+    // (single 4-byte stores from the lanes that hold them cost the fabric a 32-byte write each)
+    constexpr int NRB = (NH * kTC + B - 1) / B;
+    __shared__ float s_rs[NRB][kTR];
 
     const int tid = threadIdx.x;
     const char *xb = (const char *)x;
@@ -141,7 +145,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
             for (int h = 0; h < NH; ++h) {
                 const int64_t col = cbase + h * kTC + cc;
                 const bool live = row < R && col < C;
-                if (live && (tid % LB) == 0 && (B != 2 * kTC || h == 0)) scales[(col / B) * R + row] = m[h];
+                if ((tid % LB) == 0 && (B != 2 * kTC || h == 0)) s_rs[(h * kTC + cc) / B][p * RPP + lr] = m[h];
                 const bool slow = special[h] | !bi8_scale_is_ordinary(m[h]);
                 uint32_t code[VEC];
                 if (__builtin_expect(slow, 0)) {
@@ -183,6 +187,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
             for (int p = 0; p < NP; ++p) *(bi8_v4u *)&s_x[(p * RPP + lr) * kXPitch + (tid % LPR) * 16] = raw[h][p];
             load_half(tile + gridDim.x, h, raw[h]);
             __syncthreads();
+            if (h == 0) {
+                for (int i = tid; i < NRB * kTR; i += kThreads) {
+                    const int b = i / kTR, r = i % kTR;
+                    if (r0 + r < R && cbase + b * B < C) scales[(cbase / B + b) * R + r0 + r] = s_rs[b][r];
+                }
+            }
 
             // phase 2: column maxima over this thread's rows (one 32-bit word column: one fp32 column or two 16-bit
             // columns), then over the block's row groups
