@@ -11,6 +11,7 @@ model quality.  Prints one JSON line: ms per step and the losses for the int8 la
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import time
 
@@ -56,6 +57,10 @@ class GPT2(nn.Module):
 
 def run(int8: bool, args):
     dev = "cuda:0"
+    # start from an empty caching allocator: blocks kept from the other model's run do not fit this one's sizes, and
+    # the allocator then frees and re-allocates device memory inside the timed steps
+    gc.collect()
+    torch.cuda.empty_cache()
     torch.manual_seed(0)
     model = GPT2(args.layers, args.d_model, args.heads, args.vocab, args.ctx)
     for p in model.parameters():
