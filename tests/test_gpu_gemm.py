@@ -141,6 +141,26 @@ def test_gemm_fp16_out_and_bias_dtypes(ops):
             assert torch.equal(Cb, C + bias.to(DEV).to(torch.float16))
 
 
+@pytest.mark.parametrize("out", ["bf16", "f16"])
+@pytest.mark.parametrize("block", [64, 128])
+def test_bias_dtypes_on_the_persistent_kernel(ops, out, block):
+    """gemm_wide stages the bias of a tile's 256 columns in LDS as one dword per column, whatever its type; a workgroup
+    that walks on to a second tile fetches that tile's bias after a barrier.  Odd N: the last tile's bias ends mid-dword."""
+    from blockwise_int8_linear_amd import _lib
+    g = torch.Generator().manual_seed(7 + block)
+    M, N, K = 4400, 4501, 256
+    assert _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, 0).decode() == "gemm_wide"
+    A, W = _codes(g, M, K).to(DEV), _codes(g, N, K).to(DEV)
+    sa = (torch.rand(K // block, M, generator=g) + 0.1).to(DEV)
+    sw = (torch.rand(K // block, N, generator=g) * 0.05 + 1e-3).to(DEV)
+    with cfg_as(ops, block, DTYPES[out]):
+        C = ops.int8_matmul_block64_rowwise_dequantize(A, W.t(), sa, sw)
+        for bd in (torch.float32, torch.bfloat16, torch.float16):
+            bias = (torch.randn(N, generator=g) * 3).to(bd).to(DEV)
+            Cb = ops.int8_matmul_block64_rowwise_dequantize(A, W.t(), sa, sw, bias)
+            assert torch.equal(Cb, C + bias.to(DTYPES[out]))             # added after the cast, in the output dtype
+
+
 def test_operand_layouts(ops):
     """b given as a contiguous [K,N] tensor, operands that are column slices of wider buffers, misaligned views"""
     g = torch.Generator().manual_seed(2)
