@@ -243,9 +243,9 @@ def bench_extras(pkg, torch):
     out["quantize_dual_bf16_8192"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
                                       "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
 
-    # Context, not part of the path: what a plain device-to-device copy of the same 128 MiB (the dual quantizer's input;
-    # it writes as many bytes again) reaches on this chip, three buffer pairs in rotation.  A kernel that reads and
-    # writes equal amounts has this, not the 8 TB/s of the data sheet, as its practical ceiling.
+    # Context, not part of the path: what torch's device-to-device copy of the same 128 MiB (the dual quantizer's input;
+    # it writes as many bytes again) reaches on this chip, three buffer pairs in rotation.  For scale only: a hand-written
+    # copy kernel with non-temporal 16-byte accesses measured 6.2 TB/s, the row quantizer's rate.
     ds = [torch.empty_like(x) for x in xs]
 
     def cp():
