@@ -84,6 +84,8 @@ CASES = [
     (1, 384, 512, 128, "gemv_rows"),
     (2, 1000, 4096 + 384, 128, "gemv_rows"),        # more than four runs of 1 KiB per row, the last one partial
     (2, 700, 2048 + 128, 64, "gemv_rows"),
+    (1, 300, 8192 + 384, 128, "gemv_rows"),         # one row, K from 8192 on: six runs of every weight row in flight
+    (1, 200, 9216, 64, "gemv_rows"),
     (3, 384, 512, 128, "gemv_staged"),
     (16, 1000, 4096, 128, "gemv_staged"),           # eight stages per wave
     (7, 1000, 1152, 64, "gemv_staged"),
