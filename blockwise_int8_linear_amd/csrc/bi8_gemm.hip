@@ -148,12 +148,19 @@ struct GemmArgs {
     int64_t M, N, K, lda, ldw, ldc;
     int tiles_m, tiles_n;
     int bias_dtype;
-    // split of the contraction over gridDim.y workgroups per tile (0 or 1: none): split `y` handles `split_stages`
-    // 128-byte stages of K from y * split_stages on and writes fp32 partial sums to ws[y][M][N]
+    // split of the contraction over `splits` workgroups (<= 1: none), each of which writes fp32 partial sums (scaled,
+    // no bias) of `split_stages` 128-byte stages of K to slabs ws[...][BM][BN], in one of two forms:
+    //   split_per_tile > 0: that many workgroups per tile; workgroup w takes stages (w % split_per_tile) * split_stages
+    //     ... of tile w / split_per_tile of the XCD-aware order, slab t * split_per_tile + w % split_per_tile (t = the
+    //     tile's row-major index);
+    //   split_per_tile == 0: the (tile, stage) pairs, tiles in row-major order and a tile's stages ascending, are one
+    //     sequence, and workgroup w takes the run of split_stages pairs from w * split_stages on.  A run touches one
+    //     tile or the end of one and the start of the next; slab w + t for each.
     float *ws;
     int64_t ws_bytes;
     int splits, split_stages;
     uint32_t band_magic;            // gemm_wide: floor(2^32 / (kGroupM * tiles_n))
+    int split_per_tile;
 };
 
 __device__ __forceinline__ float load_bias(const GemmArgs &g, int64_t n) {
@@ -177,26 +184,10 @@ template <int BM, int BN, int BLK, int NBUF> struct TileLds {
 };
 
 // BM x BN output tile per workgroup, WM x WN waves (each TM x TN subtiles of 32x32), BLK = quantization block.
+// One tile (tile_m, tile_n) of the problem `g`, by one workgroup.
 template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
-__global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
+__device__ __forceinline__ void gemm_tile_body(const GemmArgs g, const int tile_m, const int tile_n) {
     using L = TileLds<BM, BN, BLK, NBUF>;
-    GemmArgs g = g_in;
-    if constexpr (!PARTIALS && CDT == BI8_F32) {
-        // One split of K is the same problem on shifted operands: codes from byte k0 of every row, scale rows from
-        // K-block k0 / BLK, fp32 output (scaled, no bias) into this split's slab of the workspace.
-        if (g.splits > 1) {
-            const int64_t k0 = (int64_t)blockIdx.y * g.split_stages * kStageK;
-            const int64_t left = g.K - k0, chunk = (int64_t)g.split_stages * kStageK;
-            g.A += k0;
-            g.W += k0;
-            g.sA += (k0 / BLK) * g.M;
-            g.sW += (k0 / BLK) * g.N;
-            g.K = left < chunk ? left : chunk;
-            g.C = g.ws + (int64_t)blockIdx.y * g.M * g.N;
-            g.ldc = g.N;
-            g.bias = nullptr;
-        }
-    }
     constexpr int kBufs = NBUF;
     constexpr int NW = WM * WN;
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
@@ -215,8 +206,6 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
     const int wm = wave / WN, wn = wave % WN;
     const int l32 = lane & 31, h = lane >> 5;
 
-    int tile_m, tile_n;
-    tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
     const int nstages = (int)(g.K / kStageK);
 
@@ -637,6 +626,65 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
                     if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[a][b][r] * div, has_bias, bias);
                 }
         }
+    }
+}
+
+// SPLIT: the kernel of a split contraction (GemmArgs::splits workgroups, fp32 slabs), a kernel of its own so that the
+// one-tile-per-workgroup form stays the code it is.
+template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS, bool SPLIT = false>
+__global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
+    if constexpr (SPLIT) {
+        static_assert(!PARTIALS && CDT == BI8_F32, "the slabs are fp32 sums");
+        // A piece of a tile's K is the same problem on shifted operands: codes from byte k0 of every row, scale rows from
+        // K-block k0 / BLK, and as output the slab, addressed so that element (m0 + i, n0 + j) is slab[i][j].
+        // (The divisions below run on the vector unit; their results are wave-uniform and go back to scalar registers,
+        // where buffer descriptors and LDS addresses have to be.)
+        const int nst = (int)(g_in.K / kStageK), per = g_in.split_per_tile, S = g_in.split_stages;
+        const bool runs = per == 0;
+        // runs: this workgroup's run of (tile, stage) pairs [u, u_end), piece by piece (at most two: a run is shorter than a
+        // tile's K); per-tile splits: one piece
+        const int total = g_in.tiles_m * g_in.tiles_n * nst;                 // below 2^30: the plan splits nothing larger
+        int u = runs ? (int)blockIdx.x * S : 0;
+        const int u_end = runs ? (u + S < total ? u + S : total) : 1;
+        while (u < u_end) {
+            int tile_m, tile_n, s_lo, s_hi, slab;
+            if (runs) {
+                const int tile = __builtin_amdgcn_readfirstlane(u / nst);
+                s_lo = u - tile * nst;
+                s_hi = u_end - u < nst - s_lo ? s_lo + (u_end - u) : nst;
+                tile_m = __builtin_amdgcn_readfirstlane(tile / g_in.tiles_n);
+                tile_n = tile - tile_m * g_in.tiles_n;
+                slab = (int)blockIdx.x + tile;
+                u += s_hi - s_lo;
+            } else {
+                const int tw = __builtin_amdgcn_readfirstlane((int)blockIdx.x / per), part = (int)blockIdx.x - tw * per;
+                tile_of_workgroup(tw, g_in.tiles_m, g_in.tiles_n, tile_m, tile_n);
+                tile_m = __builtin_amdgcn_readfirstlane(tile_m);
+                tile_n = __builtin_amdgcn_readfirstlane(tile_n);
+                s_lo = part * S;
+                s_hi = s_lo + S < nst ? s_lo + S : nst;
+                slab = (tile_m * g_in.tiles_n + tile_n) * per + part;
+                u = u_end;
+            }
+            GemmArgs g = g_in;
+            const int64_t k0 = (int64_t)s_lo * kStageK;
+            g.A += k0;
+            g.W += k0;
+            g.sA += (k0 / BLK) * g.M;
+            g.sW += (k0 / BLK) * g.N;
+            g.K = (int64_t)(s_hi - s_lo) * kStageK;
+            g.C = g.ws + (int64_t)slab * (BM * BN) - ((int64_t)tile_m * BM * BN + (int64_t)tile_n * BN);
+            g.ldc = BN;
+            g.bias = nullptr;
+            gemm_tile_body<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>(g, tile_m, tile_n);
+            __syncthreads();                       // the next piece's loads reuse the stage buffers
+        }
+    } else {
+        int tile_m, tile_n;
+        tile_of_workgroup(blockIdx.x, g_in.tiles_m, g_in.tiles_n, tile_m, tile_n);
+        // (the divisions of the tile order run on the vector unit; the tile's coordinates go back to scalar registers,
+        // where buffer descriptors have to be)
+        gemm_tile_body<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>(g_in, __builtin_amdgcn_readfirstlane(tile_m), __builtin_amdgcn_readfirstlane(tile_n));
     }
 }
 
@@ -1934,47 +1982,92 @@ __global__ __launch_bounds__(256) void gemm_generic(const GemmArgs g, int block)
     }
 }
 
-// Sum of the split-K slabs, in ascending split order (deterministic), then the cast and the bias of the one-pass
-// epilogue: one output element per thread.
-template <int CDT>
+// Sum of a tile's slabs in ascending workgroup order (deterministic), then the cast and the bias of the one-pass
+// epilogue.  One workgroup = 8 rows of one tile, a thread = four consecutive columns; a tile has at most kSplitMax slabs,
+// all loaded before the first addition.  With split_per_tile workgroups per tile, tile t's slabs are
+// t * split_per_tile ... ; with runs, the workgroups whose runs touch tile t are floor(t * nst / S) ...
+// floor(((t + 1) * nst - 1) / S), and workgroup w's slab for it is ws[w + t].
+constexpr int kSplitMax = 8;
+template <int CDT, int BM, int BN>
 __global__ __launch_bounds__(256) void splitk_reduce(const GemmArgs g) {
-    const int64_t mn = g.M * g.N;
-    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (e >= mn) return;
-    float v = g.ws[e];
-    for (int sp = 1; sp < g.splits; ++sp) v += g.ws[sp * mn + e];
-    const int64_t m = e / g.N, n = e % g.N;
+    static_assert(BN == 128 && BM % 8 == 0, "32 threads x 4 columns per row, 8 rows per workgroup");
+    const int t = blockIdx.x, tile_m = t / g.tiles_n, tile_n = t - tile_m * g.tiles_n;
+    const int nst = (int)(g.K / kStageK), S = g.split_stages;
+    int first, count;
+    if (g.split_per_tile > 0) {
+        first = t * g.split_per_tile;
+        count = (nst + S - 1) / S;
+    } else {
+        const int w0 = (t * nst) / S, w1 = ((t + 1) * nst - 1) / S;
+        first = w0 + t;
+        count = w1 - w0 + 1;
+    }
+    const int i = blockIdx.y * 8 + (threadIdx.x >> 5), j = (threadIdx.x & 31) * 4;
+    const int64_t m = (int64_t)tile_m * BM + i;
+    if (m >= g.M) return;
+    const float *src = g.ws + (int64_t)first * (BM * BN) + i * BN + j;
+    bi8_v4f x[kSplitMax];
+#pragma unroll
+    for (int q = 0; q < kSplitMax; ++q) x[q] = q < count ? *(const bi8_v4f *)(src + (int64_t)q * (BM * BN)) : bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    bi8_v4f v = x[0];
+#pragma unroll
+    for (int q = 1; q < kSplitMax; ++q)
+        if (q < count) v += x[q];
     const bool has_bias = g.bias != nullptr;
-    store_c<CDT>(g.C, m * g.ldc + n, v, has_bias, has_bias ? load_bias(g, n) : 0.0f);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int64_t n = (int64_t)tile_n * BN + j + q;
+        if (n < g.N) store_c<CDT>(g.C, m * g.ldc + n, v[q], has_bias, has_bias ? load_bias(g, n) : 0.0f);
+    }
 }
 
-// How many ways to split K for a problem that the tile kernels run on few workgroups, and with which tile
-// (kind 0: 64x128, 1: 128x128): as many splits as fill the 256 CUs once, at least kSplitMinStages stages
-// of K each, at most kSplitMax; 1 = no split.
-constexpr int kSplitMax = 8, kSplitMinStages = 8;   // measured: 4 x 8 stages beat 8 x 4 at K = 4096, 8 x 11 beat 4 x 22 at K = 11008
-static int split_ways(int64_t tiles, int64_t nstages) {
-    if (tiles <= 0 || tiles > 128) return 1;
-    int64_t sp = 256 / tiles;
-    if (sp > kSplitMax) sp = kSplitMax;
-    if (sp > nstages / kSplitMinStages) sp = nstages / kSplitMinStages;
-    return sp < 2 ? 1 : (int)sp;
+// How to split a problem that the tile kernels would run on fewer workgroups than the chip has CUs, and with which tile
+// (kind 0: 64x128, 1: 128x128).
+// Up to 128 tiles: the same number of workgroups per tile, as many as fill the 256 CUs once, at least kSplitMinStages
+// stages of K each, at most kSplitMax (measured: 4 x 8 stages beat 8 x 4 at K = 4096, 8 x 11 beat 4 x 22 at K = 11008).
+// 129 to 255 tiles: the (tile, stage) pairs are dealt to 256 workgroups in equal runs that need not end where tiles end
+// (144 tiles of 64 stages are 256 runs of 36), when that saves kRunMinSaved stages and a quarter of a tile's K: a
+// workgroup whose run crosses into a second tile fills its pipeline twice and writes two slabs, and all tiles go through
+// the second kernel (measured: 3072 x 768 x 8192 at block 64 62.1 -> 54.3 us, 1500 x 1500 x 16384 at block 128
+// 84.8 -> 70.6; runs in place of the equal split of few tiles cost 10-25 %).
+constexpr int64_t kCus = 256;                  // compute units the plan counts rounds of workgroups against (MI355X)
+constexpr int kSplitMinStages = 8, kRunMinSaved = 28;
+struct SplitGrid {
+    int groups, stages, per_tile;                  // workgroups, stages of K per workgroup, workgroups per tile (0: runs); groups <= 1: no split
+};
+static SplitGrid split_grid(int64_t tiles, int64_t nstages) {
+    const SplitGrid none{1, 0, 0};
+    if (tiles <= 0 || tiles >= kCus || tiles * nstages >= (1ll << 30)) return none;
+    if (tiles <= 128) {
+        int64_t sp = kCus / tiles;
+        if (sp > kSplitMax) sp = kSplitMax;
+        if (sp > nstages / kSplitMinStages) sp = nstages / kSplitMinStages;
+        if (sp < 2) return none;
+        const int64_t stages = (nstages + sp - 1) / sp;
+        const int64_t per = (nstages + stages - 1) / stages;               // every workgroup has work
+        return per < 2 ? none : SplitGrid{(int)(tiles * per), (int)stages, (int)per};
+    }
+    const int64_t run = (tiles * nstages + kCus - 1) / kCus;
+    if (nstages - run < kRunMinSaved || 4 * run > 3 * nstages) return none;
+    return SplitGrid{(int)((tiles * nstages + run - 1) / run), (int)run, 0};
 }
-static int plan_split(int64_t M, int64_t N, int64_t K, int &kind) {
+static SplitGrid plan_split(int64_t M, int64_t N, int64_t K, int &kind) {
     const int64_t nstages = K / kStageK;
     kind = M > 64 ? 1 : 0;
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128), t64 = ((M + 63) / 64) * ((N + 127) / 128);
     // (splitting the 256x128 tile where the 128x128 tiles are too many to split measured slower than not splitting)
-    const int sp = split_ways(kind ? t128 : t64, nstages);
+    const SplitGrid sg = split_grid(kind ? t128 : t64, nstages);
     // a short K caps the number of splits: when the 128x128 tiles then fill at most half of the CUs, the 64x128 tile
     // puts twice as many workgroups to work
-    if (kind == 1 && t128 * sp <= 128) {
-        const int sp64 = split_ways(t64, nstages);
-        if (sp64 > 1 && t64 * sp64 > t128 * sp) {
+    const int64_t wgs = sg.groups > 1 ? sg.groups : t128;
+    if (kind == 1 && wgs <= 128) {
+        const SplitGrid s64 = split_grid(t64, nstages);
+        if (s64.groups > 1 && s64.per_tile > 0 && s64.groups > wgs) {
             kind = 0;
-            return sp64;
+            return s64;
         }
     }
-    return sp;
+    return sg;
 }
 
 // A kernel that uses more than 64 KiB of dynamic LDS has to be allowed to, once per device: remembered here so that
@@ -2017,7 +2110,7 @@ static bool wide_addressable(int64_t M, int64_t N, int64_t K, int64_t lda, int64
     return (M - 1) * lda + K <= lim && (N - 1) * ldw + K <= lim && nblk * M * 4 <= lim && nblk * N * 4 <= lim && M + 256 <= lim && N + 256 <= lim;
 }
 
-template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
+template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS, bool SPLIT = false>
 int launch_tile(GemmArgs g, hipStream_t st) {
     constexpr int kLds = TileLds<BM, BN, BLK, NBUF>::kBytes;
     static_assert(TileLds<BM, BN, BLK, NBUF>::kFits, "tile does not fit the LDS");
@@ -2025,13 +2118,14 @@ int launch_tile(GemmArgs g, hipStream_t st) {
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     g.tiles_m = (int)tm;
     g.tiles_n = (int)tn;
-    auto kern = gemm_tile<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>;
+    auto kern = gemm_tile<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS, SPLIT>;
+    if (SPLIT != (g.splits > 1)) return BI8_ERR_UNSUPPORTED;         // (the plan pairs them)
     if (kLds > 64 * 1024) {
         static LdsOptIn opted;                     // one per kernel instantiation
         const int rc = opted.ensure((const void *)kern, kLds);
         if (rc != BI8_OK) return rc;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn), (unsigned)(g.splits > 1 ? g.splits : 1)), dim3(WM * WN * 64), kLds, st, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(SPLIT ? g.splits : tm * tn)), dim3(WM * WN * 64), kLds, st, g);
     return bi8_launch_rc();
 }
 
@@ -2087,19 +2181,20 @@ static const char *const kGemmKernelNames[] = {"gemm_generic", "gemv_staged", "g
                                                 "gemm_tile_64x128_splitk", "gemv_rows", "gemm_tile_128x192"};
 struct GemmPlan {
     int kernel;
-    int splits, split_stages;      // of the split kernels: workgroups per tile along K and 128-byte stages of K per split
+    int splits, split_stages;      // of the split kernels: workgroups of the split grid and 128-byte stages of K per workgroup,
+    int split_per_tile;            // ... workgroups per tile (0: runs across tiles)
+    int64_t ws_need;               // ... and the bytes of scratch memory for their slabs
 };
 // Up to 128 tiles of 256x256 the same problem is at most 256 tiles of 256x128: one round of workgroups on the 256 CUs,
 // where the smaller tile wins (1424 against 1072 TOP/s at 2048x4096x4096).  From 129 on the 256x128 grid needs a second,
 // mostly empty round and the 256x256 kernel wins (1284 against 978 TOP/s at 2304x4096x4096, 144 tiles).
 // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
 constexpr int64_t kWideMinTiles = 129;
-constexpr int64_t kCus = 256;                  // compute units the plan counts rounds of workgroups against (MI355X)
 // `aligned`: A and W 16-byte aligned, the scales 4-byte aligned (the partials entry point has no scales);
 // ws_bytes: scratch memory the split kernels may use (0: none).
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block, bool aligned, bool partials,
                           int64_t ws_bytes) {
-    GemmPlan p{kKGeneric, 1, 0};
+    GemmPlan p{kKGeneric, 1, 0, 0, 0};
     // the tiled kernels address a tile's operand rows and the scale rows with 32-bit byte offsets
     const int64_t max_ld = lda > ldw ? lda : ldw, max_mn = M > N ? M : N;
     const bool offsets_ok = max_ld < (1 << 22) && (block <= 0 || (K / block + 1) * max_mn * 4 < 0x7fffffffLL);
@@ -2145,15 +2240,17 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     if (!partials && ws_bytes > 0) {
         // few tiles and scratch memory: split K over several workgroups per tile, then sum the slabs
         int kind;
-        const int sp = plan_split(M, N, K, kind);
-        if (sp > 1) {
-            const int64_t nstages = K / kStageK;
-            const int stages = (int)((nstages + sp - 1) / sp);
-            const int splits = (int)((nstages + stages - 1) / stages);      // every split has work
-            if (splits > 1 && (int64_t)splits * M * N * 4 <= ws_bytes) {
+        const SplitGrid sg = plan_split(M, N, K, kind);
+        if (sg.groups > 1) {
+            // one slab of a tile's size per (workgroup, tile it touches); with runs the slab indices are workgroup + tile
+            const int64_t tiles = ((M + (kind ? 127 : 63)) / (kind ? 128 : 64)) * ((N + 127) / 128);
+            const int64_t need = (sg.per_tile > 0 ? sg.groups : sg.groups + tiles - 1) * (kind ? 128 : 64) * 128 * 4;
+            if (need <= ws_bytes) {
                 p.kernel = kind == 1 ? kKSplit128x128 : kKSplit64x128;
-                p.splits = splits;
-                p.split_stages = stages;
+                p.splits = sg.groups;
+                p.split_stages = sg.stages;
+                p.split_per_tile = sg.per_tile;
+                p.ws_need = need;
                 return p;
             }
         }
@@ -2231,12 +2328,16 @@ template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, co
             GemmArgs gs = g;
             gs.splits = p.splits;
             gs.split_stages = p.split_stages;
-            const int rc = p.kernel == kKSplit128x128 ? launch_tile<128, 128, 4, 2, kRing, BLK, BI8_F32, false>(gs, st)
-                                                      : launch_tile<64, 128, 2, 2, kRing, BLK, BI8_F32, false>(gs, st);
+            gs.split_per_tile = p.split_per_tile;
+            const bool big = p.kernel == kKSplit128x128;
+            const int rc = big ? launch_tile<128, 128, 4, 2, kRing, BLK, BI8_F32, false, true>(gs, st)
+                               : launch_tile<64, 128, 2, 2, kRing, BLK, BI8_F32, false, true>(gs, st);
             if (rc != BI8_OK) return rc;
-            const int64_t blocks = (g.M * g.N + 255) / 256;
-            if (blocks > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-            hipLaunchKernelGGL((splitk_reduce<CDT>), dim3((unsigned)blocks), dim3(256), 0, st, gs);
+            gs.tiles_m = (int)((g.M + (big ? 127 : 63)) / (big ? 128 : 64));
+            gs.tiles_n = (int)((g.N + 127) / 128);
+            const dim3 grid((unsigned)(gs.tiles_m * gs.tiles_n), big ? 16 : 8);     // fewer than 256 tiles, 8 rows each
+            if (big) hipLaunchKernelGGL((splitk_reduce<CDT, 128, 128>), grid, dim3(256), 0, st, gs);
+            else hipLaunchKernelGGL((splitk_reduce<CDT, 64, 128>), grid, dim3(256), 0, st, gs);
             return bi8_launch_rc();
         }
         default: break;
@@ -2287,8 +2388,8 @@ extern "C" int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float
 // The split of K needs scratch memory for its fp32 slabs.  bi8_gemm_nt_dequant_ws takes it from the caller;
 // bi8_gemm_nt_dequant_static takes it from this array, one copy per GPU that loads the library, for callers that cannot
 // allocate (HIP graph capture, serving loops, harnesses that forbid hipMalloc).  A split never wants more than
-// splits x tiles <= 256 tiles of 128 x 128 fp32 = 16 MiB (plan_split), which is the size of the array.
-constexpr int64_t kScratchBytes = 16ll << 20;
+// workgroups + tiles - 1 <= 256 + 254 slabs of 128 x 128 fp32 < 32 MiB (plan_split), which is the size of the array.
+constexpr int64_t kScratchBytes = 32ll << 20;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 // In host code `scratch` is only a handle for the runtime: the array's address on the current device comes from
@@ -2321,7 +2422,7 @@ extern "C" int bi8_gemm_nt_dequant_static(const int8_t *A, const int8_t *W, cons
     // what the split of this problem wants, were scratch memory unlimited; more than the array holds is refused
     // rather than run differently from bi8_gemm_nt_dequant_ws
     const GemmPlan p = plan_gemm(M, N, K, lda, ldw, block, true, false, INT64_MAX);
-    if (p.splits > 1 && (int64_t)p.splits * M * N * 4 > kScratchBytes) return BI8_ERR_SCRATCH_TOO_SMALL;
+    if (p.splits > 1 && p.ws_need > kScratchBytes) return BI8_ERR_SCRATCH_TOO_SMALL;
     void *ws = nullptr;
     if (p.splits > 1) {
         const int rc = scratch_of_current_device(&ws);
@@ -2334,7 +2435,7 @@ extern "C" int bi8_gemm_nt_dequant_static(const int8_t *A, const int8_t *W, cons
 extern "C" int64_t bi8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int block) {
     if (M <= 0 || N <= 0 || K <= 0 || block < 1) return 0;
     const GemmPlan p = plan_gemm(M, N, K, K, K, block, true, false, INT64_MAX);
-    return p.splits > 1 ? (int64_t)p.splits * M * N * 4 : 0;
+    return p.splits > 1 ? p.ws_need : 0;
 }
 
 extern "C" const char *bi8_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block,

@@ -125,10 +125,11 @@ int bi8_gemm_nt_dequant(const int8_t *A, const int8_t *W, const float *sA, const
                         int block, void *stream);
 
 /*
- * bi8_gemm_nt_dequant with a caller-provided scratch buffer.  On problems with few output tiles (a few hundred rows
- * of activations, or the grad-weight GEMM of a narrow layer) the contraction is split over several workgroups per
- * tile, which write fp32 partial sums to the workspace; a second kernel adds them in a fixed order, casts and adds
- * the bias.  (The reference's kernel has the same idea as SPLIT_K with atomic adds, triton_functions.py:121-139; its
+ * bi8_gemm_nt_dequant with a caller-provided scratch buffer.  On problems with fewer output tiles than the chip has
+ * compute units (a few hundred rows of activations, or the grad-weight GEMM of a narrow layer) the contraction is
+ * split: the (tile, 128-byte stage of K) pairs are dealt to the workgroups in equal runs, which need not end where a
+ * tile ends, each workgroup writes fp32 partial sums of the tiles it touches to the workspace, and a second kernel adds
+ * a tile's partial sums in a fixed order, casts and adds the bias.  (The reference's kernel has the same idea as SPLIT_K with atomic adds, triton_functions.py:121-139; its
  * launcher always passes SPLIT_K = 1.)  Results agree with bi8_gemm_nt_dequant to fp32 rounding of the sum over
  * K-blocks.  bi8_gemm_workspace_bytes tells how many bytes the split of a given problem wants (0: it would not
  * split); a NULL, misaligned (16 bytes) or smaller workspace makes the call identical to bi8_gemm_nt_dequant.
@@ -142,14 +143,14 @@ int bi8_gemm_nt_dequant_ws(const int8_t *A, const int8_t *W, const float *sA, co
 
 /*
  * bi8_gemm_nt_dequant_ws WITHOUT a workspace argument and without any allocation: the fp32 slabs of a split of K go
- * to a static array in device memory that belongs to the library (bi8_static_scratch_bytes() = 16 MiB on every GPU
+ * to a static array in device memory that belongs to the library (bi8_static_scratch_bytes() = 32 MiB on every GPU
  * the library runs on, held until the process ends).  No counterpart in the reference: it is for callers that
  * cannot allocate -- code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The call
  * makes no hipMalloc / hipFree and no allocating library call; the first call on a device looks up the array's
  * address there (hipGetSymbolAddress), so make one call on each device outside any capture.
  * Same kernels, same results (bit for bit) as bi8_gemm_nt_dequant_ws given bi8_gemm_workspace_bytes() of workspace.
  * A problem whose split wants more than the array holds returns BI8_ERR_SCRATCH_TOO_SMALL and launches nothing (with
- * the present split rule -- at most 256 slabs of 128 x 128 fp32 -- no problem does).
+ * the present split rule -- fewer than 512 slabs of 128 x 128 fp32 -- no problem does).
  * All calls on one GPU share the array, which keeps the last call's contents (every call overwrites what it reads,
  * nothing has to start at zero): calls that overlap on one GPU -- two streams, two host threads -- race on it.
  * Serialize them on one stream, or give the overlapping ones their own workspace through bi8_gemm_nt_dequant_ws.

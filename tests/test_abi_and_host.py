@@ -224,15 +224,18 @@ def test_kernel_choice_by_shape():
     assert name(1, 128, 128 * 1024, 128) == "gemv_staged"            # any K: the scales stream through LDS with the stages
     assert name(128, 4096, 4096, 128) == "gemm_tile_128x128"         # no scratch memory: one pass
     ws = lib.bi8_gemm_workspace_bytes(128, 4096, 4096, 128)
+    # 64 tiles of 64x128, four workgroups each: one fp32 slab of a tile per workgroup
     assert ws == 4 * 128 * 4096 * 4 and name(128, 4096, 4096, 128, ws) == "gemm_tile_64x128_splitk"
     assert name(128, 4096, 4096, 128, ws - 1) == "gemm_tile_128x128"     # too small a workspace is not used
     assert name(512, 4096, 4096, 128, 1 << 30) == "gemm_tile_128x128_splitk"
+    # 144 tiles of 128x128: runs that end inside tiles fill the chip when K is long enough to pay for the second kernel
+    assert name(3072, 768, 8192, 64, 1 << 30) == "gemm_tile_128x128_splitk" and name(3072, 768, 2048, 64, 1 << 30) == "gemm_tile_128x128"
     assert name(300, 500, 500, 128) == "gemm_generic" and name(300, 500, 512, 128, 0, 520) == "gemm_generic"
     assert name(300, 500, 512, 48) == "gemm_generic"
     assert name(0, 500, 512, 128) == "none"
-    # a split never wants more than 16 MiB: splits x tiles <= 256 tiles of 128 x 128 fp32
-    for M in (33, 64, 100, 128, 256, 512, 1000, 2048):
-        for N in (128, 768, 4096, 11008, 50257):
+    # a split never wants more than the static scratch array holds: workgroups + tiles - 1 < 512 slabs of 128 x 128 fp32
+    for M in (33, 64, 100, 128, 256, 512, 1000, 2048, 3072, 4000):
+        for N in (128, 768, 1024, 4096, 11008, 50257):
             for K in (1024, 4096, 11008 , 8192 * 4):
                 for block in (32, 64, 128):
-                    assert lib.bi8_gemm_workspace_bytes(M, N, K, block) <= 16 << 20, (M, N, K, block)
+                    assert lib.bi8_gemm_workspace_bytes(M, N, K, block) <= lib.bi8_static_scratch_bytes(), (M, N, K, block)

@@ -1,4 +1,5 @@
-"""bi8_gemm_nt_dequant_ws: the contraction split over several workgroups per tile through a caller-provided workspace.
+"""bi8_gemm_nt_dequant_ws: the contraction split over the workgroups in equal runs of (tile, stage of K) pairs, through
+a caller-provided workspace.
 Against the CPU checker to the GEMM tolerance, and against the one-pass entry point (same numbers up to the fp32
 rounding of a different summation order)."""
 import ctypes
@@ -47,11 +48,13 @@ def _run(lib, A, W, sa, sw, bias, block, out, ws_bytes):
 
 @pytest.mark.parametrize("out", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("M,N,K,block", [(128, 512, 2048, 128), (100, 300, 2048, 64), (48, 700, 2560, 128), (200, 130, 4096, 32),
-                                         (384, 256, 8192, 64), (128, 4096, 4096, 128), (33, 128, 2048, 128)])
+                                         (384, 256, 8192, 64), (128, 4096, 4096, 128), (33, 128, 2048, 128),
+                                         # 20 and 25 stages of K in pieces of 8, 8, 4 and 7, 7, 7, 4
+                                         (48, 700, 2560, 128), (60, 4400, 3200, 128), (200, 300, 3200, 64)])
 def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
     want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
-    assert want > 0 and want % (M * N * 4) == 0 and 2 <= want // (M * N * 4) <= 8
+    assert 0 < want <= lib.bi8_static_scratch_bytes() and want % (64 * 128 * 4) == 0     # fp32 slabs of one tile (64x128 or 128x128) each
     Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
     split = _run(lib, Ad, Wd, sad, swd, None, block, out, want)
     one = _run(lib, Ad, Wd, sad, swd, None, block, out, 0)
@@ -67,6 +70,33 @@ def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
     # the bias is added after the cast, in the output type (triton_functions.py:127-131): exactly this identity
     with_bias = _run(lib, Ad, Wd, sad, swd, bias, block, out, want)
     assert torch.equal(with_bias, split + bias.to(DEV).to(DTYPES[out]))
+
+
+@pytest.mark.parametrize("M,N,K,block", [(3072, 768, 8192, 64), (1700, 1300, 16384, 128), (3000, 700, 8192, 32)])
+def test_more_tiles_than_half_the_chip(lib, M, N, K, block):
+    """129 to 255 tiles of 128x128 and a long K: 256 workgroups, each a run of (tile, stage) pairs that ends inside a tile.
+    The checker on sampled rows (every row of tiles is hit), the one-pass kernel on everything."""
+    A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
+    want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
+    tiles = -(-M // 128) * -(-N // 128)
+    assert want % (128 * 128 * 4) == 0 and 240 + tiles <= want // (128 * 128 * 4) <= 256 + tiles - 1
+    Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
+    split = _run(lib, Ad, Wd, sad, swd, bias, block, "f32", want)
+    one = _run(lib, Ad, Wd, sad, swd, bias, block, "f32", 0)
+    rows = torch.unique(torch.cat([torch.arange(0, M, 61), torch.tensor([M - 1])]))
+    ref = oracle_torch.int8_matmul_block_dequantize(A[rows], W, sa[:, rows].contiguous(), sw, block, bias, torch.float32)
+    P = oracle_torch.gemm_nt_partials(A[rows], W, block)
+    mag = torch.zeros(len(rows), N, dtype=torch.float64)
+    for j in range(K // block):
+        mag += P[j].abs().double() * sa[j, rows].double()[:, None] * sw[j].double()[None, :]
+    mag /= 127.0 * 127.0
+    bound = 1e-3 * ref.double().abs() + 4e-6 * mag + 1e-30
+    assert ((split[rows.to(DEV)].cpu().double() - ref.double()).abs() <= bound).all()
+    # everything else against the one-pass result: both are sums of the same fp32 terms in different orders
+    scale = one.abs().max().item()
+    assert (split - one).abs().max().item() <= 2e-5 * scale
+    again = _run(lib, Ad, Wd, sad, swd, bias, block, "f32", want)
+    assert torch.equal(split, again)                                         # fixed order of the sum: deterministic
 
 
 def test_workspace_too_small_or_absent_is_the_one_pass_result(lib):

@@ -28,10 +28,10 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point():
     lib = _lib.load()
     torch.cuda.set_device(0)
     st = torch.cuda.current_stream().cuda_stream
-    assert lib.bi8_static_scratch_bytes() == 16 << 20
+    assert lib.bi8_static_scratch_bytes() == 32 << 20
     # (M, N, K, block, out dtype code, splits?)  larger problem first, then a smaller one, one without a split, the first again
-    cases = [(512, 4096, 4096, 64, 1, True), (128, 1024, 4096, 128, 0, True), (64, 256, 2048, 128, 1, True),
-             (300, 500, 512, 128, 0, False), (512, 4096, 4096, 64, 1, True)]
+    cases = [(3072, 768, 8192, 64, 1, True), (128, 1024, 4096, 128, 0, True), (64, 256, 2048, 128, 1, True),
+             (300, 500, 512, 128, 0, False), (3072, 768, 8192, 64, 1, True)]
     dts = {0: torch.float32, 1: torch.bfloat16}
     torch.cuda.synchronize()
     for i, (M, N, K, block, cdt, splits) in enumerate(cases):
@@ -51,12 +51,14 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point():
         torch.cuda.synchronize()
         assert torch.equal(c_st, c_ws), f"case {i}: static-scratch output differs from the workspace output"
         # and against the CPU checker; the bias is added to the rounded product in the output type, so the relative
-        # bound counts the magnitudes of both
+        # bound counts the magnitudes of both, and where the products differ the rounding of the sum can add one more
+        # unit in the last place of the output type
         ref, mag = gemm_reference(A, W, sa, sw, block, None, dts[cdt])
-        tol = 1e-3 if cdt == 0 else 1e-2
+        tol, ulp = (1e-3, 2.0 ** -23) if cdt == 0 else (1e-2, 2.0 ** -7)
         full = (ref + bias.to(dts[cdt])).double()
-        bound = tol * (ref.double().abs() + 2 * bias.double().abs()) + 4e-6 * mag
-        assert ((c_st.cpu().double() - full).abs() <= bound).all()
+        bound = tol * (ref.double().abs() + 2 * bias.double().abs()) + ulp * full.abs() + 4e-6 * mag
+        err = (c_st.cpu().double() - full).abs()
+        assert (err <= bound).all(), f"case {i}: {(err > bound).sum().item()} elements off, worst {(err - bound).max().item():.3e} over its bound"
     # bad arguments are refused before anything is looked up or launched
     assert lib.bi8_gemm_nt_dequant_static(None, None, None, None, None, 0, None, 0, 4, 4, 128, 64, 128, 4, 128, None) == 4
     assert b"scratch" in lib.bi8_strerror(7)
