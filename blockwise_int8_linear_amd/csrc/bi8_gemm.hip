@@ -2201,6 +2201,23 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     const bool tile_ok = K > 0 && K % kStageK == 0 && lda % 16 == 0 && ldw % 16 == 0 && aligned && offsets_ok &&
                          (block == 32 || block == 64 || block == 128);
     if (!tile_ok) return p;
+    // few tiles and scratch memory: split K over the workgroups, then sum the slabs
+    auto try_split = [&]() {
+        if (partials || ws_bytes <= 0) return false;
+        int kind;
+        const SplitGrid sg = plan_split(M, N, K, kind);
+        if (sg.groups <= 1) return false;
+        // one slab of a tile's size per (workgroup, tile it touches); with runs the slab indices are workgroup + tile
+        const int64_t tiles = ((M + (kind ? 127 : 63)) / (kind ? 128 : 64)) * ((N + 127) / 128);
+        const int64_t need = (sg.per_tile > 0 ? sg.groups : sg.groups + tiles - 1) * (kind ? 128 : 64) * 128 * 4;
+        if (need > ws_bytes) return false;
+        p.kernel = kind == 1 ? kKSplit128x128 : kKSplit64x128;
+        p.splits = sg.groups;
+        p.split_stages = sg.stages;
+        p.split_per_tile = sg.per_tile;
+        p.ws_need = need;
+        return true;
+    };
     if (!partials) {
         if (M <= kRowsMax && (block == 64 || block == 128) &&
             (block == 64 ? rows_lds_bytes<64>(M, K, 0) : rows_lds_bytes<128>(M, K, 0)) <= kRowsLdsMax && (K / block + 16) * N * 4 < 0x7fffffffLL) {
@@ -2213,7 +2230,9 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             return p;
         }
         if (M <= 32) {
-            p.kernel = kKSkinny;
+            // 17 to 32 rows (and block 32): with scratch memory the split 64x128 tiles are ahead of the kernel that gathers
+            // its operands (block 128, 4096 -> 11008: 30-34 us against 17)
+            if (!try_split()) p.kernel = kKSkinny;
             return p;
         }
         // 256x256 tiles when there is enough work to fill the 256 CUs with them
@@ -2237,24 +2256,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     }
     // small grids: one workgroup per CU at best, so the tile is spread over as many waves as its shape allows
     // (measured 25-37 % faster than 2x2 waves of 64x64 at M = 96 ... 1024)
-    if (!partials && ws_bytes > 0) {
-        // few tiles and scratch memory: split K over several workgroups per tile, then sum the slabs
-        int kind;
-        const SplitGrid sg = plan_split(M, N, K, kind);
-        if (sg.groups > 1) {
-            // one slab of a tile's size per (workgroup, tile it touches); with runs the slab indices are workgroup + tile
-            const int64_t tiles = ((M + (kind ? 127 : 63)) / (kind ? 128 : 64)) * ((N + 127) / 128);
-            const int64_t need = (sg.per_tile > 0 ? sg.groups : sg.groups + tiles - 1) * (kind ? 128 : 64) * 128 * 4;
-            if (need <= ws_bytes) {
-                p.kernel = kind == 1 ? kKSplit128x128 : kKSplit64x128;
-                p.splits = sg.groups;
-                p.split_stages = sg.stages;
-                p.split_per_tile = sg.per_tile;
-                p.ws_need = need;
-                return p;
-            }
-        }
-    }
+    if (try_split()) return p;
     // (64x128 tiles for problems of 129-255 tiles of 128x128 measured 5-10 % slower than the half-empty 128x128 grid)
     p.kernel = M > 64 ? kKTile128x128 : kKTile64x128;
     return p;

@@ -89,7 +89,8 @@ CASES = [
     (3, 384, 512, 128, "gemv_staged"),
     (16, 1000, 4096, 128, "gemv_staged"),           # eight stages per wave
     (7, 1000, 1152, 64, "gemv_staged"),
-    (24, 500, 2048, 128, "gemm_skinny"),
+    (24, 500, 640, 128, "gemm_skinny"),             # five stages of K: nothing to split
+    (24, 500, 2048, 128, "gemm_tile_64x128_splitk"),
     (16, 300, 1024, 32, "gemm_skinny"),
     (128, 1024, 4096, 128, "gemm_tile_64x128_splitk"),
     (512, 4096, 4096, 64, "gemm_tile_128x128_splitk"),
