@@ -161,6 +161,13 @@ struct GemmArgs {
     int splits, split_stages;
     uint32_t band_magic;            // gemm_wide: floor(2^32 / (kGroupM * tiles_n))
     int split_per_tile;
+    // a launch that computes part of the output only: tiles_m x tiles_n tiles from tile (tile_m0, tile_n0) on (M, N and
+    // the pointers stay those of the whole problem)
+    int tile_m0, tile_n0;
+};
+// The rectangle of the output that one launch computes (the whole of it unless the plan cuts the problem in two).
+struct Part {
+    int64_t row0, col0, rows, cols;
 };
 
 __device__ __forceinline__ float load_bias(const GemmArgs &g, int64_t n) {
@@ -666,6 +673,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
                 slab = (tile_m * g_in.tiles_n + tile_n) * per + part;
                 u = u_end;
             }
+            tile_m += g_in.tile_m0;                // from the launch's tiles to the problem's
+            tile_n += g_in.tile_n0;
             GemmArgs g = g_in;
             const int64_t k0 = (int64_t)s_lo * kStageK;
             g.A += k0;
@@ -684,7 +693,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
         tile_of_workgroup(blockIdx.x, g_in.tiles_m, g_in.tiles_n, tile_m, tile_n);
         // (the divisions of the tile order run on the vector unit; the tile's coordinates go back to scalar registers,
         // where buffer descriptors have to be)
-        gemm_tile_body<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>(g_in, __builtin_amdgcn_readfirstlane(tile_m), __builtin_amdgcn_readfirstlane(tile_n));
+        gemm_tile_body<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>(g_in, __builtin_amdgcn_readfirstlane(tile_m) + g_in.tile_m0,
+                                                                 __builtin_amdgcn_readfirstlane(tile_n) + g_in.tile_n0);
     }
 }
 
@@ -2003,7 +2013,7 @@ __global__ __launch_bounds__(256) void splitk_reduce(const GemmArgs g) {
         count = w1 - w0 + 1;
     }
     const int i = blockIdx.y * 8 + (threadIdx.x >> 5), j = (threadIdx.x & 31) * 4;
-    const int64_t m = (int64_t)tile_m * BM + i;
+    const int64_t m = (int64_t)(tile_m + g.tile_m0) * BM + i;
     if (m >= g.M) return;
     const float *src = g.ws + (int64_t)first * (BM * BN) + i * BN + j;
     bi8_v4f x[kSplitMax];
@@ -2016,7 +2026,7 @@ __global__ __launch_bounds__(256) void splitk_reduce(const GemmArgs g) {
     const bool has_bias = g.bias != nullptr;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        const int64_t n = (int64_t)tile_n * BN + j + q;
+        const int64_t n = (int64_t)(tile_n + g.tile_n0) * BN + j + q;
         if (n < g.N) store_c<CDT>(g.C, m * g.ldc + n, v[q], has_bias, has_bias ? load_bias(g, n) : 0.0f);
     }
 }
@@ -2111,13 +2121,16 @@ static bool wide_addressable(int64_t M, int64_t N, int64_t K, int64_t lda, int64
 }
 
 template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS, bool SPLIT = false>
-int launch_tile(GemmArgs g, hipStream_t st) {
+int launch_tile(GemmArgs g, const Part &part, hipStream_t st) {
     constexpr int kLds = TileLds<BM, BN, BLK, NBUF>::kBytes;
     static_assert(TileLds<BM, BN, BLK, NBUF>::kFits, "tile does not fit the LDS");
-    const int64_t tm = (g.M + BM - 1) / BM, tn = (g.N + BN - 1) / BN;
+    if (part.row0 % BM != 0 || part.col0 % BN != 0) return BI8_ERR_UNSUPPORTED;     // (the plan cuts at multiples of 256 only)
+    const int64_t tm = (part.rows + BM - 1) / BM, tn = (part.cols + BN - 1) / BN;
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     g.tiles_m = (int)tm;
     g.tiles_n = (int)tn;
+    g.tile_m0 = (int)(part.row0 / BM);
+    g.tile_n0 = (int)(part.col0 / BN);
     auto kern = gemm_tile<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS, SPLIT>;
     if (SPLIT != (g.splits > 1)) return BI8_ERR_UNSUPPORTED;         // (the plan pairs them)
     if (kLds > 64 * 1024) {
@@ -2129,9 +2142,10 @@ int launch_tile(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-template <int BLK, int CDT> int launch_wide(GemmArgs g, hipStream_t st) {
+template <int BLK, int CDT> int launch_wide(GemmArgs g, const Part &part, hipStream_t st) {
     using L = WideLds<kStageK / BLK>;
-    const int64_t tm = (g.M + 255) / 256, tn = (g.N + 255) / 256;
+    if (part.row0 != 0 || part.col0 != 0) return BI8_ERR_UNSUPPORTED;         // (the plan gives this kernel the leading part)
+    const int64_t tm = (part.rows + 255) / 256, tn = (part.cols + 255) / 256;
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     g.tiles_m = (int)tm;
     g.tiles_n = (int)tn;
@@ -2184,6 +2198,11 @@ struct GemmPlan {
     int splits, split_stages;      // of the split kernels: workgroups of the split grid and 128-byte stages of K per workgroup,
     int split_per_tile;            // ... workgroups per tile (0: runs across tiles)
     int64_t ws_need;               // ... and the bytes of scratch memory for their slabs
+    // a problem cut in two launches (cut_axis 0: one launch): `kernel` (the 256x256 kernel) on the leading `lead` rows
+    // (cut_axis 1) or columns (2) of the output, the rest_* kernel of the tile family on the others
+    int cut_axis;
+    int64_t lead;
+    int rest_kernel, rest_splits, rest_split_stages, rest_split_per_tile;
 };
 // Up to 128 tiles of 256x256 the same problem is at most 256 tiles of 256x128: one round of workgroups on the 256 CUs,
 // where the smaller tile wins (1424 against 1072 TOP/s at 2048x4096x4096).  From 129 on the 256x128 grid needs a second,
@@ -2192,9 +2211,16 @@ struct GemmPlan {
 constexpr int64_t kWideMinTiles = 129;
 // `aligned`: A and W 16-byte aligned, the scales 4-byte aligned (the partials entry point has no scales);
 // ws_bytes: scratch memory the split kernels may use (0: none).
+// A last round of 256x256 tiles that is mostly empty costs as much as a full one (1280 x 11008 x 4096: 215 tiles, 69 us;
+// 1536 x 11008 x 4096: 258 tiles, 125 us).  When whole rows or columns of tiles can be cut off so that the leading part
+// is full rounds and the rest at most kCutMaxRest tiles' worth, the rest runs as a second launch on the smaller tiles
+// that suit it (measured, both launches: 1536 x 11008 x 4096 123 -> 93 us, 2304 x 8192 x 8192 229 -> 170, 4352 x 4096 x
+// 4096 120 -> 91, 2048 x 11008 x 4096 123 -> 114, 8192 x 2304 x 768 at block 64 43 -> 37; a rest of 96 tiles, 8192 x
+// 11008 x 4096, 378 -> 383: not cut).
+constexpr int64_t kCutMaxRest = 90;
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block, bool aligned, bool partials,
-                          int64_t ws_bytes) {
-    GemmPlan p{kKGeneric, 1, 0, 0, 0};
+                          int64_t ws_bytes, bool may_cut = true) {
+    GemmPlan p{kKGeneric, 1, 0, 0, 0, 0, 0, kKGeneric, 1, 0, 0};
     // the tiled kernels address a tile's operand rows and the scale rows with 32-bit byte offsets
     const int64_t max_ld = lda > ldw ? lda : ldw, max_mn = M > N ? M : N;
     const bool offsets_ok = max_ld < (1 << 22) && (block <= 0 || (K / block + 1) * max_mn * 4 < 0x7fffffffLL);
@@ -2236,8 +2262,34 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             return p;
         }
         // 256x256 tiles when there is enough work to fill the 256 CUs with them
-        if (((M + 255) / 256) * ((N + 255) / 256) >= kWideMinTiles && (block == 32 || wide_addressable(M, N, K, lda, ldw, block))) {
+        const int64_t tm = (M + 255) / 256, tn = (N + 255) / 256;
+        if (tm * tn >= kWideMinTiles && (block == 32 || wide_addressable(M, N, K, lda, ldw, block))) {
             p.kernel = kKWide;
+            const int64_t full = (tm * tn / kCus) * kCus;             // tiles of the full rounds
+            if (may_cut && block != 32 && full > 0 && tm * tn > full) {
+                // the largest leading part of whole tile rows (columns) within the full rounds, and what the rest costs
+                int64_t best_rest = kCutMaxRest + 1;
+                for (int axis = 1; axis <= 2; ++axis) {
+                    const int64_t across = axis == 1 ? tn : tm, along = axis == 1 ? tm : tn;
+                    const int64_t lead = full / across;                // whole rows (columns) of tiles
+                    if (lead < 1 || lead >= along) continue;
+                    const int64_t rest_tiles = (along - lead) * across;
+                    if (rest_tiles >= best_rest) continue;
+                    const int64_t rm = axis == 1 ? M - lead * 256 : M, rn = axis == 1 ? N : N - lead * 256;
+                    const GemmPlan r = plan_gemm(rm, rn, K, lda, ldw, block, aligned, false, ws_bytes, false);
+                    const bool tile_family = r.kernel == kKTile256x128 || r.kernel == kKTile128x128 || r.kernel == kKTile64x128 ||
+                                             r.kernel == kKSplit128x128 || r.kernel == kKSplit64x128;
+                    if (!tile_family) continue;                        // (128x192 tiles do not start at multiples of 256)
+                    best_rest = rest_tiles;
+                    p.cut_axis = axis;
+                    p.lead = lead * 256;
+                    p.rest_kernel = r.kernel;
+                    p.rest_splits = r.splits;
+                    p.rest_split_stages = r.split_stages;
+                    p.rest_split_per_tile = r.split_per_tile;
+                    p.ws_need = r.ws_need;
+                }
+            }
             return p;
         }
     }
@@ -2298,22 +2350,26 @@ template <int BLK, int CDT> int launch_rows(const GemmArgs &g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, const GemmPlan &p, hipStream_t st) {
+// kernel `kernel` (with the split parameters, if it is one of the split kernels) on the rectangle `part` of the output
+template <int BLK, int CDT, bool PARTIALS>
+int launch_kernel(const GemmArgs &g, int kernel, int splits, int split_stages, int split_per_tile, const Part &part, hipStream_t st) {
     constexpr int kRing = 3;                       // stage buffers of the tile kernels that are not software-pipelined
-    switch (p.kernel) {
+    const bool whole = part.row0 == 0 && part.col0 == 0 && part.rows == g.M && part.cols == g.N;
+    switch (kernel) {
     case kKTile256x128:
         if constexpr (TileLds<256, 128, BLK, kRing>::kFits)
-            return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : kRing, BLK, CDT, PARTIALS>(g, st);
+            return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : kRing, BLK, CDT, PARTIALS>(g, part, st);
         break;
     case kKTile128x192:                            // 32x96 per wave
-        if constexpr (BLK == 64) return launch_tile<128, 192, 4, 2, kRing, BLK, CDT, PARTIALS>(g, st);
+        if constexpr (BLK == 64) return launch_tile<128, 192, 4, 2, kRing, BLK, CDT, PARTIALS>(g, part, st);
         break;
-    case kKTile128x128: return launch_tile<128, 128, 4, 2, kRing, BLK, CDT, PARTIALS>(g, st);
-    case kKTile64x128: return launch_tile<64, 128, 2, 2, kRing, BLK, CDT, PARTIALS>(g, st);
+    case kKTile128x128: return launch_tile<128, 128, 4, 2, kRing, BLK, CDT, PARTIALS>(g, part, st);
+    case kKTile64x128: return launch_tile<64, 128, 2, 2, kRing, BLK, CDT, PARTIALS>(g, part, st);
     default: break;
     }
     if constexpr (!PARTIALS) {
-        switch (p.kernel) {
+        if (!whole && kernel != kKWide && kernel != kKSplit128x128 && kernel != kKSplit64x128) return BI8_ERR_UNSUPPORTED;
+        switch (kernel) {
         case kKRows:
             if constexpr (BLK != 32) return launch_rows<BLK, CDT>(g, st);
             break;
@@ -2323,20 +2379,23 @@ template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, co
         case kKSkinny: return launch_skinny<BLK, CDT>(g, st);
         case kKWide:
             // blocks 128 and 64: 16x16x64 MFMAs, 64x128 per wave; block 32 (one MFMA per K-block): 32x32x32, 32x256 per wave
-            if constexpr (BLK == 32) return launch_wide32<BLK, CDT>(g, st);
-            else return launch_wide<BLK, CDT>(g, st);
+            if constexpr (BLK == 32) return whole ? launch_wide32<BLK, CDT>(g, st) : BI8_ERR_UNSUPPORTED;
+            else return launch_wide<BLK, CDT>(g, part, st);
         case kKSplit128x128:
         case kKSplit64x128: {
             GemmArgs gs = g;
-            gs.splits = p.splits;
-            gs.split_stages = p.split_stages;
-            gs.split_per_tile = p.split_per_tile;
-            const bool big = p.kernel == kKSplit128x128;
-            const int rc = big ? launch_tile<128, 128, 4, 2, kRing, BLK, BI8_F32, false, true>(gs, st)
-                               : launch_tile<64, 128, 2, 2, kRing, BLK, BI8_F32, false, true>(gs, st);
+            gs.splits = splits;
+            gs.split_stages = split_stages;
+            gs.split_per_tile = split_per_tile;
+            const bool big = kernel == kKSplit128x128;
+            const int rc = big ? launch_tile<128, 128, 4, 2, kRing, BLK, BI8_F32, false, true>(gs, part, st)
+                               : launch_tile<64, 128, 2, 2, kRing, BLK, BI8_F32, false, true>(gs, part, st);
             if (rc != BI8_OK) return rc;
-            gs.tiles_m = (int)((g.M + (big ? 127 : 63)) / (big ? 128 : 64));
-            gs.tiles_n = (int)((g.N + 127) / 128);
+            const int bm = big ? 128 : 64;
+            gs.tiles_m = (int)((part.rows + bm - 1) / bm);
+            gs.tiles_n = (int)((part.cols + 127) / 128);
+            gs.tile_m0 = (int)(part.row0 / bm);
+            gs.tile_n0 = (int)(part.col0 / 128);
             const dim3 grid((unsigned)(gs.tiles_m * gs.tiles_n), big ? 16 : 8);     // fewer than 256 tiles, 8 rows each
             if (big) hipLaunchKernelGGL((splitk_reduce<CDT, 128, 128>), grid, dim3(256), 0, st, gs);
             else hipLaunchKernelGGL((splitk_reduce<CDT, 64, 128>), grid, dim3(256), 0, st, gs);
@@ -2346,6 +2405,16 @@ template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, co
         }
     }
     return BI8_ERR_UNSUPPORTED;                    // plan_gemm never pairs these (kernel, block)
+}
+
+template <int BLK, int CDT, bool PARTIALS> int launch_plan(const GemmArgs &g, const GemmPlan &p, hipStream_t st) {
+    if (p.cut_axis == 0)
+        return launch_kernel<BLK, CDT, PARTIALS>(g, p.kernel, p.splits, p.split_stages, p.split_per_tile, Part{0, 0, g.M, g.N}, st);
+    const Part lead = p.cut_axis == 1 ? Part{0, 0, p.lead, g.N} : Part{0, 0, g.M, p.lead};
+    const Part rest = p.cut_axis == 1 ? Part{p.lead, 0, g.M - p.lead, g.N} : Part{0, p.lead, g.M, g.N - p.lead};
+    const int rc = launch_kernel<BLK, CDT, PARTIALS>(g, p.kernel, 1, 0, 0, lead, st);
+    if (rc != BI8_OK) return rc;
+    return launch_kernel<BLK, CDT, PARTIALS>(g, p.rest_kernel, p.rest_splits, p.rest_split_stages, p.rest_split_per_tile, rest, st);
 }
 
 template <int CDT, bool PARTIALS> int dispatch(const GemmArgs &g, int block, hipStream_t st) {
@@ -2424,9 +2493,9 @@ extern "C" int bi8_gemm_nt_dequant_static(const int8_t *A, const int8_t *W, cons
     // what the split of this problem wants, were scratch memory unlimited; more than the array holds is refused
     // rather than run differently from bi8_gemm_nt_dequant_ws
     const GemmPlan p = plan_gemm(M, N, K, lda, ldw, block, true, false, INT64_MAX);
-    if (p.splits > 1 && p.ws_need > kScratchBytes) return BI8_ERR_SCRATCH_TOO_SMALL;
+    if (p.ws_need > kScratchBytes) return BI8_ERR_SCRATCH_TOO_SMALL;
     void *ws = nullptr;
-    if (p.splits > 1) {
+    if (p.ws_need > 0) {
         const int rc = scratch_of_current_device(&ws);
         if (rc != BI8_OK) return rc;
     }
@@ -2437,13 +2506,23 @@ extern "C" int bi8_gemm_nt_dequant_static(const int8_t *A, const int8_t *W, cons
 extern "C" int64_t bi8_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int block) {
     if (M <= 0 || N <= 0 || K <= 0 || block < 1) return 0;
     const GemmPlan p = plan_gemm(M, N, K, K, K, block, true, false, INT64_MAX);
-    return p.splits > 1 ? p.ws_need : 0;
+    return p.ws_need;
 }
 
 extern "C" const char *bi8_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block,
                                             int64_t workspace_bytes) {
     if (M <= 0 || N <= 0 || K < 0 || block < 1) return "none";
-    return kGemmKernelNames[plan_gemm(M, N, K, lda, ldw, block, true, false, workspace_bytes).kernel];
+    const GemmPlan p = plan_gemm(M, N, K, lda, ldw, block, true, false, workspace_bytes);
+    if (p.cut_axis != 0) {                         // two launches: the 256x256 kernel, then the rest on smaller tiles
+        switch (p.rest_kernel) {
+        case kKTile256x128: return "gemm_wide+gemm_tile_256x128";
+        case kKTile128x128: return "gemm_wide+gemm_tile_128x128";
+        case kKTile64x128: return "gemm_wide+gemm_tile_64x128";
+        case kKSplit128x128: return "gemm_wide+gemm_tile_128x128_splitk";
+        default: return "gemm_wide+gemm_tile_64x128_splitk";
+        }
+    }
+    return kGemmKernelNames[p.kernel];
 }
 
 template <int DT> int launch_few_rows(const GemmArgs &g, const void *x, int64_t ldx, int block, size_t lds, hipStream_t st) {

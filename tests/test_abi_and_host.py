@@ -213,6 +213,10 @@ def test_kernel_choice_by_shape():
     assert name(8192, 8192, 8192, 32) == "gemm_wide"                 # (the 32x32x32-MFMA form of the 256x256 kernel)
     assert name(2048, 4096, 4096, 32) == "gemm_tile_128x128"         # block 32 has no 256x128 tile
     assert name(2944, 2944, 512, 128) == "gemm_wide"                 # 12 x 12 = 144 tiles of 256x256
+    # a last round of 256x256 tiles that is mostly empty: whole rows (columns) of tiles cut off for a second launch
+    assert name(1536, 11008, 4096, 128) == "gemm_wide+gemm_tile_128x128" and name(2048, 11008, 4096, 128) == "gemm_wide+gemm_tile_256x128"
+    assert name(1536, 11008, 4096, 128, 1 << 30) == "gemm_wide+gemm_tile_64x128_splitk"
+    assert name(2048, 12288, 4096, 128) == "gemm_wide" and name(1280, 11008, 4096, 128) == "gemm_wide"   # half a round left / one round
     assert name(8192, 768, 3072, 64) == "gemm_tile_128x192" and name(8192, 768, 3072, 128) == "gemm_tile_256x128"
     assert name(2048, 4096, 4096, 128) == "gemm_tile_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
     assert name(2048, 4096, 512, 64) == "gemm_tile_256x128" and name(2048, 2304, 512, 64) == "gemm_tile_128x192"

@@ -79,7 +79,8 @@ def test_gemm_golden(ops):
 SHAPES = [(253, 257, 234), (129, 266, 75), (389, 138, 45), (256, 512, 512), (1, 384, 256), (16, 1000, 1024),
           (64, 128, 128), (48, 700, 640), (100, 300, 384), (300, 500, 512), (1024, 512, 512), (3584, 3584, 256), (3500, 3700, 384),
           (2304, 4500, 1152), (2560, 4096, 128),
-          (4400, 4501, 384),       # 324 tiles of 256x256: more than one per workgroup of the persistent grid, ragged edges
+          (4400, 4501, 384),       # 324 tiles of 256x256, ragged edges: one round on the 256x256 kernel, the last four rows of tiles on 128x128 tiles
+          (5200, 5101, 384),       # 420 tiles: more than one per workgroup of the persistent grid
           (5, 130, 66048)]         # a long contraction for the few-row kernel: 516 stages
 
 
@@ -148,7 +149,7 @@ def test_bias_dtypes_on_the_persistent_kernel(ops, out, block):
     that walks on to a second tile fetches that tile's bias after a barrier.  Odd N: the last tile's bias ends mid-dword."""
     from blockwise_int8_linear_amd import _lib
     g = torch.Generator().manual_seed(7 + block)
-    M, N, K = 4400, 4501, 256
+    M, N, K = 5200, 5101, 256
     assert _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, 0).decode() == "gemm_wide"
     A, W = _codes(g, M, K).to(DEV), _codes(g, N, K).to(DEV)
     sa = (torch.rand(K // block, M, generator=g) + 0.1).to(DEV)
@@ -368,7 +369,8 @@ def _run_nonfinite_few_rows(ops, A, W, block, g):
 
 
 # (M, N, K, kernel family)
-NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (4400, 4500, 256, "gemm_wide"), (2048, 2304, 256, "gemm_tile_256x128"),
+NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (5200, 5100, 256, "gemm_wide"),
+                    (4400, 4500, 256, "gemm_wide+gemm_tile_128x128"), (2048, 2304, 256, "gemm_tile_256x128"),
                     (8, 256, 512, "gemv_staged"), (24, 256, 512, "gemm_skinny"), (70, 90, 200, "gemm_generic"), (8, 256, 2560, "gemv_staged_long"),
                     (2, 256, 1536, "gemv_rows")]
 

@@ -67,8 +67,15 @@ CASES = [
     (2944, 2900, 384, 128, "gemm_wide"),            # odd number of stages (the loop runs a padding stage), ragged N
     (2944, 2944, 512, 64, "gemm_wide"),             # two K-blocks per stage
     (2900, 2944, 384, 64, "gemm_wide"),
-    (4400, 4500, 384, 128, "gemm_wide"),            # 324 tiles: workgroups of the persistent grid walk on to a second tile
-    (4500, 4400, 256, 64, "gemm_wide"),
+    (5200, 5200, 384, 128, "gemm_wide"),            # 441 tiles: workgroups of the persistent grid walk on to a second tile
+    (5200, 5100, 256, 64, "gemm_wide"),
+    # 324 tiles = one full round and 68: the leading 14 rows of tiles on the 256x256 kernel, the other rows on 128x128 tiles
+    (4400, 4500, 384, 128, "gemm_wide+gemm_tile_128x128"),
+    (4500, 4400, 256, 64, "gemm_wide+gemm_tile_128x128"),
+    (2048, 8900, 256, 128, "gemm_wide+gemm_tile_128x128"),         # cut by columns: 8 x 35 tiles, the last 3 columns of tiles apart
+    (2000, 8900, 384, 64, "gemm_wide+gemm_tile_128x128"),
+    (4352, 4096, 2048, 128, "gemm_wide+gemm_tile_64x128_splitk"),  # the rest (one row of 16 tiles) splits K
+    (4300, 4096, 4096, 64, "gemm_wide+gemm_tile_128x128_splitk"),
     (2944, 2944, 256, 32, "gemm_wide"),             # block 32: the 32x32x32-MFMA form, four K-blocks per stage
     (2900, 2944, 384, 32, "gemm_wide"),
     (2048, 2304, 512, 128, "gemm_tile_256x128"),    # the software-pipelined block-128 instantiation
