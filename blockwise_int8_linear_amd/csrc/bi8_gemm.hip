@@ -4,16 +4,20 @@
 //
 //   C[m,n] = cast( (1/127^2) * sum_j sA[j,m] * sW[j,n] * P_j[m,n] ),   P_j = int32 dot over K-block j
 //
-// NT GEMM, both operands K-contiguous.  Four kernels, chosen by shape in dispatch():
-//   gemm_wide    blocks 128 / 64, problems of >= 129 tiles of 256x256: v_mfma_i32_16x16x64_i8, 64x128 per wave;
+// NT GEMM, both operands K-contiguous.  The kernels, chosen by shape in plan_gemm():
+//   gemm_wide    blocks 128 / 64, problems of >= 129 tiles of 256x256: v_mfma_i32_16x16x64_i8, 64x128 per wave, persistent
+//                grid; when its last round of tiles would be mostly empty it runs on the leading rows or columns only and
+//                a gemm_tile launch takes the rest;
 //   gemm_wide32  block 32, same problems and tile: v_mfma_i32_32x32x32_i8, 32x256 per wave;
-//   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x128 / 64x128 tiles, 64x64 per wave; also
-//                the int32 block partials;
+//   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x192 / 128x128 / 64x128 tiles; also the int32
+//                block partials, and (SPLIT) fp32 partial sums over part of K for problems of fewer tiles than CUs, which
+//                splitk_reduce adds up;
 //   gemv_rows    M <= 2, blocks 64/128 (single-token decode; also bi8_linear_few_rows, which quantizes the activations in
 //                the same launch): one pass over W in 1 KiB runs of whole rows, v_dot4_i32_i8 on the vector unit;
 //   gemv_staged  M <= 16, blocks 64/128 (small decode batches): one pass over W, 16 columns per workgroup, K split over
 //                4 or 8 waves that each stream whole cache lines of W through a private LDS ring into 16x16x64 MFMAs;
-//   gemm_skinny  M <= 32 otherwise: the same idea with 32x32x32 MFMAs and one stage of lookahead;
+//   gemm_skinny  M <= 32 where neither of these nor the split applies: operands gathered in operand layout, 32x32x32 MFMAs,
+//                one stage of lookahead;
 //   gemm_generic anything else (K not a multiple of 128, rows not 16-byte aligned, other block sizes): same
 //                MFMA, operands gathered straight from global memory with byte loads.
 // Common to the tiled kernels:
