@@ -1644,6 +1644,12 @@ __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
     issue_w(NSW - 2, NSW - 2);
     auto stage = [&](int s, auto slot_c) {
         constexpr int SW = decltype(slot_c)::value, SA = SW & 1;
+        // The loads below overwrite the slots that the stage before has read.  Its ds_reads may still be in flight (the
+        // compiler waits for them where their results are first used, which it places after these loads), and a load of A,
+        // which every workgroup reads and the CU's L1 therefore often holds, can land within their latency: the reads
+        // have to be complete first.  (Without this wait, a workgroup that shares its CU with an older one now and then
+        // multiplied a stage's W by the A of two stages on.)
+        __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0)
         issue_a(s + 1, SA ^ 1);
         issue_w(s + NSW - 1, (SW + NSW - 1) % NSW);
         __builtin_amdgcn_s_waitcnt(0x0F70 | 10);   // vmcnt(10): everything up to A(s) has landed
@@ -2223,7 +2229,7 @@ constexpr int64_t kWideMinTiles = 129;
 // 11008 x 4096, 378 -> 383: not cut).
 constexpr int64_t kCutMaxRest = 90;
 static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldw, int block, bool aligned, bool partials,
-                          int64_t ws_bytes, bool may_cut = true) {
+                          int64_t ws_bytes, bool rest_of_cut = false) {
     GemmPlan p{kKGeneric, 1, 0, 0, 0, 0, 0, kKGeneric, 1, 0, 0};
     // the tiled kernels address a tile's operand rows and the scale rows with 32-bit byte offsets
     const int64_t max_ld = lda > ldw ? lda : ldw, max_mn = M > N ? M : N;
@@ -2248,7 +2254,8 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
         p.ws_need = need;
         return true;
     };
-    if (!partials) {
+    // (the rest of a cut problem shares the whole problem's pointers and strides, which only the tile kernels take)
+    if (!partials && !rest_of_cut) {
         if (M <= kRowsMax && (block == 64 || block == 128) &&
             (block == 64 ? rows_lds_bytes<64>(M, K, 0) : rows_lds_bytes<128>(M, K, 0)) <= kRowsLdsMax && (K / block + 16) * N * 4 < 0x7fffffffLL) {
             p.kernel = kKRows;
@@ -2270,7 +2277,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
         if (tm * tn >= kWideMinTiles && (block == 32 || wide_addressable(M, N, K, lda, ldw, block))) {
             p.kernel = kKWide;
             const int64_t full = (tm * tn / kCus) * kCus;             // tiles of the full rounds
-            if (may_cut && block != 32 && full > 0 && tm * tn > full) {
+            if (block != 32 && full > 0 && tm * tn > full) {
                 // the largest leading part of whole tile rows (columns) within the full rounds, and what the rest costs
                 int64_t best_rest = kCutMaxRest + 1;
                 for (int axis = 1; axis <= 2; ++axis) {
@@ -2280,7 +2287,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                     const int64_t rest_tiles = (along - lead) * across;
                     if (rest_tiles >= best_rest) continue;
                     const int64_t rm = axis == 1 ? M - lead * 256 : M, rn = axis == 1 ? N : N - lead * 256;
-                    const GemmPlan r = plan_gemm(rm, rn, K, lda, ldw, block, aligned, false, ws_bytes, false);
+                    const GemmPlan r = plan_gemm(rm, rn, K, lda, ldw, block, aligned, false, ws_bytes, true);
                     const bool tile_family = r.kernel == kKTile256x128 || r.kernel == kKTile128x128 || r.kernel == kKTile64x128 ||
                                              r.kernel == kKSplit128x128 || r.kernel == kKSplit64x128;
                     if (!tile_family) continue;                        // (128x192 tiles do not start at multiples of 256)
@@ -2307,7 +2314,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
         // kernel, against which the 128x192 tile measured 18 % slower)
         const int64_t t256 = ((M + 255) / 256) * ((N + 127) / 128), t192 = ((M + 127) / 128) * ((N + 191) / 192);
         const int64_t cost256 = ((t256 + kCus - 1) / kCus) * 256 * 128, cost192 = ((t192 + kCus - 1) / kCus) * 128 * 192;
-        p.kernel = (block == 64 && cost192 < cost256) ? kKTile128x192 : kKTile256x128;
+        p.kernel = (block == 64 && cost192 < cost256 && !rest_of_cut) ? kKTile128x192 : kKTile256x128;     // (192 does not divide the cut's 256)
         return p;
     }
     // small grids: one workgroup per CU at best, so the tile is spread over as many waves as its shape allows

@@ -162,6 +162,36 @@ def test_bias_dtypes_on_the_persistent_kernel(ops, out, block):
             assert torch.equal(Cb, C + bias.to(DTYPES[out]))             # added after the cast, in the output dtype
 
 
+@pytest.mark.parametrize("M,N,K", [(7, 11008, 2048), (16, 11008, 4096), (3, 8192, 2048)])
+def test_small_batches_against_many_columns_call_after_call(ops, M, N, K):
+    """3 to 16 rows against more than 6144 columns run gemv_staged with four waves per workgroup, two or three workgroups
+    per CU.  Every wave streams W and A through a private LDS ring with direct-to-LDS loads; a load that overwrites a slot
+    must not be issued while the stage before is still reading it (a load of A, which the CU's L1 holds for the younger
+    workgroups, can land within an LDS read's latency: such workgroups used to return wrong sums now and then).  Ten calls
+    on fresh weights, each compared with the same rows run through the tile kernels inside a 33-row problem."""
+    from blockwise_int8_linear_amd import _lib
+    block = 128
+    assert _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, 0).decode() == "gemv_staged"
+    with cfg_as(ops, block, torch.float32):
+        for it in range(10):
+            g = torch.Generator().manual_seed(1000 * M + it)
+            W, A = _codes(g, N, K).to(DEV), _codes(g, M, K).to(DEV)
+            sa = (torch.rand(K // block, M, generator=g) + 0.5).to(DEV)
+            sw = (torch.rand(K // block, N, generator=g) * 0.02 + 1e-3).to(DEV)
+            Ap = torch.zeros(33, K, device=DEV, dtype=torch.int8)
+            Ap[:M] = A
+            sap = torch.zeros(K // block, 33, device=DEV)
+            sap[:, :M] = sa
+            want = ops.int8_matmul_block64_rowwise_dequantize(Ap, W.t(), sap, sw)[:M]
+            for _ in range(3):
+                got = ops.int8_matmul_block64_rowwise_dequantize(A, W.t(), sa, sw)
+                bad = (got - want).abs() > 1e-4 * want.abs() + 1e-5
+                assert not bad.any(), f"round {it}: {int(bad.sum())} elements off in workgroups {sorted(set((bad.nonzero()[:, 1] // 16).tolist()))[:8]}"
+        # and one of them against the CPU checker
+        ref = oracle_torch.int8_matmul_block_dequantize(A.cpu(), W.cpu(), sa.cpu(), sw.cpu(), block, None, torch.float32)
+        assert ((got.cpu() - ref).abs() <= 1e-3 * ref.abs() + 1e-6).all()
+
+
 def test_operand_layouts(ops):
     """b given as a contiguous [K,N] tensor, operands that are column slices of wider buffers, misaligned views"""
     g = torch.Generator().manual_seed(2)

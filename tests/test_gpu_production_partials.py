@@ -71,10 +71,14 @@ CASES = [
     (5200, 5100, 256, 64, "gemm_wide"),
     # 324 tiles = one full round and 68: the leading 14 rows of tiles on the 256x256 kernel, the other rows on 128x128 tiles
     (4400, 4500, 384, 128, "gemm_wide+gemm_tile_128x128"),
-    (4500, 4400, 256, 64, "gemm_wide+gemm_tile_128x128"),
+    (4500, 4400, 256, 64, "gemm_wide+gemm_tile_256x128"),
     (2048, 8900, 256, 128, "gemm_wide+gemm_tile_128x128"),         # cut by columns: 8 x 35 tiles, the last 3 columns of tiles apart
     (2000, 8900, 384, 64, "gemm_wide+gemm_tile_128x128"),
     (4352, 4096, 2048, 128, "gemm_wide+gemm_tile_64x128_splitk"),  # the rest (one row of 16 tiles) splits K
+    (4353, 4096, 256, 128, "gemm_wide+gemm_tile_128x128"),         # the rest is 257 rows: its last tiles hold one row
+    (4400, 4097, 384, 128, "gemm_wide+gemm_tile_128x128"),         # ... one column
+    (4097, 4096, 256, 128, "gemm_wide+gemm_tile_64x128"),          # a rest of a single row still runs on tiles
+    (4097, 4096, 2048, 64, "gemm_wide+gemm_tile_64x128_splitk"),
     (4300, 4096, 4096, 64, "gemm_wide+gemm_tile_128x128_splitk"),
     (2944, 2944, 256, 32, "gemm_wide"),             # block 32: the 32x32x32-MFMA form, four K-blocks per stage
     (2900, 2944, 384, 32, "gemm_wide"),
@@ -96,6 +100,8 @@ CASES = [
     (3, 384, 512, 128, "gemv_staged"),
     (16, 1000, 4096, 128, "gemv_staged"),           # eight stages per wave
     (7, 1000, 1152, 64, "gemv_staged"),
+    (7, 8192, 2048, 128, "gemv_staged"),            # more than 6144 columns: four waves per workgroup, several workgroups per CU
+    (12, 11008, 2048, 64, "gemv_staged"),
     (24, 500, 640, 128, "gemm_skinny"),             # five stages of K: nothing to split
     (24, 500, 2048, 128, "gemm_tile_64x128_splitk"),
     (16, 300, 1024, 32, "gemm_skinny"),
