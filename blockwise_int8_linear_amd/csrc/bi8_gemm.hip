@@ -14,10 +14,10 @@
 //                splitk_reduce adds up;
 //   gemv_rows    M <= 2, blocks 64/128 (single-token decode; also bi8_linear_few_rows, which quantizes the activations in
 //                the same launch): one pass over W in 1 KiB runs of whole rows, v_dot4_i32_i8 on the vector unit;
-//   gemv_staged  M <= 16, blocks 64/128 (small decode batches): one pass over W, 16 columns per workgroup, K split over
+//   gemv_staged  M <= 32, blocks 64/128 (small decode batches): one pass over W, 16 columns per workgroup, K split over
 //                4 or 8 waves that each stream whole cache lines of W through a private LDS ring into 16x16x64 MFMAs;
-//   gemm_skinny  M <= 32 where neither of these nor the split applies: operands gathered in operand layout, 32x32x32 MFMAs,
-//                one stage of lookahead;
+//   gemm_skinny  M <= 32 at block 32 (when nothing splits): operands gathered in operand layout, 32x32x32 MFMAs, one stage
+//                of lookahead;
 //   gemm_generic anything else (K not a multiple of 128, rows not 16-byte aligned, other block sizes): same
 //                MFMA, operands gathered straight from global memory with byte loads.
 // Common to the tiled kernels:
@@ -1560,8 +1560,8 @@ __global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
     }
 }
 
-// ---- up to 16 rows, weight rows read as whole cache lines through LDS ----------------------------------------------------
-// Few-row GEMM (M <= 16, blocks 64 and 128): decode.  HBM-bound on W: one pass over the weight codes.  A load in MFMA
+// ---- up to 32 rows, weight rows read as whole cache lines through LDS ----------------------------------------------------
+// Few-row GEMM (M <= 32 as one or two groups of 16 rows, blocks 64 and 128): decode.  HBM-bound on W: one pass over the weight codes.  A load in MFMA
 // operand layout would fetch 64 bytes of 16 rows (half a cache line per row and instruction); here a wave's load
 // instruction fetches whole 128-byte lines (8 rows x 128 bytes, straight into LDS), and the operands are read back from
 // LDS in operand layout.  One workgroup = 16 output columns; its NW waves split K in interleaved 128-byte chunks and
@@ -1571,17 +1571,26 @@ __global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
 // scales).  Measured at M = 16, block 128, against the same kernel with operands gathered from global memory in operand
 // layout through an 8-stage register ring: 4096 -> 11008 16.0 -> 12.8 us, 11008 -> 4096 17.1 -> 14.4 us.
 constexpr int kLdsGemvSlotsW = 4, kLdsGemvSlotsA = 2;
-constexpr int kLdsGemvSlot = 16 * 128;             // bytes of one stage of one operand
-constexpr int kLdsGemvScales = 256;                // bytes of one stage's scales: [K-block][16] column scales, then row scales
-constexpr size_t kLdsGemvWaveBytes = (size_t)(kLdsGemvSlotsW + kLdsGemvSlotsA) * kLdsGemvSlot + kLdsGemvSlotsW * kLdsGemvScales;
-template <int BLK, int CDT, int NW>
+constexpr int kLdsGemvSlot = 16 * 128;             // bytes of one stage of W, or of 16 rows of A
+// MT = groups of 16 rows of A (1: M <= 16, 2: M <= 32).  One stage's scales: [K-block][16] column scales (128 bytes), then
+// [K-block][16 * MT] row scales.
+template <int MT> struct GemvLds {
+    static constexpr int kAStage = MT * kLdsGemvSlot;
+    static constexpr int kScales = 128 + 128 * MT;
+    static constexpr int kAReg = kLdsGemvSlotsW * kLdsGemvSlot;
+    static constexpr int kScReg = kAReg + kLdsGemvSlotsA * kAStage;
+    static constexpr int kWaveBytes = kScReg + kLdsGemvSlotsW * kScales;
+};
+template <int BLK, int CDT, int NW, int MT>
 __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
+    using L = GemvLds<MT>;
     constexpr int KW = 128;                        // bytes of K per wave and stage
     constexpr int NSW = kLdsGemvSlotsW, NSA = kLdsGemvSlotsA;
     constexpr int BPS = KW / BLK;                  // K-blocks per stage of a wave
     constexpr int kSlot = kLdsGemvSlot;
     static_assert(BLK == 64 || BLK == 128, "one or two 64-byte MFMAs per K-block");
     static_assert(NSW == 4 && NSA == 2, "the K loop is unrolled over the period of both rings");
+    static_assert(MT == 1 || MT == 2, "16 or 32 rows of A");
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -1592,51 +1601,57 @@ __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
     const int nchunks = (int)(g.K / KW);
     const int nst = (((nchunks + NW - 1) / NW) + 3) & ~3;           // stages of every wave; those past the end of K load zeros
     const int nblk = (int)(g.K / BLK);
-    constexpr int wave_bytes = (int)kLdsGemvWaveBytes;
+    constexpr int wave_bytes = L::kWaveBytes;
     uint8_t *mine = lds + wave * wave_bytes;
     const uint32_t mine_addr = bi8_lds_address(lds) + (uint32_t)(wave * wave_bytes);
-    constexpr int kAReg = NSW * kSlot, kScReg = (NSW + NSA) * kSlot;
+    constexpr int kAReg = L::kAReg, kScReg = L::kScReg;
 
     const int64_t wrows = g.N - n0 < 16 ? g.N - n0 : 16;
     const bi8_rsrc rw = bi8_make_rsrc(g.W + n0 * g.ldw, (wrows - 1) * g.ldw + g.K);
     const bi8_rsrc ra = bi8_make_rsrc(g.A, (g.M - 1) * g.lda + g.K);
     const bi8_rsrc rsw = bi8_make_rsrc(g.sW, (int64_t)nblk * g.N * 4);
     const bi8_rsrc rsa = bi8_make_rsrc(g.sA, (int64_t)nblk * g.M * 4);
-    // scales of a stage: lane -> K-block lane/16 of the stage's BPS, column (or row) lane%16; rows past M read as zeros
+    // scales of a stage: column scales lane -> K-block lane / 16 of the stage's BPS, column lane % 16; row scales lane ->
+    // K-block lane / (16 MT), row lane % (16 MT); rows past M read as zeros
+    constexpr int kRowsA = 16 * MT;
     const uint32_t vsw = (uint32_t)((q * (int)g.N + (int)(n < g.N ? n : g.N - 1)) * 4);
-    const uint32_t vsa = r16 < g.M ? (uint32_t)((q * (int)g.M + r16) * 4) : (uint32_t)kBufOut;
+    const uint32_t vsa = lane % kRowsA < g.M ? (uint32_t)(((lane / kRowsA) * (int)g.M + lane % kRowsA) * 4) : (uint32_t)kBufOut;
 
     // ---- loader: instruction i of a stage covers rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which
-    // holds source chunk (lane%8) ^ ((row >> 1) & 7) = (lane%8) ^ (lane/16) ^ 4i
+    // holds source chunk (lane%8) ^ ((row >> 1) & 7) = (lane%8) ^ (lane/16) ^ 4(i & 1)
     const int ld_row = lane >> 3;
     const int ld_chunk = (lane & 7) ^ ((lane >> 4) & 3);
-    uint32_t vw[2], va[2];
+    uint32_t vw[2], va[2 * MT];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        vw[i] = (uint32_t)((8 * i + ld_row) * (int)g.ldw + 16 * (ld_chunk ^ (4 * i)));
-        va[i] = (uint32_t)((8 * i + ld_row) * (int)g.lda + 16 * (ld_chunk ^ (4 * i)));
-    }
+    for (int i = 0; i < 2; ++i) vw[i] = (uint32_t)((8 * i + ld_row) * (int)g.ldw + 16 * (ld_chunk ^ (4 * i)));
+#pragma unroll
+    for (int i = 0; i < 2 * MT; ++i) va[i] = (uint32_t)((8 * i + ld_row) * (int)g.lda + 16 * (ld_chunk ^ (4 * (i & 1))));
     auto issue_w = [&](int s, int slot) {          // s, slot: wave-uniform; four load instructions
         const int c = s * NW + wave;
         const bool live = c < nchunks;
         const uint32_t k0 = live ? (uint32_t)(c * KW) : (uint32_t)kBufOut;
 #pragma unroll
         for (int i = 0; i < 2; ++i) bi8_buffer_to_lds16(rw, mine_addr + slot * kSlot + i * 1024, vw[i], k0);
-        if (lane < 16 * BPS) {                     // (the loads write LDS for the active lanes only)
-            bi8_buffer_to_lds4(rsw, mine_addr + kScReg + slot * kLdsGemvScales, vsw, live ? (uint32_t)(c * BPS * (int)g.N * 4) : (uint32_t)kBufOut);
-            bi8_buffer_to_lds4(rsa, mine_addr + kScReg + slot * kLdsGemvScales + 128, vsa, live ? (uint32_t)(c * BPS * (int)g.M * 4) : (uint32_t)kBufOut);
-        }
+        if (lane < 16 * BPS)                       // (the loads write LDS for the active lanes only)
+            bi8_buffer_to_lds4(rsw, mine_addr + kScReg + slot * L::kScales, vsw, live ? (uint32_t)(c * BPS * (int)g.N * 4) : (uint32_t)kBufOut);
+        if (lane < kRowsA * BPS)
+            bi8_buffer_to_lds4(rsa, mine_addr + kScReg + slot * L::kScales + 128, vsa, live ? (uint32_t)(c * BPS * (int)g.M * 4) : (uint32_t)kBufOut);
     };
-    auto issue_a = [&](int s, int slot) {
+    auto issue_a = [&](int s, int slot) {          // 2 MT load instructions
         const int c = s * NW + wave;
         const uint32_t k0 = c < nchunks ? (uint32_t)(c * KW) : (uint32_t)kBufOut;
 #pragma unroll
-        for (int i = 0; i < 2; ++i) bi8_buffer_to_lds16(ra, mine_addr + kAReg + slot * kSlot + i * 1024, va[i], k0);
+        for (int i = 0; i < 2 * MT; ++i) bi8_buffer_to_lds16(ra, mine_addr + kAReg + slot * L::kAStage + i * 1024, va[i], k0);
     };
-    // operand fragments: lane -> row r16, chunk 4j + q of the stage's eight, stored at (4j + q) ^ ((r16 >> 1) & 7)
+    // operand fragments: lane -> row r16 (of W, or of a group of 16 rows of A), chunk 4j + q of the stage's eight, stored
+    // at (4j + q) ^ ((r16 >> 1) & 7)
     const int frag = r16 * KW + ((q ^ ((r16 >> 1) & 7)) << 4);
 
-    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    float acc[MT][4];
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[t][r] = 0.0f;
     // in flight at the top of stage s, oldest first: ..., A(s), W(s + NSW - 2)
 #pragma unroll
     for (int d = 0; d < NSW - 2; ++d) issue_w(d, d);
@@ -1652,28 +1667,34 @@ __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
         __builtin_amdgcn_s_waitcnt(0xC07F);        // lgkmcnt(0)
         issue_a(s + 1, SA ^ 1);
         issue_w(s + NSW - 1, (SW + NSW - 1) % NSW);
-        __builtin_amdgcn_s_waitcnt(0x0F70 | 10);   // vmcnt(10): everything up to A(s) has landed
+        // everything up to A(s) has landed when only W(s + 3), A(s + 1) and W(s + 2) are outstanding
+        constexpr int kPending = 8 + 2 * MT;
+        __builtin_amdgcn_s_waitcnt(0x0F70 | kPending);
         const bi8_v4i zero = {0, 0, 0, 0};
-        bi8_v4i wf[2], af[2];
+        bi8_v4i wf[2], af[MT][2];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             wf[j] = *(const bi8_v4i *)(mine + SW * kSlot + (frag ^ (j << 6)));
-            af[j] = *(const bi8_v4i *)(mine + kAReg + SA * kSlot + (frag ^ (j << 6)));
-        }
-        bi8_v4i p[BPS];
-        if constexpr (BPS == 1) {
-            p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[0], wf[0], zero, 0, 0, 0);
-            p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[1], wf[1], p[0], 0, 0, 0);
-        } else {
-            p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[0], wf[0], zero, 0, 0, 0);
-            p[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[1], wf[1], zero, 0, 0, 0);
+#pragma unroll
+            for (int t = 0; t < MT; ++t) af[t][j] = *(const bi8_v4i *)(mine + kAReg + SA * L::kAStage + t * kSlot + (frag ^ (j << 6)));
         }
 #pragma unroll
-        for (int b = 0; b < BPS; ++b) {
-            const float sw = *(const float *)(mine + kScReg + SW * kLdsGemvScales + b * 64 + r16 * 4);
-            const bi8_v4f sx = *(const bi8_v4f *)(mine + kScReg + SW * kLdsGemvScales + 128 + b * 64 + q * 16);
+        for (int t = 0; t < MT; ++t) {
+            bi8_v4i p[BPS];
+            if constexpr (BPS == 1) {
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[t][0], wf[0], zero, 0, 0, 0);
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[t][1], wf[1], p[0], 0, 0, 0);
+            } else {
+                p[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[t][0], wf[0], zero, 0, 0, 0);
+                p[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af[t][1], wf[1], zero, 0, 0, 0);
+            }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] = __builtin_fmaf((float)p[b][r] * sx[r], sw, acc[r]);
+            for (int b = 0; b < BPS; ++b) {
+                const float sw = *(const float *)(mine + kScReg + SW * L::kScales + b * 64 + r16 * 4);
+                const bi8_v4f sx = *(const bi8_v4f *)(mine + kScReg + SW * L::kScales + 128 + b * (64 * MT) + t * 64 + q * 16);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[t][r] = __builtin_fmaf((float)p[b][r] * sx[r], sw, acc[t][r]);
+            }
         }
     };
     for (int s = 0; s < nst; s += NSW) {
@@ -1681,33 +1702,29 @@ __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
         stage(s + 1, std::integral_constant<int, 1>{});
         stage(s + 2, std::integral_constant<int, 2>{});
         stage(s + 3, std::integral_constant<int, 3>{});
-        if constexpr (NSW > 4) {
-            stage(s + 4, std::integral_constant<int, 4>{});
-            stage(s + 5, std::integral_constant<int, 5>{});
-        }
-        if constexpr (NSW > 6) {
-            stage(s + 6, std::integral_constant<int, 6>{});
-            stage(s + 7, std::integral_constant<int, 7>{});
-        }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);            // vmcnt(0): nothing may still be writing LDS when the rings are reused
     __syncthreads();
-    float(*red)[4][64] = (float(*)[4][64])lds;     // [wave][register][lane], over the rings
+    float(*red)[MT * 4][64] = (float(*)[MT * 4][64])lds;            // [wave][register][lane], over the rings
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) red[wave][t * 4 + r][lane] = acc[t][r];
     __syncthreads();
     if (wave == 0) {
         const float div = (float)(1.0 / (127.0 * 127.0));
         const bool has_bias = g.bias != nullptr;
         const float bias = (has_bias && n < g.N) ? load_bias(g, n) : 0.0f;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            float v = red[0][r][lane];
+        for (int t = 0; t < MT; ++t)
 #pragma unroll
-            for (int w = 1; w < NW; ++w) v += red[w][r][lane];
-            const int64_t m = 4 * q + r;
-            if (m < g.M && n < g.N) store_c<CDT>(g.C, m * g.ldc + n, v * div, has_bias, bias);
-        }
+            for (int r = 0; r < 4; ++r) {
+                float v = red[0][t * 4 + r][lane];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) v += red[w][t * 4 + r][lane];
+                const int64_t m = 16 * t + 4 * q + r;
+                if (m < g.M && n < g.N) store_c<CDT>(g.C, m * g.ldc + n, v * div, has_bias, bias);
+            }
     }
 }
 
@@ -2219,6 +2236,7 @@ struct GemmPlan {
 // mostly empty round and the 256x256 kernel wins (1284 against 978 TOP/s at 2304x4096x4096, 144 tiles).
 // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
 constexpr int64_t kWideMinTiles = 129;
+constexpr int64_t kStagedMaxRows = 32;         // gemv_staged: one or two groups of 16 rows
 // `aligned`: A and W 16-byte aligned, the scales 4-byte aligned (the partials entry point has no scales);
 // ws_bytes: scratch memory the split kernels may use (0: none).
 // A last round of 256x256 tiles that is mostly empty costs as much as a full one (1280 x 11008 x 4096: 215 tiles, 69 us;
@@ -2261,14 +2279,14 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             p.kernel = kKRows;
             return p;
         }
-        if (M <= 16 && (block == 64 || block == 128) && (K / block + 16) * N * 4 < 0x3fffffffLL && 16 * ldw + K < 0x3fffffffLL &&
-            16 * lda + K < 0x3fffffffLL) {         // (gemv_staged addresses its buffers with 32-bit offsets)
+        if (M <= kStagedMaxRows && (block == 64 || block == 128) && (K / block + 16) * N * 4 < 0x3fffffffLL && 16 * ldw + K < 0x3fffffffLL &&
+            32 * lda + K < 0x3fffffffLL && (K / block + 16) * M * 4 < 0x3fffffffLL) {         // (gemv_staged addresses its buffers with 32-bit offsets)
             p.kernel = kKGemv;
             return p;
         }
         if (M <= 32) {
-            // 17 to 32 rows (and block 32): with scratch memory the split 64x128 tiles are ahead of the kernel that gathers
-            // its operands (block 128, 4096 -> 11008: 30-34 us against 17)
+            // (block 32) with scratch memory the split 64x128 tiles are ahead of the kernel that gathers its operands (measured
+            // at block 128, 4096 -> 11008, 17 to 32 rows: 30-34 us against 17)
             if (!try_split()) p.kernel = kKSkinny;
             return p;
         }
@@ -2332,21 +2350,24 @@ template <int BLK, int CDT> int launch_skinny(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-template <int BLK, int CDT> int launch_staged(GemmArgs g, hipStream_t st) {
+template <int BLK, int CDT, int NW, int MT> int launch_staged_as(const GemmArgs &g, unsigned tn, hipStream_t st) {
+    constexpr int lds = NW * GemvLds<MT>::kWaveBytes;
+    auto kern = gemv_staged<BLK, CDT, NW, MT>;
+    if (lds > 64 * 1024) {
+        static LdsOptIn opted;                     // one per kernel instantiation
+        const int rc = opted.ensure((const void *)kern, lds);
+        if (rc != BI8_OK) return rc;
+    }
+    hipLaunchKernelGGL(kern, dim3(tn), dim3(NW * 64), lds, st, g);
+    return bi8_launch_rc();
+}
+template <int BLK, int CDT> int launch_staged(const GemmArgs &g, hipStream_t st) {
     const int64_t tn = (g.N + 15) / 16;
     if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-    // eight waves per workgroup where four would leave CUs with a single workgroup's loads in flight
-    if (tn <= 384) {
-        constexpr size_t lds = 8 * kLdsGemvWaveBytes;
-        auto kern = gemv_staged<BLK, CDT, 8>;
-        static LdsOptIn opted;
-        const int rc = opted.ensure((const void *)kern, (int)lds);
-        if (rc != BI8_OK) return rc;
-        hipLaunchKernelGGL(kern, dim3((unsigned)tn), dim3(512), lds, st, g);
-    } else {
-        hipLaunchKernelGGL((gemv_staged<BLK, CDT, 4>), dim3((unsigned)tn), dim3(256), 4 * kLdsGemvWaveBytes, st, g);
-    }
-    return bi8_launch_rc();
+    // eight waves per workgroup where four would leave CUs with a single workgroup's loads in flight; up to 16 rows three
+    // workgroups of four waves share a CU, up to 32 rows (twice the A ring) two
+    if (g.M <= 16) return tn <= 384 ? launch_staged_as<BLK, CDT, 8, 1>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 1>(g, (unsigned)tn, st);
+    return tn <= 384 ? launch_staged_as<BLK, CDT, 8, 2>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 2>(g, (unsigned)tn, st);
 }
 
 template <int BLK, int CDT> int launch_rows(const GemmArgs &g, hipStream_t st) {

@@ -255,8 +255,8 @@ def _int8_matmul(a, b, state_x, state_w, bias=None, a_store=None, w_store=None):
         bias_ptr, bias_dt = bias.data_ptr(), _DT[bias.dtype]
     lib = _lib.load()
     # fewer output tiles than compute units: the library splits K over the workgroups if it is given scratch memory
-    # (up to 16 rows at blocks 64 / 128 run the one-pass decode kernels whatever they are given: not asked)
-    ws_bytes = lib.bi8_gemm_workspace_bytes(M, N, K, block) if M > 16 or block == 32 else 0
+    # (up to 32 rows at blocks 64 / 128 run the one-pass decode kernels whatever they are given: not asked)
+    ws_bytes = lib.bi8_gemm_workspace_bytes(M, N, K, block) if M > 32 or block == 32 else 0
     ws = torch.empty(ws_bytes, device=a.device, dtype=torch.uint8) if ws_bytes else None
     with _on_device(a):
         rc = lib.bi8_gemm_nt_dequant_ws(a.data_ptr(), w.data_ptr(), state_x.data_ptr(), state_w.data_ptr(),

@@ -224,8 +224,10 @@ def test_kernel_choice_by_shape():
     assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
     assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 11008, 4096, 64) == "gemv_staged"
     assert name(2, 4096, 32768, 128) == "gemv_staged"                  # 2 x 32768 codes do not fit the few-row kernel's LDS
-    assert name(16, 4096, 4096, 32) == "gemm_skinny" and name(24, 4096, 4096, 128) == "gemm_skinny"
-    assert name(24, 4096, 4096, 128, 1 << 30) == "gemm_tile_64x128_splitk"     # with scratch memory the split tiles are ahead
+    assert name(16, 4096, 4096, 32) == "gemm_skinny" and name(24, 4096, 4096, 32) == "gemm_skinny"     # block 32, few rows
+    assert name(24, 4096, 4096, 128) == "gemv_staged" and name(32, 11008, 4096, 64, 1 << 30) == "gemv_staged"   # two groups of 16 rows
+    assert name(24, 4096, 4096, 32, 1 << 30) == "gemm_tile_64x128_splitk"      # block 32 with scratch memory: the split tiles are ahead
+    assert name(33, 4096, 4096, 128, 1 << 30) == "gemm_tile_64x128_splitk"
     assert name(1, 128, 128 * 1024, 128) == "gemv_staged"            # any K: the scales stream through LDS with the stages
     assert name(128, 4096, 4096, 128) == "gemm_tile_128x128"         # no scratch memory: one pass
     ws = lib.bi8_gemm_workspace_bytes(128, 4096, 4096, 128)

@@ -162,10 +162,10 @@ def test_bias_dtypes_on_the_persistent_kernel(ops, out, block):
             assert torch.equal(Cb, C + bias.to(DTYPES[out]))             # added after the cast, in the output dtype
 
 
-@pytest.mark.parametrize("M,N,K", [(7, 11008, 2048), (16, 11008, 4096), (3, 8192, 2048)])
+@pytest.mark.parametrize("M,N,K", [(7, 11008, 2048), (16, 11008, 4096), (3, 8192, 2048), (17, 11008, 2048), (32, 8192, 4096), (25, 4096, 2048)])
 def test_small_batches_against_many_columns_call_after_call(ops, M, N, K):
-    """3 to 16 rows against more than 6144 columns run gemv_staged with four waves per workgroup, two or three workgroups
-    per CU.  Every wave streams W and A through a private LDS ring with direct-to-LDS loads; a load that overwrites a slot
+    """3 to 32 rows against more than 6144 columns run gemv_staged with four waves per workgroup, two or three workgroups
+    per CU (the last shape: eight waves, one workgroup per CU).  Every wave streams W and A through a private LDS ring with direct-to-LDS loads; a load that overwrites a slot
     must not be issued while the stage before is still reading it (a load of A, which the CU's L1 holds for the younger
     workgroups, can land within an LDS read's latency: such workgroups used to return wrong sums now and then).  Ten calls
     on fresh weights, each compared with the same rows run through the tile kernels inside a 33-row problem."""
@@ -401,8 +401,8 @@ def _run_nonfinite_few_rows(ops, A, W, block, g):
 # (M, N, K, kernel family)
 NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (5200, 5100, 256, "gemm_wide"),
                     (4400, 4500, 256, "gemm_wide+gemm_tile_128x128"), (2048, 2304, 256, "gemm_tile_256x128"),
-                    (8, 256, 512, "gemv_staged"), (24, 256, 512, "gemm_skinny"), (70, 90, 200, "gemm_generic"), (8, 256, 2560, "gemv_staged_long"),
-                    (2, 256, 1536, "gemv_rows")]
+                    (8, 256, 512, "gemv_staged"), (24, 256, 512, "gemv_staged_two_row_groups"), (24, 256, 512, "gemm_skinny", 32),
+                    (70, 90, 200, "gemm_generic"), (8, 256, 2560, "gemv_staged_long"), (2, 256, 1536, "gemv_rows")]
 
 
 @pytest.mark.parametrize("shape", NONFINITE_SHAPES, ids=lambda s: s[3])
@@ -413,9 +413,9 @@ def test_infinite_and_nan_scales(ops, shape):
     (M > 32), whose fold computes fma(1.5*2^23 + P, b, -1.5*2^23 * b), give NaN for the whole column instead of +-inf:
     the one place where non-finite results differ from the reference's, pinned here.  Everything else stays finite."""
     from blockwise_int8_linear_amd import _lib
-    M, N, K, family = shape
-    block = 128 if K % 128 == 0 else 64
-    assert _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, 0).decode() == family.replace("_long", "")
+    M, N, K, family = shape[:4]
+    block = shape[4] if len(shape) > 4 else 128 if K % 128 == 0 else 64
+    assert _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, 0).decode() == family.replace("_long", "").replace("_two_row_groups", "")
     g = torch.Generator().manual_seed(M + N)
     A, W = _codes(g, M, K), _codes(g, N, K)
     nblk = -(-K // block)
@@ -446,7 +446,7 @@ def test_infinite_and_nan_scales(ops, shape):
         ref = oracle_torch.int8_matmul_block_dequantize(A, W, sa, sw2, block, None, torch.float32)
         got = run(sa, sw2)
         assert ref[5, 2].isnan() and ref[:, 2].isinf().sum() >= M - 3
-        if family in ("gemv_staged", "gemv_staged_long", "gemm_skinny", "gemm_generic"):
+        if family in ("gemv_staged", "gemv_staged_long", "gemv_staged_two_row_groups", "gemm_skinny", "gemm_generic"):
             assert torch.equal(got.isnan(), ref.isnan()) and torch.equal(got[ref.isinf()], ref[ref.isinf()])
         else:
             assert got[:, 2].isnan().all()

@@ -102,8 +102,12 @@ CASES = [
     (7, 1000, 1152, 64, "gemv_staged"),
     (7, 8192, 2048, 128, "gemv_staged"),            # more than 6144 columns: four waves per workgroup, several workgroups per CU
     (12, 11008, 2048, 64, "gemv_staged"),
-    (24, 500, 640, 128, "gemm_skinny"),             # five stages of K: nothing to split
-    (24, 500, 2048, 128, "gemm_tile_64x128_splitk"),
+    (24, 500, 640, 128, "gemv_staged"),             # two groups of 16 rows
+    (32, 1000, 2048 + 128, 64, "gemv_staged"),
+    (17, 8192, 2048, 128, "gemv_staged"),           # ... four waves per workgroup, two workgroups per CU
+    (29, 11008, 1024, 64, "gemv_staged"),
+    (24, 500, 640, 32, "gemm_skinny"),              # block 32, five stages of K: nothing to split
+    (24, 500, 2048, 32, "gemm_tile_64x128_splitk"),
     (16, 300, 1024, 32, "gemm_skinny"),
     (128, 1024, 4096, 128, "gemm_tile_64x128_splitk"),
     (512, 4096, 4096, 64, "gemm_tile_128x128_splitk"),
