@@ -174,7 +174,7 @@ def bench_extras(pkg, torch):
         nset = max(2, int(600e6 // (N * K)))
         ws = [torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8) for _ in range(nset)]
         sw = torch.rand(K // B, N, device="cuda") * 0.02
-        for M in (1, 16):
+        for M in (1, 16, 32):
             x = torch.randint(-127, 128, (M, K), device="cuda", dtype=torch.int8)
             sx = torch.rand(K // B, M, device="cuda") + 0.5
             c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
@@ -211,6 +211,24 @@ def bench_extras(pkg, torch):
                 t1 = min(event_ms(one, 50) for _ in range(2))
                 out[f"decode_linear_M1_K{K}_N{N}"] = {"one_kernel_us": round(t1 * 1e3, 2), "two_launches_us": round(t2 * 1e3, 2)}
         del ws
+
+    # Llama-7B prefill shapes at 2048 tokens (the first: 344 tiles of 256x256, run as 256 of them and a second launch)
+    for (M, N, K) in ((2048, 11008, 4096), (2048, 4096, 4096)):
+        x = torch.randint(-127, 128, (M, K), device="cuda", dtype=torch.int8)
+        w = torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8)
+        sx = torch.rand(K // B, M, device="cuda") + 0.5
+        sw = torch.rand(K // B, N, device="cuda") * 0.02
+        c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+
+        def gp():
+            assert lib.bi8_gemm_nt_dequant(x.data_ptr(), w.data_ptr(), sx.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
+                                           M, N, K, K, K, N, B, st) == 0
+        for _ in range(20):
+            gp()
+        t = min(event_ms(gp, 30) for _ in range(2))
+        out[f"prefill_gemm_M{M}_K{K}_N{N}"] = {"us": round(t * 1e3, 1), "TOPS": round(2.0 * M * N * K / t / 1e9, 1),
+                                               "kernel": lib.bi8_gemm_kernel_name(M, N, K, K, K, B, 0).decode()}
+        del x, w, c
 
     M = K = 8192
     xs = [torch.randn(M, K, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3)]
