@@ -65,3 +65,39 @@ def test_quantizers_call_after_call(pkg, shape, block):
         assert torch.equal(a[0], q1) and torch.equal(a[1], s1)
         qt, st = pkg.quantize_block_rowwise(x.t().contiguous(), block)
         assert torch.equal(a[2], qt) and torch.equal(a[3], st)
+
+
+@pytest.mark.parametrize("M,N,K,block", [(1536, 11008, 4096, 128), (3072, 768, 8192, 64), (24, 11008, 4096, 128), (128, 4096, 4096, 128),
+                                         (4352, 4096, 2048, 128)])
+def test_plans_of_several_launches_in_a_hip_graph(pkg, M, N, K, block):
+    """the cut (256x256 kernel + tile kernel), the split (tile kernel + reduce, with its workspace from torch's allocator)
+    and the few-row kernel recorded into a HIP graph: every replay, with eager work between the replays, equals the eager
+    call"""
+    cfg = pkg.block_linear_config
+    old = (cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE)
+    cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = block, torch.bfloat16
+    try:
+        g = torch.Generator().manual_seed(M + N)
+        A, W = _codes(g, M, K), _codes(g, N, K)
+        sa = (torch.rand(K // block, M, generator=g) + 0.5).to(DEV)
+        sw = (torch.rand(K // block, N, generator=g) * 0.02 + 1e-3).to(DEV)
+        bias = torch.randn(N, generator=g).to(torch.bfloat16).to(DEV)
+        eager = pkg.int8_matmul_block64_rowwise_dequantize(A, W.t(), sa, sw, bias)
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            pkg.int8_matmul_block64_rowwise_dequantize(A, W.t(), sa, sw, bias)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = pkg.int8_matmul_block64_rowwise_dequantize(A, W.t(), sa, sw, bias)
+        for _ in range(3):
+            out.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+            torch.randn(1 << 20, device=DEV).sum().item()              # eager work and a synchronization between replays
+    finally:
+        cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE = old
