@@ -48,6 +48,12 @@ def event_ms(fn, iters: int) -> float:
     return start.elapsed_time(stop) / iters
 
 
+def median_ms(fn, iters: int, reps: int = 3) -> float:
+    """median of `reps` averages over `iters` back-to-back launches"""
+    ts = sorted(event_ms(fn, iters) for _ in range(reps))
+    return ts[len(ts) // 2]
+
+
 def preroll(fn, torch):
     """Untimed launches until the chip's clocks have settled: after idle the first launches run at ramping clocks (up
     to 30 % slower, for about a hundred launches).  Batches of PREROLL_BATCH launches are timed with events until three
@@ -75,8 +81,9 @@ def bench_quantize(pkg, torch, iters: int):
         gen = torch.Generator(device="cuda").manual_seed(i)
         x = torch.randn(M, K, device="cuda", generator=gen, dtype=torch.float32)
         gen1 = torch.Generator(device="cuda").manual_seed(100 + i)
-        pos = torch.randint(0, E, (E // 1000,), device="cuda", generator=gen1)
+        pos = torch.randperm(E, device="cuda", generator=gen1)[:E // 1000]      # distinct positions: exactly 0.1 %
         x.view(-1)[pos] *= 50.0
+        del pos
         xs.append(x.to(torch.bfloat16))
         del x
     st = torch.cuda.current_stream().cuda_stream
@@ -101,8 +108,10 @@ def bench_quantize(pkg, torch, iters: int):
             for _ in range(2 * NSETS):
                 f()
         torch.cuda.synchronize()
-        tq = min(event_ms(fq, iters) for _ in range(3))
-        td = min(event_ms(fd, iters) for _ in range(3))
+        # five averages over `iters` launches each: the median is the figure reported, the best one next to it
+        tqs = sorted(event_ms(fq, iters) for _ in range(5))
+        tds = sorted(event_ms(fd, iters) for _ in range(5))
+        tq, td = tqs[2], tds[2]
         nbytes = E * 3 + 4 * E // B                 # read 2 B + write 1 B per element (or the reverse) + scales
         mse = ((ds[0].float() - xs[0].float()) ** 2).mean().item()
         out[f"block{B}"] = {
@@ -111,6 +120,8 @@ def bench_quantize(pkg, torch, iters: int):
             "quantize_frac_hbm": round(nbytes / tq / 1e6 / HBM_PEAK_GBS, 4),
             "dequantize_us": round(td * 1e3, 2), "dequantize_GBps": round(nbytes / td / 1e6, 1),
             "dequantize_frac_hbm": round(nbytes / td / 1e6 / HBM_PEAK_GBS, 4),
+            "quantize_best_us": round(tqs[0] * 1e3, 2), "dequantize_best_us": round(tds[0] * 1e3, 2),
+            "timing": f"median of 5 averages over {iters} launches (best next to it)",
             "roundtrip_mse": mse,
         }
         del qs, ss, ds
@@ -118,7 +129,8 @@ def bench_quantize(pkg, torch, iters: int):
 
 
 def bench_extras(pkg, torch):
-    """secondary figures of the same path, all through the C ABI with preallocated outputs: the block-64 GEMM at
+    """secondary figures of the same path (each the median of three averages over a run of back-to-back launches), all
+    through the C ABI with preallocated outputs: the block-64 GEMM at
     8192^3, the few-row (decode) GEMM at Llama-7B shapes with the weights rotated through ~600 MB so that they come
     from HBM (and the one-token eval-path linear, quantize included, as two launches and as one kernel), the
     transposed quantizer of the backward pass and the quantizer that writes both directions from one read"""
@@ -137,7 +149,7 @@ def bench_extras(pkg, torch):
         assert lib.bi8_gemm_nt_dequant(a.data_ptr(), w.data_ptr(), sa.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
                                        S, S, S, S, S, S, B, st) == 0
     g64()
-    t = min(event_ms(g64, 10) for _ in range(2))
+    t = median_ms(g64, 10)
     out["gemm_block64_8192"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1)}
     del sa, sw, c
 
@@ -149,7 +161,7 @@ def bench_extras(pkg, torch):
         wt = w.t()
         for _ in range(30):
             torch._int_mm(a, wt)
-        t = min(event_ms(lambda: torch._int_mm(a, wt), 30) for _ in range(2))
+        t = median_ms(lambda: torch._int_mm(a, wt), 30)
         out["context_vendor_plain_int8_gemm_8192_random_codes"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1),
                                                                    "what": "torch._int_mm (hipBLASLt), int32 out, no dequantize"}
     except Exception as e:                          # not every torch build has it: the figure is context only
@@ -165,7 +177,7 @@ def bench_extras(pkg, torch):
                                        S, S, S, S, S, S, 128, st) == 0
     for _ in range(30):
         gz()
-    t = min(event_ms(gz, 20) for _ in range(2))
+    t = median_ms(gz, 20)
     out["context_gemm_block128_8192_zero_codes"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1)}
     del z, sa, sw, c
 
@@ -186,7 +198,7 @@ def bench_extras(pkg, torch):
                                                M, N, K, K, K, N, B, st) == 0
             for _ in range(5):
                 gv()
-            t = min(event_ms(gv, 50) for _ in range(2))
+            t = median_ms(gv, 50)
             nbytes = N * K + 4 * (K // B) * (N + M) + M * K + 2 * M * N
             out[f"decode_gemm_M{M}_K{K}_N{N}"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
                                                   "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
@@ -207,8 +219,8 @@ def bench_extras(pkg, torch):
                                                    M, N, K, K, K, N, B, st) == 0
                 for _ in range(5):
                     two(), one()
-                t2 = min(event_ms(two, 50) for _ in range(2))
-                t1 = min(event_ms(one, 50) for _ in range(2))
+                t2 = median_ms(two, 50)
+                t1 = median_ms(one, 50)
                 out[f"decode_linear_M1_K{K}_N{N}"] = {"one_kernel_us": round(t1 * 1e3, 2), "two_launches_us": round(t2 * 1e3, 2)}
         del ws
 
@@ -225,7 +237,7 @@ def bench_extras(pkg, torch):
                                            M, N, K, K, K, N, B, st) == 0
         for _ in range(20):
             gp()
-        t = min(event_ms(gp, 30) for _ in range(2))
+        t = median_ms(gp, 30)
         out[f"prefill_gemm_M{M}_K{K}_N{N}"] = {"us": round(t * 1e3, 1), "TOPS": round(2.0 * M * N * K / t / 1e9, 1),
                                                "kernel": lib.bi8_gemm_kernel_name(M, N, K, K, K, B, 0).decode()}
         del x, w, c
@@ -241,7 +253,7 @@ def bench_extras(pkg, torch):
         assert lib.bi8_quantize_transposed(xs[i].data_ptr(), 1, qs[i].data_ptr(), ss[i].data_ptr(), M, K, K, M, 128, st) == 0
     for _ in range(6):
         qt()
-    t = min(event_ms(qt, 30) for _ in range(2))
+    t = median_ms(qt, 30)
     nbytes = M * K * 3 + 4 * M * K // 128
     out["quantize_transposed_bf16_8192"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
                                             "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
@@ -256,7 +268,7 @@ def bench_extras(pkg, torch):
                                      M, K, K, K, M, 128, st) == 0
     for _ in range(6):
         qd()
-    t = min(event_ms(qd, 30) for _ in range(2))
+    t = median_ms(qd, 30)
     nbytes = M * K * 4 + 8 * M * K // 128
     out["quantize_dual_bf16_8192"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
                                       "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
@@ -271,7 +283,7 @@ def bench_extras(pkg, torch):
         ds[i].copy_(xs[i])
     for _ in range(6):
         cp()
-    t = min(event_ms(cp, 30) for _ in range(2))
+    t = median_ms(cp, 30)
     nbytes = 2 * xs[0].numel() * xs[0].element_size()
     out["context_device_copy_128MiB"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
                                          "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4), "what": "torch dst.copy_(src), read + write"}
@@ -366,7 +378,7 @@ def main():
     ops_per_launch = 2.0 * S * S * S
     kern_ms = evs[0].elapsed_time(evs[-1]) / args.steps
     per_launch = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
-    median_ms = per_launch[len(per_launch) // 2] if len(per_launch) % 2 else 0.5 * (per_launch[len(per_launch) // 2 - 1] + per_launch[len(per_launch) // 2])
+    launch_median = per_launch[len(per_launch) // 2] if len(per_launch) % 2 else 0.5 * (per_launch[len(per_launch) // 2 - 1] + per_launch[len(per_launch) // 2])
     achieved = ops_per_launch / kern_ms / 1e9       # TOPS
     lib = _lib.load()
     kernel = lib.bi8_gemm_kernel_name(S, S, S, S, S, B, lib.bi8_gemm_workspace_bytes(S, S, S, B)).decode()
@@ -386,7 +398,7 @@ def main():
                      "traffic": GEMM_8192_TRAFFIC_BYTES if (S == 8192 and B == 128) else None,
                      "traffic_source": GEMM_8192_TRAFFIC_SOURCE if (S == 8192 and B == 128) else None,
                      "kernel": f"{kernel}<{B},bf16> (the library's choice for this shape: bi8_gemm_kernel_name)",
-                     "ops_per_launch": ops_per_launch, "avg_launch_ms": round(kern_ms, 4), "median_launch_ms": round(median_ms, 4),
+                     "ops_per_launch": ops_per_launch, "avg_launch_ms": round(kern_ms, 4), "median_launch_ms": round(launch_median, 4),
                      "frac_of_5033_TOPs_at_2p4GHz": round(achieved / 5033.2, 4),
                      "preroll_launches": preroll_launches, "preroll_last_batch_ms": None if preroll_ms is None else round(preroll_ms, 4)},
     }

@@ -11,8 +11,8 @@ Differences from the reference that do not change results:
     fp32 sums in a fixed order);
   * switching the module back to training mode drops the cached int8 weights, so a later ``eval()``
     re-quantizes the current weights (the reference keeps serving the first cache, block_linear.py:138-139);
-  * the eval path with at most 4 rows (token-by-token decode) quantizes and multiplies in one kernel
-    (block_linear.py:141-144 are two launches);
+  * the eval path with one or two rows (token-by-token decode) quantizes and multiplies in one kernel
+    (block_linear.py:141-144 are two launches; from three rows on the two launches run);
   * ``blockwise_int8_linear_Wint8`` is the working form of the reference's function of that name
     (block_linear.py:42-67, which passes un-quantized activations to the GEMM and multiplies the gradient with weight
     codes blocked along the wrong dimension): the forward pass runs on weight codes quantized ahead of time, the
@@ -22,6 +22,7 @@ from __future__ import annotations
 
 import torch
 import torch.nn as nn
+from torch.optim.optimizer import register_optimizer_step_post_hook
 
 from . import block_linear_config
 from .ops import (
@@ -57,6 +58,18 @@ def replace_linear_with_blockwise_int8(model):
         new.train(module.training)
         model._modules[name] = new
     return model
+
+
+# Every optimizer step in the process moves this count, which is part of the state the cached int8 weights are keyed on:
+# optimizers that update through ``p.data`` (apex- and DeepSpeed-style) leave the parameter's version counter alone.
+_optimizer_steps = [0]
+
+
+def _count_optimizer_step(optimizer, args, kwargs):
+    _optimizer_steps[0] += 1
+
+
+register_optimizer_step_post_hook(_count_optimizer_step)
 
 
 class blockwise_int8_linear(torch.autograd.Function):
@@ -188,19 +201,30 @@ class BlockInt8Linear(nn.Linear):
     Eval mode: weights quantized once into the buffers ``W_int8`` [N,K] int8 and ``state_W``
     [ceil(K/B),N], activations quantized per call, one fused GEMM."""
 
-    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None):
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, device=None, dtype=None, *,
+                 quantized_weight_training: bool = False):
         super().__init__(in_features, out_features, bias, device, dtype)
         # training on weight codes quantized ahead of the step (blockwise_int8_linear_Wint8): the codes are made when
         # the weight has changed since they were last made (frozen weights, several micro-batches per optimizer step:
         # once), not in every forward and again in every backward pass
-        self.quantized_weight_training = False
+        self.quantized_weight_training = quantized_weight_training
         self._train_cache = None
         self._eval_cache_of = None                 # state of the weight the eval cache was quantized from
+        self._invalidations = 0
 
     def _weight_state(self):
-        """changes whenever the weight's values may have: in-place updates bump the version, assignments move the data"""
+        """Changes whenever the weight's values may have: in-place updates through the parameter bump its version,
+        assignments move the data, every ``torch.optim`` optimizer step anywhere in the process moves the step count
+        (an optimizer that writes through ``p.data`` bumps no version), and ``invalidate_quantized_weight()`` covers
+        the writes that none of these see (``p.data.copy_(ema)`` outside an optimizer)."""
         w = self.weight
-        return (w._version, w.data_ptr(), block_linear_config.GROUP_SIZE)
+        return (w._version, w.data_ptr(), block_linear_config.GROUP_SIZE, _optimizer_steps[0], self._invalidations)
+
+    def invalidate_quantized_weight(self):
+        """Drop the cached int8 copies of the weight (eval cache and quantized-weight-training cache): the next forward
+        quantizes the weight again.  Needed after the weight's VALUES were changed behind the parameter's back, i.e.
+        through ``weight.data`` outside a ``torch.optim`` optimizer step; every other kind of update is noticed."""
+        self._invalidations += 1
 
     def prepare_for_eval(self):
         W_int8, state_W = quantize_block_rowwise(self.weight.detach())

@@ -2275,7 +2275,8 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     // (the rest of a cut problem shares the whole problem's pointers and strides, which only the tile kernels take)
     if (!partials && !rest_of_cut) {
         if (M <= kRowsMax && (block == 64 || block == 128) &&
-            (block == 64 ? rows_lds_bytes<64>(M, K, 0) : rows_lds_bytes<128>(M, K, 0)) <= kRowsLdsMax && (K / block + 16) * N * 4 < 0x7fffffffLL) {
+            (block == 64 ? rows_lds_bytes<64>(M, K, 0) : rows_lds_bytes<128>(M, K, 0)) <= kRowsLdsMax && (K / block + 16) * N * 4 < kBufOut) {
+            // (offsets of kBufOut and beyond mark lanes that load nothing: every buffer of the kernel has to end below it)
             p.kernel = kKRows;
             return p;
         }
@@ -2581,7 +2582,7 @@ extern "C" int bi8_linear_few_rows(const void *x, int dtype, const int8_t *W, co
     if (!x || !W || !sW || !C) return BI8_ERR_NULL_POINTER;
     const int64_t vec = dtype == BI8_F32 ? 4 : 8;
     if (M < 1 || M > kRowsMax || N < 1 || (block != 64 && block != 128) || K < kStageK || K % kStageK != 0 || ldx % vec != 0 ||
-        ldw % 16 != 0 || ldw >= (1 << 22) || (K / block) * N * 4 >= 0x7fffffffLL || !bi8_aligned(x, 16) || !bi8_aligned(W, 16) ||
+        ldw % 16 != 0 || ldw >= (1 << 22) || (K / block + 16) * N * 4 >= kBufOut || !bi8_aligned(x, 16) || !bi8_aligned(W, 16) ||
         !bi8_aligned(sW, 4) || (N + 15) / 16 > 0x7fffffffLL)
         return BI8_ERR_UNSUPPORTED;
     const size_t lds = block == 64 ? rows_lds_bytes<64>(M, K, bi8_dtype_size(dtype)) : rows_lds_bytes<128>(M, K, bi8_dtype_size(dtype));

@@ -51,14 +51,17 @@ def _do_bench(fn, warmup=5, rep=20, quantiles=(0.5, 0.2, 0.8)):
     return [torch.quantile(t, q).item() for q in quantiles]
 
 
-def benchmark(sizes=None, K=512, providers=("dense", "blockwise_int8", "blockwise_int8_quantise", "dense+copy"), print_data=True):
+def benchmark(sizes=None, K=512, providers=("dense", "int8 matmul", "blockwise_int8", "blockwise_int8_quantise", "dense+copy"),
+              print_data=True):
     """The reference's sweep (triton_functions.py:521-566): square M = N, fixed K = 512, operands of
     INPUT_OUTPUT_TORCH_TYPE; TOP/s = 2*M*N*K / median time, with the 0.2 / 0.8 quantiles.
       dense                    torch.matmul in bf16 (hipBLASLt)               -- the reference's 'cublas' line
+      int8 matmul              the vendor library's plain int8 GEMM, int32 out, no scales (torch._int_mm, hipBLASLt) on
+                               the quantized codes -- the reference's line of that name (triton_functions.py:547-552, there
+                               through its torch_cublas_matmul_int8 extension)
       blockwise_int8           the int8 GEMM with fused dequantize alone, operands quantized beforehand
       blockwise_int8_quantise  quantize both operands + that GEMM
       dense+copy               copy_then_matmul
-    The reference's 'int8 matmul' line needs its torch_cublas_matmul_int8 extension, which it does not ship.
     Returns {provider: [(M, median, q80, q20), ...]}."""
     sizes = sizes or [1024 * i for i in range(2, 16, 2)]
     dtype = block_linear_config.INPUT_OUTPUT_TORCH_TYPE
@@ -71,6 +74,11 @@ def benchmark(sizes=None, K=512, providers=("dense", "blockwise_int8", "blockwis
             if p == "dense":
                 a16, b16 = a.to(torch.bfloat16), b.to(torch.bfloat16)
                 fn = lambda: torch.matmul(a16, b16)
+            elif p == "int8 matmul":
+                qa, _ = quantize_block_rowwise(a)
+                qb, _ = quantize_block_rowwise(b.t().contiguous())
+                qbt = qb.t()                        # [K,N], K contiguous: the layout the blockwise GEMM is given too
+                fn = lambda: torch._int_mm(qa, qbt)
             elif p == "dense+copy":
                 fn = lambda: copy_then_matmul(a, b)
             elif p == "blockwise_int8":

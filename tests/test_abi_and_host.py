@@ -101,7 +101,10 @@ def test_python_api_mirrors_reference_names_and_defaults():
     assert list(inspect.signature(ops.dequantize_block_rowwise).parameters) == ["x", "state_x", "fblock_size"]
     assert list(inspect.signature(ops.int8_matmul_block64_rowwise_dequantize).parameters) == ["a", "b", "state_x", "state_w", "bias"]
     assert inspect.signature(ops.int8_matmul_block64_rowwise_dequantize).parameters["bias"].default is None
-    assert list(inspect.signature(pkg.BlockInt8Linear.__init__).parameters) == ["self", "in_features", "out_features", "bias", "device", "dtype"]
+    # the reference's positional parameters, then one keyword-only addition
+    sig = inspect.signature(pkg.BlockInt8Linear.__init__).parameters
+    assert list(sig) == ["self", "in_features", "out_features", "bias", "device", "dtype", "quantized_weight_training"]
+    assert sig["quantized_weight_training"].kind is inspect.Parameter.KEYWORD_ONLY and sig["quantized_weight_training"].default is False
     for name in ("prepare_for_eval", "infer", "forward", "weight_quant_training"):
         assert callable(getattr(pkg.BlockInt8Linear, name))
     assert issubclass(pkg.BlockInt8Linear, nn.Linear) and issubclass(pkg.blockwise_int8_linear, torch.autograd.Function)
@@ -148,6 +151,21 @@ def test_model_surgery_on_cpu_modules():
     assert len(lins) == 3 and all(isinstance(m, pkg.BlockInt8Linear) and m.training for m in lins)
     assert [p.data_ptr() for p in net2.parameters()] == ptrs and lins[2].bias is None
     assert not lins[0].quantized_weight_training
+    # the state that the cached int8 weights are keyed on moves with in-place updates, with any optimizer step of the
+    # process (optimizers that write through .data bump no version) and with an explicit invalidation
+    lin = pkg.BlockInt8Linear(8, 4, quantized_weight_training=True)
+    assert lin.quantized_weight_training
+    seen = {lin._weight_state()}
+    with torch.no_grad():
+        lin.weight.mul_(2.0)
+    seen.add(lin._weight_state())
+    lin.weight.data.mul_(2.0)                                   # invisible ...
+    assert lin._weight_state() in seen
+    torch.optim.SGD([nn.Parameter(torch.zeros(1))], lr=0.1).step()         # ... unless an optimizer step went by
+    seen.add(lin._weight_state())
+    lin.invalidate_quantized_weight()
+    seen.add(lin._weight_state())
+    assert len(seen) == 4
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):

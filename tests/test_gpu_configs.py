@@ -204,7 +204,7 @@ def test_reference_benchmark_sweep_and_accuracy_demo(pkg):
     from blockwise_int8_linear_amd import triton_functions as tf
     from blockwise_int8_linear_amd.examples import accuracy
     rows = tf.benchmark(sizes=[256, 512], print_data=False)
-    assert set(rows) == {"dense", "blockwise_int8", "blockwise_int8_quantise", "dense+copy"}
+    assert set(rows) == {"dense", "int8 matmul", "blockwise_int8", "blockwise_int8_quantise", "dense+copy"}
     assert all(len(v) == 2 and all(r[1] > 0 for r in v) for v in rows.values())
     a = torch.randn(70, 256, device=DEV).bfloat16()
     b = torch.randn(90, 256, device=DEV).bfloat16()

@@ -145,6 +145,57 @@ def test_eval_cache_follows_the_weight(pkg):
         assert_close_rms(y2.cpu(), ref2, 1e-2, b.bias.detach().cpu())
 
 
+class _DataSGD(torch.optim.Optimizer):
+    """an optimizer of the kind that updates through ``p.data`` (apex / DeepSpeed style): no version counter moves"""
+
+    def __init__(self, params, lr):
+        super().__init__(params, {"lr": lr})
+
+    @torch.no_grad()
+    def step(self):
+        for group in self.param_groups:
+            for p in group["params"]:
+                if p.grad is not None:
+                    p.data.add_(p.grad.data, alpha=-group["lr"])
+
+
+def test_cached_codes_follow_updates_made_through_data(pkg):
+    """The quantized-weight-training cache and the eval cache are keyed on more than the parameter's version counter:
+    an optimizer that writes through ``p.data`` is seen through the process-wide optimizer step count, and a bare
+    ``weight.data`` edit through ``invalidate_quantized_weight()``.  Each forward is compared with a module that holds
+    the same weight and no cache."""
+    with config_as(pkg, 128, torch.bfloat16):
+        torch.manual_seed(1)
+        lin = pkg.BlockInt8Linear(256, 128, device=DEV, dtype=torch.bfloat16, quantized_weight_training=True)
+        assert lin.quantized_weight_training
+        fresh = lambda: pkg.blockwise_int8_linear.apply(x, lin.weight.detach(), lin.bias.detach())
+        x = torch.randn(32, 256, device=DEV, dtype=torch.bfloat16)
+        y0 = lin(x)
+        assert torch.equal(y0, fresh())
+        opt = _DataSGD(lin.parameters(), lr=0.5)
+        y0.float().pow(2).mean().backward()
+        v = lin.weight._version
+        opt.step()
+        assert lin.weight._version == v                         # nothing the version counter could have told
+        y1 = lin(x)
+        assert torch.equal(y1, fresh()) and not torch.equal(y1, y0)
+        # a bare edit through .data: the module has to be told
+        lin.weight.data.mul_(2.0)
+        assert torch.equal(lin(x), y1)                          # (documented: stale until invalidated)
+        lin.invalidate_quantized_weight()
+        y2 = lin(x)
+        assert torch.equal(y2, fresh()) and not torch.equal(y2, y1)
+        # the eval cache is keyed the same way
+        lin.eval()
+        with torch.no_grad():
+            e0 = lin(x)
+            lin.weight.data.mul_(0.5)
+            lin.invalidate_quantized_weight()
+            e1 = lin(x)
+            q, s = pkg.quantize_block_rowwise(lin.weight.detach())
+        assert torch.equal(lin.W_int8, q) and torch.equal(lin.state_W, s) and not torch.equal(e0, e1)
+
+
 def test_recursive_surgery(pkg):
     class Inner(nn.Module):
         def __init__(self):

@@ -2,7 +2,9 @@
 static array in device memory that the library owns.  Called here straight through the C ABI and compared bit for bit
 with bi8_gemm_nt_dequant_ws (caller-provided workspace) on the same operands: two calls in a row, the second on a
 smaller problem (the array still holds the first call's slabs), then a problem that does not split at all, and the
-first one again.  Outputs of the existing entry point are themselves checked against the CPU checker."""
+first one again; one case passes operands whose rows are longer than K (leading dimensions above K).  Outputs of the
+existing entry point are themselves checked against the CPU checker.  "Allocates nothing" is checked on the device's
+own count of free memory (hipMemGetInfo), which a hipMalloc inside the library would move, and on torch's allocator."""
 
 import pytest
 import torch
@@ -29,26 +31,35 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point():
     torch.cuda.set_device(0)
     st = torch.cuda.current_stream().cuda_stream
     assert lib.bi8_static_scratch_bytes() == 32 << 20
-    # (M, N, K, block, out dtype code, splits?)  larger problem first, then a smaller one, one without a split, the first again
-    cases = [(3072, 768, 8192, 64, 1, True), (128, 1024, 4096, 128, 0, True), (64, 256, 2048, 128, 1, True),
-             (300, 500, 512, 128, 0, False), (3072, 768, 8192, 64, 1, True)]
+    # (M, N, K, block, out dtype code, splits?, extra row length of A and W)  larger problem first, then a smaller one, one
+    # with padded rows, one without a split, the first again
+    cases = [(3072, 768, 8192, 64, 1, True, 0), (128, 1024, 4096, 128, 0, True, 0), (64, 256, 2048, 128, 1, True, 0),
+             (128, 512, 4096, 128, 1, True, 256), (300, 500, 512, 128, 0, False, 0), (3072, 768, 8192, 64, 1, True, 0)]
     dts = {0: torch.float32, 1: torch.bfloat16}
     torch.cuda.synchronize()
-    for i, (M, N, K, block, cdt, splits) in enumerate(cases):
+    for i, (M, N, K, block, cdt, splits, pad) in enumerate(cases):
         A, W, sa, sw, bias = _problem(M, N, K, block, 100 + i)
-        Ad, Wd, sad, swd, bd = (t.to(DEV) for t in (A, W, sa, sw, bias))
+        sad, swd, bd = (t.to(DEV) for t in (sa, sw, bias))
+        # operands as views of buffers with rows of K + pad codes (the padding holds codes that must not be read)
+        Ad = torch.full((M, K + pad), 77, device=DEV, dtype=torch.int8)[:, :K]
+        Wd = torch.full((N, K + pad), -77, device=DEV, dtype=torch.int8)[:, :K]
+        Ad.copy_(A)
+        Wd.copy_(W)
         need = lib.bi8_gemm_workspace_bytes(M, N, K, block)
         assert (need > 0) == splits and need <= lib.bi8_static_scratch_bytes()
         ws = torch.empty(max(need, 16), device=DEV, dtype=torch.uint8)
         c_ws = torch.empty(M, N, device=DEV, dtype=dts[cdt])
         c_st = torch.full((M, N), float("nan"), device=DEV, dtype=dts[cdt])
         args = (Ad.data_ptr(), Wd.data_ptr(), sad.data_ptr(), swd.data_ptr(), bd.data_ptr(), 0)
-        dims = (M, N, K, K, K, N, block)
+        dims = (M, N, K, K + pad, K + pad, N, block)
         assert lib.bi8_gemm_nt_dequant_ws(*args, c_ws.data_ptr(), cdt, *dims, ws.data_ptr(), need, st) == 0
-        before = torch.cuda.memory_allocated()
-        assert lib.bi8_gemm_nt_dequant_static(*args, c_st.data_ptr(), cdt, *dims, st) == 0
-        assert torch.cuda.memory_allocated() == before
         torch.cuda.synchronize()
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+        assert lib.bi8_gemm_nt_dequant_static(*args, c_st.data_ptr(), cdt, *dims, st) == 0
+        torch.cuda.synchronize()
+        # (the first call on a device makes the runtime look up the array's address; the array itself is part of the
+        # loaded code object, so not even that call takes device memory)
+        assert torch.cuda.memory_allocated() == before and torch.cuda.mem_get_info()[0] == free_before
         assert torch.equal(c_st, c_ws), f"case {i}: static-scratch output differs from the workspace output"
         # and against the CPU checker; the bias is added to the rounded product in the output type, so the relative
         # bound counts the magnitudes of both, and where the products differ the rounding of the sum can add one more

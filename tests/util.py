@@ -36,7 +36,7 @@ def outlier_tensor(M: int, K: int, dtype=torch.bfloat16, seed: int = 0, frac: fl
     g1 = torch.Generator().manual_seed(seed + 1)
     n_out = int(E * frac)
     if n_out:
-        pos = torch.randint(0, E, (n_out,), generator=g1)
+        pos = torch.randperm(E, generator=g1)[:n_out]            # distinct positions: exactly n_out outliers
         x.view(-1)[pos] *= scale
     return x.to(dtype)
 
