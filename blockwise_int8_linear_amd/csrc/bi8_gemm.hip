@@ -9,7 +9,9 @@
 //                grid; when its last round of tiles would be mostly empty it runs on the leading rows or columns only and
 //                a gemm_tile launch takes the rest;
 //   gemm_wide32  block 32, same problems and tile: v_mfma_i32_32x32x32_i8, 32x256 per wave;
-//   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x192 / 128x128 / 64x128 tiles; also the int32
+//   gemm_wide<.., 4>  the same kernel on 256x128 tiles (64x64 per wave) for problems of more than 256 tiles of 128x128 that
+//                do not fill the chip with 256x256 tiles (Llama prefill at 2048 tokens, the GPT-2 layer GEMMs);
+//   gemm_tile    blocks 32/64/128: v_mfma_i32_32x32x32_i8, 256x128 / 128x128 / 64x128 tiles; also the int32
 //                block partials, and (SPLIT) fp32 partial sums over part of K for problems of fewer tiles than CUs, which
 //                splitk_reduce adds up;
 //   gemv_rows    M <= 2, blocks 64/128 (single-token decode; also bi8_linear_few_rows, which quantizes the activations in
@@ -720,13 +722,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // of the XCD-aware order and never drains its pipeline between them, so a tile's outputs leave (through a small
 // wave-private LDS strip) while the next tile's first stages land.  Measured against one workgroup per tile:
 // 8192^3 -1.5 %, 8192 x 50257 x 768 -13 %.
-template <int NBS> struct WideLds {                 // NBS = K-blocks per stage
-    static constexpr int kABuf = 256 * kStageK, kWBuf = 256 * kStageK;       // 32 KiB per operand per stage
+template <int NBS, int BN = 256> struct WideLds {   // NBS = K-blocks per stage, BN = columns of the tile (256 or 128)
+    static constexpr int kABuf = 256 * kStageK, kWBuf = BN * kStageK;        // 32 KiB (16 KiB) per operand per stage
     static constexpr int kSRow = 256 * 4;                                    // one row-scale row of the tile
     static constexpr int kSBuf = NBS * kSRow;                                // the stage's row scales, one row per K-block
     // column scales are stored prepared: per column the pair (b, -1.5*2^23*b), b = the scale rounded to 22 significant
-    // bits; a wave's 128 columns as [column pair 2p, 2p+1][r16][b0, c0, b1, c1], so a lane reads two columns' pairs at once
-    static constexpr int kCRow = 256 * 8;
+    // bits; a wave's BN/2 columns as [column pair 2p, 2p+1][r16][b0, c0, b1, c1], so a lane reads two columns' pairs at once
+    static constexpr int kCRow = BN * 8;
     static constexpr int kCBuf = NBS * kCRow;
     static constexpr int kAReg = 0;
     static constexpr int kWReg = kAReg + 2 * kABuf;
@@ -736,7 +738,7 @@ template <int NBS> struct WideLds {                 // NBS = K-blocks per stage
     // (256 + 16 bytes) puts the four row groups of one accumulator register into different banks
     static constexpr int kOutPitch = 272;
     static constexpr int kDummy = kSWReg + 2 * kCBuf;                        // gemm_wide32: 1 KiB written and never read
-    static constexpr int kBiasReg = kDummy;                                  // gemm_wide: the tile's bias, 256 x 4 bytes
+    static constexpr int kBiasReg = kDummy;                                  // gemm_wide: the tile's bias, BN x 4 bytes
     static constexpr int kStages = kDummy + 1024;                            // 135 / 141 KiB
     // gemm_wide: next to the stage buffers every wave owns a strip of 16 rows x 64 columns of 16-bit outputs, through
     // which its accumulators leave as row-major runs while the next tile's first stages are already landing in the
@@ -749,12 +751,15 @@ template <int NBS> struct WideLds {                 // NBS = K-blocks per stage
     static constexpr int kBytes = kOut > kStages ? kOut : kStages;           // of the CU's 160 KiB
 };
 
-template <int BLK, int CDT>
+// NJ = column subtiles of a wave: 8 is the 256x256 tile described above; 4 a 256x128 tile (64x64 per wave) for problems
+// that do not fill the chip with 256x256 tiles -- the same loop on half the columns, so half the MFMAs per LDS read of A.
+template <int BLK, int CDT, int NJ = 8>
 __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     static_assert(BLK == 128 || BLK == 64, "a K-block is one or two 64-byte MFMAs");
+    static_assert(NJ == 8 || NJ == 4, "64x128 or 64x64 per wave");
     constexpr int NBS = kStageK / BLK;
-    using L = WideLds<NBS>;
-    constexpr int BM = 256, BN = 256, NW = 8;
+    constexpr int BM = 256, BN = 32 * NJ, WC = 16 * NJ, NW = 8;       // WC = columns of a wave
+    using L = WideLds<NBS, BN>;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     const int tid = threadIdx.x;
@@ -774,8 +779,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     {
         int tile_m, tile_n;
         tile_of_workgroup_scalar(pid, g.tiles_m, g.tiles_n, g.band_magic, tile_m, tile_n);
-        m0 = tile_m * BM;
-        n0 = tile_n * BN;
+        m0 = (tile_m + g.tile_m0) * BM;
+        n0 = (tile_n + g.tile_n0) * BN;
     }
 
     // ---- loader (same scheme as gemm_tile): wave instruction i covers tile rows 8i .. 8i+7, lane -> row
@@ -789,23 +794,25 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     const uint32_t a_off = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_off = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
     const uint32_t a_wave = (uint32_t)(wave * 8 * g.lda), w_wave = (uint32_t)(wave * 8 * g.ldw);
     const uint32_t a_step = (uint32_t)(NW * 8 * g.lda), w_step = (uint32_t)(NW * 8 * g.ldw);
-    // scale rows of the stage's K-blocks: waves 0-3 fetch 64 row scales each, waves 4-7 64 column scales each
+    // scale rows of the stage's K-blocks: waves 0-3 fetch 64 row scales each, waves 4-7 64 column scales each (of a
+    // 128-column tile: waves 6 and 7 repeat what waves 4 and 5 do)
     const int64_t nblk = g.K / BLK;
     const bool s_is_a = wave < 4;
-    const int s_part = wave & 3;
+    const int s_part = s_is_a ? wave : (wave & 3) % (BN / 64);
     const bi8_brsrc s_brsrc = s_is_a ? bi8_make_brsrc(g.sA, nblk * g.M * 4) : bi8_make_brsrc(g.sW, nblk * g.N * 4);
     const uint32_t s_off = (uint32_t)((s_part * 64 + lane) * 4);
     const uint32_t s_inc = (uint32_t)((s_is_a ? g.M : g.N) * 4);
     // The scales come into a register of the fetching lane, which stores them to LDS just before the barrier that
     // publishes the stage.  Row scales are stored as they are.  Column scales are stored prepared, so that the
     // preparation is done once per column instead of once per wave row and lane group: lane -> tile column
-    // s_part * 64 + lane = wave column (s_part >> 1), subtile j = 4 * (s_part & 1) + lane / 16, r16 = lane % 16.
+    // s_part * 64 + lane = wave column wn, subtile j, r16 = lane % 16; pair j / 2, half j % 2 of its 16 bytes.
     // Both kinds run the same instructions (no branch: a branch in the K loop costs the register allocator its
     // footing): two 4-byte stores, the second of a row-scale lane to a slot nobody reads.
     float s_raw[NBS];
 #pragma unroll
     for (int kb = 0; kb < NBS; ++kb) s_raw[kb] = 0.0f;
-    const int c_dst = L::kSWReg + (s_part >> 1) * 1024 + (((2 * (s_part & 1) + (lane >> 5)) * 16 + (lane & 15)) * 2 + ((lane >> 4) & 1)) * 8;
+    const int c_col = s_part * 64 + lane, c_j = (c_col % WC) >> 4;
+    const int c_dst = L::kSWReg + (c_col / WC) * (WC * 8) + (((c_j >> 1) * 16 + (lane & 15)) * 2 + (c_j & 1)) * 8;
     int p_dst0 = s_is_a ? L::kSAReg + (s_part * 64 + lane) * 4 : c_dst;
     int p_dst1 = s_is_a ? L::kStrips + wave * L::kStripBytes + lane * 4 : c_dst + 4;     // the wave's strip is idle during the K loop
     const int p_buf0 = s_is_a ? L::kSBuf : L::kCBuf, p_row0 = s_is_a ? L::kSRow : L::kCRow;
@@ -821,30 +828,32 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         int tile_m, tile_n;
         // past the last tile: tile 0 once more, a stage or two loaded and never used
         tile_of_workgroup_scalar(p < ntiles ? p : 0, g.tiles_m, g.tiles_n, g.band_magic, tile_m, tile_n);
-        m0_nxt = tile_m * BM;
-        n0_nxt = tile_n * BN;
+        m0_nxt = (tile_m + g.tile_m0) * BM;
+        n0_nxt = (tile_n + g.tile_n0) * BN;
         ao_nxt = (uint32_t)(m0_nxt * g.lda);
         wo_nxt = (uint32_t)(n0_nxt * g.ldw);
         so_nxt = (uint32_t)((s_is_a ? m0_nxt : n0_nxt) * 4);
     };
-    constexpr int kLoadsPerStage = 4 + 4 + NBS;
-    // A wave's nine or ten load instructions of a stage are spread out so that the texture path never sees all of
+    constexpr int kWLoads = BN / 64;                // a wave's load instructions for the rows of W
+    constexpr int kLoadsPerStage = 4 + kWLoads + NBS;
+    // A wave's nine or ten (seven or eight) load instructions of a stage are spread out so that the texture path never sees all of
     // the workgroup's at once: the first kEarly right after the barrier that releases their buffer (last column
     // step of the stage two before), the others two per step during the first steps of the stage before.
     constexpr int kEarly = 3, kLateCols = (kLoadsPerStage - kEarly + 1) / 2;
     static_assert(kEarly <= 4, "the early loads are rows of A");
+    static_assert(kLateCols <= NJ - 1, "the late loads are issued before the last column step of the stage before");
     // The stage in buffer F gives the stage after it (buffer G) its late loads, at L, and the stage after that
     // (buffer F again) its early loads, at E.
 
     const uint32_t lds_base = bi8_lds_address(lds);
-    // load instruction idx of a stage: 0-3 = A rows, 4-7 = W rows, 8.. = scale rows; the K position advances after the last
+    // load instruction idx of a stage: 0-3 = A rows, then kWLoads of W rows, then the scale rows; the K position advances after the last
     auto issue_one = [&](int buf, int idx) {
         if (idx < 4) {
             bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + idx * NW) * 1024, a_off, idx < kEarly ? ao_E : ao_L, a_wave + idx * a_step);
-        } else if (idx < 8) {
+        } else if (idx < 4 + kWLoads) {
             bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (wave + (idx - 4) * NW) * 1024, w_off, wo_L, w_wave + (idx - 4) * w_step);
         } else if (idx < kLoadsPerStage) {
-            s_raw[idx - 8] = bi8_buffer_load_f32(s_brsrc, (int)s_off, (int)so_L);
+            s_raw[idx - 4 - kWLoads] = bi8_buffer_load_f32(s_brsrc, (int)s_off, (int)so_L);
             so_L += s_inc;
         }
     };
@@ -864,22 +873,22 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     // so the address of kb = 1 is the address of kb = 0 with bit 6 flipped.
     int a_base[2], w_base[2];
     a_base[0] = L::kAReg + (wm * 64 + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
-    w_base[0] = L::kWReg + (wn * 128 + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
+    w_base[0] = L::kWReg + (wn * WC + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
     a_base[1] = a_base[0] ^ 64;
     w_base[1] = w_base[0] ^ 64;
     // a subtile's outputs: lane -> column r16, rows 4q .. 4q+3
     int sa_base = L::kSAReg + (wm * 64 + 4 * q) * 4;
-    int sw_base = L::kSWReg + wn * 1024 + r16 * 16;
+    int sw_base = L::kSWReg + wn * (WC * 8) + r16 * 16;
     // The region offsets (64 KiB and up) stay inside these six registers: every access below is one of them plus an
     // immediate under 64 KiB.  Left to itself the compiler folds each region offset into the immediates, finds them
     // too large for the instruction's 16-bit field, and keeps a separate address register per access (24 spilled).
     asm volatile("" : "+v"(a_base[0]), "+v"(a_base[1]), "+v"(w_base[0]), "+v"(w_base[1]), "+v"(sa_base), "+v"(sw_base), "+v"(p_dst0), "+v"(p_dst1));
 
-    float acc[4][8][4];
+    float acc[4][NJ][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
 
@@ -912,6 +921,19 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             dst[r] = __builtin_fmaf(u, s[r], dst[r]);
         }
     };
+    // the same for the four elements of a partial, the four products first, so that no instruction reads the result of
+    // the one before it (measured: a dependent pair of FMAs whose sources share a register bank costs 12 % more than an
+    // independent one; 8192^3 0.535 -> 0.530 ms)
+    auto fold4 = [&](const bi8_v4i &pt, const bi8_v4f &s, int col, float *dst) {
+        const float b = bc[(col >> 1) & 1][2 * (col & 1)], cm = bc[(col >> 1) & 1][2 * (col & 1) + 1];
+        float u[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) u[r] = __builtin_fmaf(bi8_u2f((uint32_t)pt[r]), b, cm);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dst[r] = __builtin_fmaf(u[r], s[r], dst[r]);
+        __builtin_amdgcn_sched_barrier(0);
+    };
     auto wait_vm = [&](auto pending_c) {
         constexpr int kPending = decltype(pending_c)::value;
         __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
@@ -926,11 +948,11 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     auto stage = [&](auto buf_c) {                  // BLK = 128
         constexpr int F = decltype(buf_c)::value, G = 1 - F;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            constexpr int kPrevCol[8] = {7, 0, 1, 2, 3, 4, 5, 6};
+        for (int j = 0; j < NJ; ++j) {
+            constexpr int kPrevCol[8] = {NJ - 1, 0, 1, 2, 3, 4, 5, 6};
             const int jb = j & 1;
             if (j < kLateCols) issue_one(G, kEarly + 2 * j);
-            if (j < 7) {
+            if (j < NJ - 1) {
                 read_b(Bf[jb ^ 1], j + 1, F);
             } else {
                 __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -948,17 +970,14 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) cB[jb][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[i][1], Bf[jb][1], cB[jb][i], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (j == 7) {                          // every MFMA of this stage is issued: the next stage's row subtiles
+            if (j == NJ - 1) {                     // every MFMA of this stage is issued: the next stage's row subtiles
                 issue_one(F, kEarly - 1);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) read_a(A[i], i, G);
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                fold2(cB[jb ^ 1][i], 0, sx[i], kPrevCol[j], acc[i][kPrevCol[j]]);
-                fold2(cB[jb ^ 1][i], 2, sx[i], kPrevCol[j], acc[i][kPrevCol[j]]);
-            }
+            for (int i = 0; i < 4; ++i) fold4(cB[jb ^ 1][i], sx[i], kPrevCol[j], acc[i][kPrevCol[j]]);
             __builtin_amdgcn_sched_barrier(0);
             if (j == 0) {                          // this stage's row scales: first needed by the fold in column 1
 #pragma unroll
@@ -975,7 +994,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     // read one step ahead, the row scales of K-block 1 after the fold of step 8.
     bi8_v4i Bh[2];                                 // [step parity]
     auto read_bh = [&](bi8_v4i &dst, int step, int buf) {
-        const int kb = step >> 3, j = step & 7;
+        const int kb = step / NJ, j = step % NJ;
         dst = *(const bi8_v4i *)(lds + w_base[kb] + buf * L::kWBuf + j * 16 * kStageK);
         if ((j & 1) == 0) bc[(j >> 1) & 1] = *(const bi8_v4f *)(lds + sw_base + buf * L::kCBuf + kb * L::kCRow + (j >> 1) * 256);
     };
@@ -985,10 +1004,10 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     auto stage64 = [&](auto buf_c) {               // same burst schedule: four MFMAs, then the fold of the step before
         constexpr int F = decltype(buf_c)::value, G = 1 - F;
 #pragma unroll
-        for (int h = 0; h < 16; ++h) {
-            const int kb = h >> 3, hb = h & 1, jprev = (h + 15) & 7;
+        for (int h = 0; h < 2 * NJ; ++h) {
+            const int kb = h / NJ, hb = h & 1, jprev = (h + 2 * NJ - 1) % NJ;
             if (h < kLateCols) issue_one(G, kEarly + 2 * h);
-            if (h < 15) {
+            if (h < 2 * NJ - 1) {
                 read_bh(Bh[hb ^ 1], h + 1, F);
             } else {
                 __builtin_amdgcn_s_waitcnt(0xC07F);                // lgkmcnt(0) only
@@ -1004,13 +1023,13 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) cB[hb][i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[i][kb], Bh[hb], magic, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (h == 15) {                                         // every MFMA of this stage is issued
+            if (h == 2 * NJ - 1) {                                 // every MFMA of this stage is issued
                 issue_one(F, kEarly - 1);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) read_a(A[i], i, G);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            // the step before: at h = 0 the previous stage's last step, at h = 8 the last step of K-block 0, both with
+            // the step before: at h = 0 the previous stage's last step, at h = NJ the last step of K-block 0, both with
             // the row scales still in sx
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -1018,7 +1037,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
                 fold2(cB[hb ^ 1][i], 2, sx[i], jprev, acc[i][jprev]);
             }
             __builtin_amdgcn_sched_barrier(0);
-            if (h == 0 || h == 8) {                                // this K-block's row scales: first needed one step on
+            if (h == 0 || h == NJ) {                               // this K-block's row scales: first needed one step on
 #pragma unroll
                 for (int i = 0; i < 4; ++i) read_sx64(sx[i], i, kb, F);
             }
@@ -1027,12 +1046,12 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         }
     };
 
-    // 16-bit outputs: the bias of the tile's 256 columns waits in LDS for the tile's end, one dword per column (a
-    // 16-bit element zero-extended), fetched by waves 4-7, 64 columns each.  The waits and barriers of the stages
+    // 16-bit outputs: the bias of the tile's columns waits in LDS for the tile's end, one dword per column (a
+    // 16-bit element zero-extended), fetched by waves 4-7 (4-5 for 128 columns), 64 columns each.  The waits and barriers of the stages
     // that follow complete and publish it; columns past N read as zeros.
     const bi8_rsrc bias_rsrc = bi8_make_rsrc(g.bias, g.bias ? g.N * (g.bias_dtype == BI8_F32 ? 4 : 2) : 0);
     auto fetch_bias = [&]() {
-        if (wave >= 4) {
+        if (wave >= 4 && wave < 4 + BN / 64) {
             const uint32_t dst = lds_base + L::kBiasReg + (wave - 4) * 256, col = (uint32_t)(n0 + (wave - 4) * 64);
             if (g.bias_dtype == BI8_F32) bi8_buffer_to_lds4(bias_rsrc, dst, (uint32_t)(lane * 4), col * 4);
             else bi8_buffer_to_lds2(bias_rsrc, dst, (uint32_t)(lane * 2), col * 2);
@@ -1081,8 +1100,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {              // the last column of the last (possibly padding) stage
-            fold2(cB[1][i], 0, sx[i], 7, acc[i][7]);
-            fold2(cB[1][i], 2, sx[i], 7, acc[i][7]);
+            fold2(cB[1][i], 0, sx[i], NJ - 1, acc[i][NJ - 1]);
+            fold2(cB[1][i], 2, sx[i], NJ - 1, acc[i][NJ - 1]);
         }
 
         if constexpr (CDT != BI8_F32) {
@@ -1099,16 +1118,16 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             const uint8_t *strip_r = strip + (lane_e >> 3) * L::kStripPitch + (lane_e & 7) * 16;
             const int row_e = lane_e >> 3, col_e = (lane_e & 7) * 8;        // of the strip, as read back
             const int m_left = (int)(g.M - m0) - wm * 64 - row_e;             // rows 16i + 8p below this are inside C
-            const int n_e = n0 + wn * 128 + col_e;
-            uint8_t *c_tile = (uint8_t *)g.C + ((int64_t)(m0 + wm * 64) * g.ldc + n0 + wn * 128) * 2;
+            const int n_e = n0 + wn * WC + col_e;
+            uint8_t *c_tile = (uint8_t *)g.C + ((int64_t)(m0 + wm * 64) * g.ldc + n0 + wn * WC) * 2;
             const uint32_t c_lane = (uint32_t)((row_e * g.ldc + col_e) * 2);
-            const uint8_t *bias_lds = lds + L::kBiasReg + (wn * 128 + er16) * 4;
+            const uint8_t *bias_lds = lds + L::kBiasReg + (wn * WC + er16) * 4;
             auto leave = [&](auto with_bias_c) {
                 constexpr bool kBias = decltype(with_bias_c)::value;
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
 #pragma unroll
-                    for (int jh = 0; jh < 2; ++jh) {
+                    for (int jh = 0; jh < NJ / 4; ++jh) {
 #pragma unroll
                         for (int jj = 0; jj < 4; ++jj) {
                             float bias = 0.0f;
@@ -1151,8 +1170,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             else leave(std::false_type{});
         } else {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int64_t n = (int64_t)n0 + wn * 128 + j * 16 + r16;
+            for (int j = 0; j < NJ; ++j) {
+                const int64_t n = (int64_t)n0 + wn * WC + j * 16 + r16;
                 const bool n_ok = n < g.N;
                 const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
 #pragma unroll
@@ -1180,7 +1199,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             cB[1][i] = magic;
             sx[i] = bi8_v4f{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int j = 0; j < 8; ++j)
+            for (int j = 0; j < NJ; ++j)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
         }
@@ -2169,16 +2188,19 @@ int launch_tile(GemmArgs g, const Part &part, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-template <int BLK, int CDT> int launch_wide(GemmArgs g, const Part &part, hipStream_t st) {
-    using L = WideLds<kStageK / BLK>;
-    if (part.row0 != 0 || part.col0 != 0) return BI8_ERR_UNSUPPORTED;         // (the plan gives this kernel the leading part)
-    const int64_t tm = (part.rows + 255) / 256, tn = (part.cols + 255) / 256;
+template <int BLK, int CDT, int NJ = 8> int launch_wide(GemmArgs g, const Part &part, hipStream_t st) {
+    constexpr int BN = 32 * NJ;
+    using L = WideLds<kStageK / BLK, BN>;
+    if (part.row0 % 256 != 0 || part.col0 % BN != 0) return BI8_ERR_UNSUPPORTED;   // (the plan cuts at multiples of 256 only)
+    const int64_t tm = (part.rows + 255) / 256, tn = (part.cols + BN - 1) / BN;
     if (tm * tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
     g.tiles_m = (int)tm;
     g.tiles_n = (int)tn;
+    g.tile_m0 = (int)(part.row0 / 256);
+    g.tile_n0 = (int)(part.col0 / BN);
     if (!wide_addressable(g.M, g.N, g.K, g.lda, g.ldw, BLK)) return BI8_ERR_TOO_LARGE;       // the plan does not send such a problem here
     g.band_magic = (uint32_t)((1ull << 32) / (uint64_t)(kGroupM * tn));
-    auto kern = gemm_wide<BLK, CDT>;
+    auto kern = gemm_wide<BLK, CDT, NJ>;
     static LdsOptIn opted;                         // one per kernel instantiation
     const int rc = opted.ensure((const void *)kern, L::kBytesPersistent);
     if (rc != BI8_OK) return rc;
@@ -2216,10 +2238,10 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
 
 // ---- which kernel runs a problem ------------------------------------------------------------------------------------
 // One rule, used by the launcher, by bi8_gemm_workspace_bytes and by bi8_gemm_kernel_name.
-enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKTile128x192 };
+enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKWideHalf };
 static const char *const kGemmKernelNames[] = {"gemm_generic", "gemv_staged", "gemm_skinny", "gemm_wide", "gemm_tile_256x128",
                                                 "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk",
-                                                "gemm_tile_64x128_splitk", "gemv_rows", "gemm_tile_128x192"};
+                                                "gemm_tile_64x128_splitk", "gemv_rows", "gemm_wide_256x128"};
 struct GemmPlan {
     int kernel;
     int splits, split_stages;      // of the split kernels: workgroups of the split grid and 128-byte stages of K per workgroup,
@@ -2307,9 +2329,9 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                     if (rest_tiles >= best_rest) continue;
                     const int64_t rm = axis == 1 ? M - lead * 256 : M, rn = axis == 1 ? N : N - lead * 256;
                     const GemmPlan r = plan_gemm(rm, rn, K, lda, ldw, block, aligned, false, ws_bytes, true);
-                    const bool tile_family = r.kernel == kKTile256x128 || r.kernel == kKTile128x128 || r.kernel == kKTile64x128 ||
+                    const bool tile_family = r.kernel == kKTile256x128 || r.kernel == kKWideHalf || r.kernel == kKTile128x128 || r.kernel == kKTile64x128 ||
                                              r.kernel == kKSplit128x128 || r.kernel == kKSplit64x128;
-                    if (!tile_family) continue;                        // (128x192 tiles do not start at multiples of 256)
+                    if (!tile_family) continue;
                     best_rest = rest_tiles;
                     p.cut_axis = axis;
                     p.lead = lead * 256;
@@ -2328,12 +2350,12 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
     static_assert(!TileLds<256, 128, 32, 3>::kFits && TileLds<256, 128, 64, 3>::kFits, "block 32 has no 256x128 tile: its stage ring exceeds the LDS");
     if (M > 128 && t128 > 256 && block != 32) {
-        // 256x128 tiles; for block 64, 128x192 tiles where those make fewer rounds' worth of work per CU (8192 x 768: 256
-        // tiles of 128x192 against 192 of 256x128, measured 6-14 % faster; block 128 has a software-pipelined 256x128
-        // kernel, against which the 128x192 tile measured 18 % slower)
-        const int64_t t256 = ((M + 255) / 256) * ((N + 127) / 128), t192 = ((M + 127) / 128) * ((N + 191) / 192);
-        const int64_t cost256 = ((t256 + kCus - 1) / kCus) * 256 * 128, cost192 = ((t192 + kCus - 1) / kCus) * 128 * 192;
-        p.kernel = (block == 64 && cost192 < cost256 && !rest_of_cut) ? kKTile128x192 : kKTile256x128;     // (192 does not divide the cut's 256)
+        // 256x128 tiles: on gemm_wide's loop (64x64 per wave) where its 32-bit operand offsets reach, else (and for the
+        // int32 partials) on the tile kernel.  Measured, bf16 out, gemm_tile 256x128 (block 64: 128x192 tiles, since
+        // removed) -> gemm_wide<.., 4>: 2048 x 4096 x 4096 47.1 -> 44.8 us, 2048 x 4096 x 11008 111.8 -> 107.5, 1024 x 8192 x
+        // 8192 85.4 -> 81.8; block 64: 8192 x 768 x 768 15.4 -> 14.3, 8192 x 768 x 3072 39.1 -> 37.0, 2048 x 4096 x 4096
+        // 61.8 -> 54.0, 4096 x 2048 x 2048 34.8 -> 30.9; same output bits.
+        p.kernel = (!partials && wide_addressable(M, N, K, lda, ldw, block)) ? kKWideHalf : kKTile256x128;
         return p;
     }
     // small grids: one workgroup per CU at best, so the tile is spread over as many waves as its shape allows
@@ -2393,15 +2415,12 @@ int launch_kernel(const GemmArgs &g, int kernel, int splits, int split_stages, i
         if constexpr (TileLds<256, 128, BLK, kRing>::kFits)
             return launch_tile<256, 128, 4, 2, (BLK == 128 && !PARTIALS) ? 2 : kRing, BLK, CDT, PARTIALS>(g, part, st);
         break;
-    case kKTile128x192:                            // 32x96 per wave
-        if constexpr (BLK == 64) return launch_tile<128, 192, 4, 2, kRing, BLK, CDT, PARTIALS>(g, part, st);
-        break;
     case kKTile128x128: return launch_tile<128, 128, 4, 2, kRing, BLK, CDT, PARTIALS>(g, part, st);
     case kKTile64x128: return launch_tile<64, 128, 2, 2, kRing, BLK, CDT, PARTIALS>(g, part, st);
     default: break;
     }
     if constexpr (!PARTIALS) {
-        if (!whole && kernel != kKWide && kernel != kKSplit128x128 && kernel != kKSplit64x128) return BI8_ERR_UNSUPPORTED;
+        if (!whole && kernel != kKWide && kernel != kKWideHalf && kernel != kKSplit128x128 && kernel != kKSplit64x128) return BI8_ERR_UNSUPPORTED;
         switch (kernel) {
         case kKRows:
             if constexpr (BLK != 32) return launch_rows<BLK, CDT>(g, st);
@@ -2414,6 +2433,9 @@ int launch_kernel(const GemmArgs &g, int kernel, int splits, int split_stages, i
             // blocks 128 and 64: 16x16x64 MFMAs, 64x128 per wave; block 32 (one MFMA per K-block): 32x32x32, 32x256 per wave
             if constexpr (BLK == 32) return whole ? launch_wide32<BLK, CDT>(g, st) : BI8_ERR_UNSUPPORTED;
             else return launch_wide<BLK, CDT>(g, part, st);
+        case kKWideHalf:
+            if constexpr (BLK != 32) return launch_wide<BLK, CDT, 4>(g, part, st);
+            break;
         case kKSplit128x128:
         case kKSplit64x128: {
             GemmArgs gs = g;
@@ -2549,6 +2571,7 @@ extern "C" const char *bi8_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int
     if (p.cut_axis != 0) {                         // two launches: the 256x256 kernel, then the rest on smaller tiles
         switch (p.rest_kernel) {
         case kKTile256x128: return "gemm_wide+gemm_tile_256x128";
+        case kKWideHalf: return "gemm_wide+gemm_wide_256x128";
         case kKTile128x128: return "gemm_wide+gemm_tile_128x128";
         case kKTile64x128: return "gemm_wide+gemm_tile_64x128";
         case kKSplit128x128: return "gemm_wide+gemm_tile_128x128_splitk";

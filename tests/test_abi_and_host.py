@@ -232,12 +232,14 @@ def test_kernel_choice_by_shape():
     assert name(2048, 4096, 4096, 32) == "gemm_tile_128x128"         # block 32 has no 256x128 tile
     assert name(2944, 2944, 512, 128) == "gemm_wide"                 # 12 x 12 = 144 tiles of 256x256
     # a last round of 256x256 tiles that is mostly empty: whole rows (columns) of tiles cut off for a second launch
-    assert name(1536, 11008, 4096, 128) == "gemm_wide+gemm_tile_128x128" and name(2048, 11008, 4096, 128) == "gemm_wide+gemm_tile_256x128"
+    assert name(1536, 11008, 4096, 128) == "gemm_wide+gemm_tile_128x128" and name(2048, 11008, 4096, 128) == "gemm_wide+gemm_wide_256x128"
     assert name(1536, 11008, 4096, 128, 1 << 30) == "gemm_wide+gemm_tile_64x128_splitk"
     assert name(2048, 12288, 4096, 128) == "gemm_wide" and name(1280, 11008, 4096, 128) == "gemm_wide"   # half a round left / one round
-    assert name(8192, 768, 3072, 64) == "gemm_tile_128x192" and name(8192, 768, 3072, 128) == "gemm_tile_256x128"
-    assert name(2048, 4096, 4096, 128) == "gemm_tile_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
-    assert name(2048, 4096, 512, 64) == "gemm_tile_256x128" and name(2048, 2304, 512, 64) == "gemm_tile_128x192"
+    # more than 256 tiles of 128x128 that do not fill the chip with 256x256 tiles: the 256x256 kernel's loop on 256x128 tiles
+    assert name(8192, 768, 3072, 64) == "gemm_wide_256x128" and name(8192, 768, 3072, 128) == "gemm_wide_256x128"
+    assert name(2048, 4096, 4096, 128) == "gemm_wide_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
+    assert name(2048, 4096, 512, 64) == "gemm_wide_256x128" and name(2048, 2304, 512, 64) == "gemm_wide_256x128"
+    assert name(2048, 4096, 4096, 128, 0, 1 << 21, 4096) == "gemm_tile_256x128"     # rows 2 MiB apart: beyond its 32-bit offsets
     assert name(300, 500, 512, 128) == "gemm_tile_128x128" and name(48, 700, 640, 128) == "gemm_tile_64x128"
     assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
     assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 11008, 4096, 64) == "gemv_staged"

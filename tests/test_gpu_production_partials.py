@@ -56,9 +56,18 @@ def _blocks_to_check(nblk):
     return sorted(set(range(nblk)) if nblk <= 6 else {0, 1, nblk // 2, nblk - 2, nblk - 1})
 
 
-def _kernel(ops, M, N, K, block, ws):
+def _kernel(ops, M, N, K, block, ws, lda=None):
     from blockwise_int8_linear_amd import _lib
-    return _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, ws).decode()
+    return _lib.load().bi8_gemm_kernel_name(M, N, K, lda or K, K, block, ws).decode()
+
+
+def _device_codes(A, pitch):
+    """A on the device, as a view of a buffer whose rows are `pitch` codes apart"""
+    if pitch == A.shape[1]:
+        return A.to(DEV)
+    view = torch.empty((A.shape[0], pitch), device=DEV, dtype=torch.int8)[:, :A.shape[1]]
+    view.copy_(A)
+    return view
 
 
 # (M, N, K, block, kernel the shipped operator runs on it)
@@ -71,7 +80,7 @@ CASES = [
     (5200, 5100, 256, 64, "gemm_wide"),
     # 324 tiles = one full round and 68: the leading 14 rows of tiles on the 256x256 kernel, the other rows on 128x128 tiles
     (4400, 4500, 384, 128, "gemm_wide+gemm_tile_128x128"),
-    (4500, 4400, 256, 64, "gemm_wide+gemm_tile_256x128"),
+    (4500, 4400, 256, 64, "gemm_wide+gemm_wide_256x128"),          # ... on the same loop, 256x128 tiles from tile row 14 on
     (2048, 8900, 256, 128, "gemm_wide+gemm_tile_128x128"),         # cut by columns: 8 x 35 tiles, the last 3 columns of tiles apart
     (2000, 8900, 384, 64, "gemm_wide+gemm_tile_128x128"),
     (4352, 4096, 2048, 128, "gemm_wide+gemm_tile_64x128_splitk"),  # the rest (one row of 16 tiles) splits K
@@ -82,12 +91,16 @@ CASES = [
     (4300, 4096, 4096, 64, "gemm_wide+gemm_tile_128x128_splitk"),
     (2944, 2944, 256, 32, "gemm_wide"),             # block 32: the 32x32x32-MFMA form, four K-blocks per stage
     (2900, 2944, 384, 32, "gemm_wide"),
-    (2048, 2304, 512, 128, "gemm_tile_256x128"),    # the software-pipelined block-128 instantiation
-    (2000, 2304, 384, 128, "gemm_tile_256x128"),
-    (2048, 4096, 512, 64, "gemm_tile_256x128"),
-    (2048, 2304, 512, 64, "gemm_tile_128x192"),     # 192 tiles of 128x192 against 144 of 256x128
-    (8192, 768, 256, 64, "gemm_tile_128x192"),      # 256 tiles of 128x192 where 256x128 tiles would be 192
-    (8100, 760, 384, 64, "gemm_tile_128x192"),
+    (2048, 2304, 512, 128, "gemm_wide_256x128"),    # 256x128 tiles on the 256x256 kernel's loop, 64x64 per wave
+    (2000, 2304, 384, 128, "gemm_wide_256x128"),    # odd number of stages, ragged M
+    (2048, 4096, 512, 64, "gemm_wide_256x128"),
+    (2048, 2304, 512, 64, "gemm_wide_256x128"),
+    (8192, 768, 256, 64, "gemm_wide_256x128"),
+    (8100, 760, 384, 64, "gemm_wide_256x128"),      # ragged M and N
+    # rows of A 4 MiB apart put the operand beyond the 32-bit offsets of the 256x256 kernel's loop: the tile kernel's
+    # software-pipelined block-128 instantiation, and its three-buffer form at block 64 (sixth entry: row pitch of A)
+    (600, 11008, 256, 128, "gemm_tile_256x128", (1 << 22) - 128),
+    (600, 11008, 256, 64, "gemm_tile_256x128", (1 << 22) - 128),
     (300, 500, 512, 128, "gemm_tile_128x128"),
     (300, 500, 512, 32, "gemm_tile_128x128"),
     (2304, 2304, 256, 32, "gemm_tile_128x128"),
@@ -118,15 +131,16 @@ CASES = [
 @pytest.mark.parametrize("out", ["f32", "bf16"])
 def test_partials_of_the_shipping_kernels(ops, case, out):
     from blockwise_int8_linear_amd import _lib
-    M, N, K, block, kernel = case
+    M, N, K, block, kernel = case[:5]
+    lda = case[5] if len(case) > 5 else K
     ws = _lib.load().bi8_gemm_workspace_bytes(M, N, K, block)          # what the operator asks for and passes
-    assert _kernel(ops, M, N, K, block, ws) == kernel
+    assert _kernel(ops, M, N, K, block, ws, lda) == kernel
     g = torch.Generator().manual_seed(M + 3 * N + K + block)
     full = out == "f32"
     A, W = _codes(g, M, K, full), _codes(g, N, K, full)
     nblk = K // block
     P_ref = oracle_torch.gemm_nt_partials(A, W, block)                  # int32 [nblk, M, N]
-    Ad, Wd = A.to(DEV), W.to(DEV)
+    Ad, Wd = _device_codes(A, lda), W.to(DEV)
     sw = torch.ones(nblk, N, device=DEV)
     with cfg_as(ops, block, DT[out]):
         for j in _blocks_to_check(nblk):
@@ -154,7 +168,7 @@ def test_partials_of_the_shipping_kernels(ops, case, out):
 
 @pytest.mark.parametrize("case", CASES[:2] + CASES[4:7], ids=lambda c: "x".join(map(str, c[:4])) + "-" + c[4])
 def test_partials_of_the_f16_instantiations(ops, case):
-    M, N, K, block, kernel = case
+    M, N, K, block, kernel = case[:5]
     g = torch.Generator().manual_seed(K + block)
     A, W = _codes(g, M, K, False), _codes(g, N, K, False)
     nblk = K // block
