@@ -29,8 +29,8 @@ from .ops import (
     _int8_matmul,
     _quantize_block_dual,
     dequantize_block_rowwise,
+    few_rows_plan,
     int8_matmul_block64_rowwise_dequantize,
-    linear_few_rows,
     quantize_block_dual,
     quantize_block_rowwise,
     quantize_block_transposed,
@@ -211,6 +211,7 @@ class BlockInt8Linear(nn.Linear):
         self._train_cache = None
         self._eval_cache_of = None                 # state of the weight the eval cache was quantized from
         self._invalidations = 0
+        self._few_rows = None                      # (key, closure) of the one-launch decode path
 
     def _weight_state(self):
         """Changes whenever the weight's values may have: in-place updates through the parameter bump its version,
@@ -246,17 +247,28 @@ class BlockInt8Linear(nn.Linear):
     def infer(self, x):
         # quantize the weight on first use (block_linear.py:138-139) and again when it has changed since: the reference
         # keeps serving the first cache
-        if getattr(self, "W_int8", None) is None or self._eval_cache_of != self._weight_state():
+        bufs = self._buffers                       # (read directly: Module.__getattr__ costs as much as a tensor op)
+        if bufs.get("W_int8") is None or self._eval_cache_of != self._weight_state():
             self.prepare_for_eval()
+        W_int8, state_W, bias = bufs["W_int8"], bufs["state_W"], self._parameters.get("bias")
         X = x.reshape(-1, x.size(-1))
         out = None
         if X.shape[0] <= 2:
             # token-by-token decode: quantize and multiply in one kernel.  Every workgroup of that kernel quantizes x
-            # for itself, which pays off for one or two rows (measured; from four rows on the two launches are as fast)
-            out = linear_few_rows(X, self.W_int8, self.state_W, self.bias)
+            # for itself, which pays off for one or two rows (measured; from four rows on the two launches are as fast).
+            # What does not change from token to token (shapes, pointers of the cached weights, the configuration) is
+            # checked once and kept in a closure: the Python side of a decode step is most of its cost.
+            # (the closure holds the tensors it was made for, so their ids stay theirs)
+            key = (X.shape, X.dtype, block_linear_config.GROUP_SIZE, block_linear_config.INPUT_OUTPUT_TORCH_TYPE,
+                   id(W_int8), id(state_W), id(bias))
+            plan = self._few_rows
+            if plan is None or plan[0] != key:
+                plan = self._few_rows = (key, few_rows_plan(X, W_int8, state_W, bias))
+            if plan[1] is not None:
+                out = plan[1](X)
         if out is None:
             X_int8, state_X = quantize_block_rowwise(X)
-            out = int8_matmul_block64_rowwise_dequantize(X_int8, self.W_int8.t(), state_X, self.state_W, self.bias)
+            out = int8_matmul_block64_rowwise_dequantize(X_int8, W_int8.t(), state_X, state_W, bias)
         return out.view(*x.size()[:-1], -1)
 
     def forward(self, x):

@@ -753,10 +753,15 @@ template <int NBS, int BN = 256> struct WideLds {   // NBS = K-blocks per stage,
 
 // NJ = column subtiles of a wave: 8 is the 256x256 tile described above; 4 a 256x128 tile (64x64 per wave) for problems
 // that do not fill the chip with 256x256 tiles -- the same loop on half the columns, so half the MFMAs per LDS read of A.
-template <int BLK, int CDT, int NJ = 8>
+// SPLIT: the contraction is split over gridDim.y workgroups per tile (GemmArgs::split_stages stages of K each, an even
+// number, so that the padding stage of an odd trip count exists only at the end of K, where the scales read as zeros);
+// workgroup (t, y) writes the fp32 sums of its piece, scaled, without bias, to slab (row-major tile index) * gridDim.y + y
+// of the workspace, and splitk_reduce adds a tile's slabs.  One piece per workgroup: the grid is not persistent.
+template <int BLK, int CDT, int NJ = 8, bool SPLIT = false>
 __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     static_assert(BLK == 128 || BLK == 64, "a K-block is one or two 64-byte MFMAs");
     static_assert(NJ == 8 || NJ == 4, "64x128 or 64x64 per wave");
+    static_assert(!SPLIT || CDT == BI8_F32, "the slabs are fp32 sums");
     constexpr int NBS = kStageK / BLK;
     constexpr int BM = 256, BN = 32 * NJ, WC = 16 * NJ, NW = 8;       // WC = columns of a wave
     using L = WideLds<NBS, BN>;
@@ -772,15 +777,18 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     // stage pipeline runs on across tile boundaries: while a tile's last two stages are computed the loader already
     // fetches the first two stages of the workgroup's next tile, and they land while the accumulators leave.
     const int ntiles = g.tiles_m * g.tiles_n;
-    const int nstages = (int)(g.K / kStageK);
+    const int stage_lo = SPLIT ? (int)blockIdx.y * g.split_stages : 0;          // this workgroup's first stage of K
+    const int nstages = SPLIT ? ((int)(g.K / kStageK) - stage_lo < g.split_stages ? (int)(g.K / kStageK) - stage_lo : g.split_stages)
+                              : (int)(g.K / kStageK);
     const int npairs = (nstages + 1) >> 1;         // the trip count is rounded up to even (see below)
     int pid = blockIdx.x;                          // the tile being computed
-    int m0, n0;
+    int m0, n0, slab = 0;
     {
         int tile_m, tile_n;
         tile_of_workgroup_scalar(pid, g.tiles_m, g.tiles_n, g.band_magic, tile_m, tile_n);
         m0 = (tile_m + g.tile_m0) * BM;
         n0 = (tile_n + g.tile_n0) * BN;
+        if constexpr (SPLIT) slab = (tile_m * g.tiles_n + tile_n) * (int)gridDim.y + (int)blockIdx.y;
     }
 
     // ---- loader (same scheme as gemm_tile): wave instruction i covers tile rows 8i .. 8i+7, lane -> row
@@ -820,8 +828,8 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     // The loader walks the stream of stages (this tile's, then the next tile's) at two positions one stage apart:
     // E, where a stage gets its first kEarly loads (rows of A), and L, where it gets the others.  A position is the
     // byte offset of (tile, K position) in each operand; all of them are wave-uniform.
-    uint32_t ao_E = (uint32_t)(m0 * g.lda), ao_L = ao_E, wo_L = (uint32_t)(n0 * g.ldw);
-    uint32_t so_L = (uint32_t)((s_is_a ? m0 : n0) * 4);
+    uint32_t ao_E = (uint32_t)(m0 * g.lda + stage_lo * kStageK), ao_L = ao_E, wo_L = (uint32_t)(n0 * g.ldw + stage_lo * kStageK);
+    uint32_t so_L = (uint32_t)((s_is_a ? m0 : n0) * 4) + (uint32_t)(stage_lo * NBS) * s_inc;
     uint32_t ao_nxt = 0, wo_nxt = 0, so_nxt = 0;   // the workgroup's next tile
     int m0_nxt = 0, n0_nxt = 0;
     auto aim_next = [&](int p) {
@@ -923,7 +931,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
     };
     // the same for the four elements of a partial, the four products first, so that no instruction reads the result of
     // the one before it (measured: a dependent pair of FMAs whose sources share a register bank costs 12 % more than an
-    // independent one; 8192^3 0.535 -> 0.530 ms)
+    // independent one; 8192^3 0.535 -> 0.530 ms, at block 64 0.692 -> 0.680)
     auto fold4 = [&](const bi8_v4i &pt, const bi8_v4f &s, int col, float *dst) {
         const float b = bc[(col >> 1) & 1][2 * (col & 1)], cm = bc[(col >> 1) & 1][2 * (col & 1) + 1];
         float u[4];
@@ -1032,10 +1040,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             // the step before: at h = 0 the previous stage's last step, at h = NJ the last step of K-block 0, both with
             // the row scales still in sx
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                fold2(cB[hb ^ 1][i], 0, sx[i], jprev, acc[i][jprev]);
-                fold2(cB[hb ^ 1][i], 2, sx[i], jprev, acc[i][jprev]);
-            }
+            for (int i = 0; i < 4; ++i) fold4(cB[hb ^ 1][i], sx[i], jprev, acc[i][jprev]);
             __builtin_amdgcn_sched_barrier(0);
             if (h == 0 || h == NJ) {                               // this K-block's row scales: first needed one step on
 #pragma unroll
@@ -1168,6 +1173,15 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
             };
             if (has_bias) leave(std::true_type{});
             else leave(std::false_type{});
+        } else if constexpr (SPLIT) {
+            // the piece's sums, scaled, to its slab [256][BN]: the whole tile (rows and columns past the matrix hold zeros)
+            float *out = g.ws + (int64_t)slab * (BM * BN) + (wm * 64 + 4 * q) * BN + wn * WC + r16;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) out[(i * 16 + r) * BN + j * 16] = acc[i][j][r] * div;
         } else {
 #pragma unroll
             for (int j = 0; j < NJ; ++j) {
@@ -1185,7 +1199,7 @@ __global__ __launch_bounds__(512) void gemm_wide(const GemmArgs g) {
         }
 
         pid += (int)gridDim.x;
-        if (pid >= ntiles) break;
+        if (SPLIT || pid >= ntiles) break;
         // The next tile: its first stage is published, its operands of column 0 are in A and Bf[0].  The first step
         // folds "the column before" from an empty partial with zero scales, as at the start of the kernel.
         m0 = m0_nxt;
@@ -1591,8 +1605,8 @@ __global__ __launch_bounds__(512) void gemm_skinny(const GemmArgs g) {
 // layout through an 8-stage register ring: 4096 -> 11008 16.0 -> 12.8 us, 11008 -> 4096 17.1 -> 14.4 us.
 constexpr int kLdsGemvSlotsW = 4, kLdsGemvSlotsA = 2;
 constexpr int kLdsGemvSlot = 16 * 128;             // bytes of one stage of W, or of 16 rows of A
-// MT = groups of 16 rows of A (1: M <= 16, 2: M <= 32).  One stage's scales: [K-block][16] column scales (128 bytes), then
-// [K-block][16 * MT] row scales.
+// MT = groups of 16 rows of A (1, 2 or 4: M <= 16, 32, 64).  One stage's scales: [K-block][16] column scales (128 bytes),
+// then [K-block][16 * MT] row scales.
 template <int MT> struct GemvLds {
     static constexpr int kAStage = MT * kLdsGemvSlot;
     static constexpr int kScales = 128 + 128 * MT;
@@ -1609,7 +1623,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
     constexpr int kSlot = kLdsGemvSlot;
     static_assert(BLK == 64 || BLK == 128, "one or two 64-byte MFMAs per K-block");
     static_assert(NSW == 4 && NSA == 2, "the K loop is unrolled over the period of both rings");
-    static_assert(MT == 1 || MT == 2, "16 or 32 rows of A");
+    static_assert(MT == 1 || MT == 2 || MT == 4, "16 to 64 rows of A");
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -1630,21 +1644,29 @@ __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
     const bi8_rsrc ra = bi8_make_rsrc(g.A, (g.M - 1) * g.lda + g.K);
     const bi8_rsrc rsw = bi8_make_rsrc(g.sW, (int64_t)nblk * g.N * 4);
     const bi8_rsrc rsa = bi8_make_rsrc(g.sA, (int64_t)nblk * g.M * 4);
-    // scales of a stage: column scales lane -> K-block lane / 16 of the stage's BPS, column lane % 16; row scales lane ->
-    // K-block lane / (16 MT), row lane % (16 MT); rows past M read as zeros
+    // scales of a stage: column scales lane -> K-block lane / 16 of the stage's BPS, column lane % 16; row scales: element
+    // e = 64 u + lane of load instruction u -> K-block e / (16 MT), row e % (16 MT); rows past M read as zeros
     constexpr int kRowsA = 16 * MT;
+    constexpr int kSaLoads = (kRowsA * BPS + 63) / 64;        // load instructions for a stage's row scales
     const uint32_t vsw = (uint32_t)((q * (int)g.N + (int)(n < g.N ? n : g.N - 1)) * 4);
-    const uint32_t vsa = lane % kRowsA < g.M ? (uint32_t)(((lane / kRowsA) * (int)g.M + lane % kRowsA) * 4) : (uint32_t)kBufOut;
+    uint32_t vsa[kSaLoads];
+#pragma unroll
+    for (int u = 0; u < kSaLoads; ++u) {
+        const int e = 64 * u + lane;
+        vsa[u] = e % kRowsA < g.M ? (uint32_t)(((e / kRowsA) * (int)g.M + e % kRowsA) * 4) : (uint32_t)kBufOut;
+    }
 
     // ---- loader: instruction i of a stage covers rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which
     // holds source chunk (lane%8) ^ ((row >> 1) & 7) = (lane%8) ^ (lane/16) ^ 4(i & 1)
     const int ld_row = lane >> 3;
     const int ld_chunk = (lane & 7) ^ ((lane >> 4) & 3);
-    uint32_t vw[2], va[2 * MT];
+    // (of A, instruction i = 2 t + p: the 16 rows of group t go into the scalar offset, so two registers serve all groups)
+    uint32_t vw[2], va[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) vw[i] = (uint32_t)((8 * i + ld_row) * (int)g.ldw + 16 * (ld_chunk ^ (4 * i)));
 #pragma unroll
-    for (int i = 0; i < 2 * MT; ++i) va[i] = (uint32_t)((8 * i + ld_row) * (int)g.lda + 16 * (ld_chunk ^ (4 * (i & 1))));
+    for (int i = 0; i < 2; ++i) va[i] = (uint32_t)((8 * i + ld_row) * (int)g.lda + 16 * (ld_chunk ^ (4 * i)));
+    const uint32_t a_group = (uint32_t)(16 * (int)g.lda);
     auto issue_w = [&](int s, int slot) {          // s, slot: wave-uniform; four load instructions
         const int c = s * NW + wave;
         const bool live = c < nchunks;
@@ -1653,14 +1675,17 @@ __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
         for (int i = 0; i < 2; ++i) bi8_buffer_to_lds16(rw, mine_addr + slot * kSlot + i * 1024, vw[i], k0);
         if (lane < 16 * BPS)                       // (the loads write LDS for the active lanes only)
             bi8_buffer_to_lds4(rsw, mine_addr + kScReg + slot * L::kScales, vsw, live ? (uint32_t)(c * BPS * (int)g.N * 4) : (uint32_t)kBufOut);
-        if (lane < kRowsA * BPS)
-            bi8_buffer_to_lds4(rsa, mine_addr + kScReg + slot * L::kScales + 128, vsa, live ? (uint32_t)(c * BPS * (int)g.M * 4) : (uint32_t)kBufOut);
+#pragma unroll
+        for (int u = 0; u < kSaLoads; ++u)
+            if (64 * u + lane < kRowsA * BPS)
+                bi8_buffer_to_lds4(rsa, mine_addr + kScReg + slot * L::kScales + 128 + u * 256, vsa[u], live ? (uint32_t)(c * BPS * (int)g.M * 4) : (uint32_t)kBufOut);
     };
     auto issue_a = [&](int s, int slot) {          // 2 MT load instructions
         const int c = s * NW + wave;
         const uint32_t k0 = c < nchunks ? (uint32_t)(c * KW) : (uint32_t)kBufOut;
+        // (a dead stage's offset stays past the end of the buffer with the rows of a group added: below 2^31, see the plan)
 #pragma unroll
-        for (int i = 0; i < 2 * MT; ++i) bi8_buffer_to_lds16(ra, mine_addr + kAReg + slot * L::kAStage + i * 1024, va[i], k0);
+        for (int i = 0; i < 2 * MT; ++i) bi8_buffer_to_lds16(ra, mine_addr + kAReg + slot * L::kAStage + i * 1024, va[i & 1], k0 + (i >> 1) * a_group);
     };
     // operand fragments: lane -> row r16 (of W, or of a group of 16 rows of A), chunk 4j + q of the stage's eight, stored
     // at (4j + q) ^ ((r16 >> 1) & 7)
@@ -1687,8 +1712,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_staged(const GemmArgs g) {
         issue_a(s + 1, SA ^ 1);
         issue_w(s + NSW - 1, (SW + NSW - 1) % NSW);
         // everything up to A(s) has landed when only W(s + 3), A(s + 1) and W(s + 2) are outstanding
-        constexpr int kPending = 8 + 2 * MT;
-        __builtin_amdgcn_s_waitcnt(0x0F70 | kPending);
+        constexpr int kPending = 2 * (3 + kSaLoads) + 2 * MT;
+        static_assert(kPending < 64, "vmcnt is a 6-bit field");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
         const bi8_v4i zero = {0, 0, 0, 0};
         bi8_v4i wf[2], af[MT][2];
 #pragma unroll
@@ -2088,6 +2114,14 @@ __global__ __launch_bounds__(256) void splitk_reduce(const GemmArgs g) {
 // 84.8 -> 70.6; runs in place of the equal split of few tiles cost 10-25 %).
 constexpr int64_t kCus = 256;                  // compute units the plan counts rounds of workgroups against (MI355X)
 constexpr int kSplitMinStages = 8, kRunMinSaved = 28;
+// The split of 256x128 tiles on gemm_wide's loop pays where pieces are long and the tiles few: every piece writes and the
+// second kernel reads a slab of 128 KiB.  Measured against the split (or unsplit) 128x128 tiles, bf16 out: block 64, K = 8192
+// (the GPT-2 grad-weight GEMMs), 3072 x 768 (3 pieces of 22 stages per tile) 50.2 -> 43.5 us, 768 x 3072 49.2 -> 42.8, 2304 x
+// 768 (4 x 16) 40.3 -> 35.1; block 128: 1024 x 2048 x 8192 (4 x 16) 34.9 -> 34.2, but 512 x 4096 x 4096 (4 x 8) 23.5 -> 24.9,
+// 256 x 4096 x 11008 (8 x 12) 27.3 -> 29.2, 1024 x 4096 x 4096 (2 x 16, 256 slabs) 28.0 -> 34.7, 256 x 11008 x 4096 25.9 -> 30.5.
+constexpr int64_t kWideSplitMinGroups = 160;   // workgroups that the split 256x128 tiles have to put to work,
+constexpr int64_t kWideSplitMinStages = 16;    // ... the least stages of K per piece
+constexpr int64_t kWideSplitMinPer = 3;        // ... and pieces per tile
 struct SplitGrid {
     int groups, stages, per_tile;                  // workgroups, stages of K per workgroup, workgroups per tile (0: runs); groups <= 1: no split
 };
@@ -2188,7 +2222,7 @@ int launch_tile(GemmArgs g, const Part &part, hipStream_t st) {
     return bi8_launch_rc();
 }
 
-template <int BLK, int CDT, int NJ = 8> int launch_wide(GemmArgs g, const Part &part, hipStream_t st) {
+template <int BLK, int CDT, int NJ = 8, bool SPLIT = false> int launch_wide(GemmArgs g, const Part &part, hipStream_t st) {
     constexpr int BN = 32 * NJ;
     using L = WideLds<kStageK / BLK, BN>;
     if (part.row0 % 256 != 0 || part.col0 % BN != 0) return BI8_ERR_UNSUPPORTED;   // (the plan cuts at multiples of 256 only)
@@ -2200,10 +2234,15 @@ template <int BLK, int CDT, int NJ = 8> int launch_wide(GemmArgs g, const Part &
     g.tile_n0 = (int)(part.col0 / BN);
     if (!wide_addressable(g.M, g.N, g.K, g.lda, g.ldw, BLK)) return BI8_ERR_TOO_LARGE;       // the plan does not send such a problem here
     g.band_magic = (uint32_t)((1ull << 32) / (uint64_t)(kGroupM * tn));
-    auto kern = gemm_wide<BLK, CDT, NJ>;
+    auto kern = gemm_wide<BLK, CDT, NJ, SPLIT>;
     static LdsOptIn opted;                         // one per kernel instantiation
     const int rc = opted.ensure((const void *)kern, L::kBytesPersistent);
     if (rc != BI8_OK) return rc;
+    if constexpr (SPLIT) {                         // one piece per workgroup: split_per_tile pieces of every tile
+        if (g.split_per_tile < 2 || g.split_stages < 2 || g.split_stages % 2 != 0 || tm * tn * g.split_per_tile > kCus) return BI8_ERR_UNSUPPORTED;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(tm * tn), (unsigned)g.split_per_tile), dim3(512), L::kBytesPersistent, st, g);
+        return bi8_launch_rc();
+    }
     int cus = 0;
     const int rc_cus = compute_units(&cus);
     if (rc_cus != BI8_OK) return rc_cus;
@@ -2238,10 +2277,10 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
 
 // ---- which kernel runs a problem ------------------------------------------------------------------------------------
 // One rule, used by the launcher, by bi8_gemm_workspace_bytes and by bi8_gemm_kernel_name.
-enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKWideHalf };
+enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKWideHalf, kKSplitWideHalf };
 static const char *const kGemmKernelNames[] = {"gemm_generic", "gemv_staged", "gemm_skinny", "gemm_wide", "gemm_tile_256x128",
                                                 "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk",
-                                                "gemm_tile_64x128_splitk", "gemv_rows", "gemm_wide_256x128"};
+                                                "gemm_tile_64x128_splitk", "gemv_rows", "gemm_wide_256x128", "gemm_wide_256x128_splitk"};
 struct GemmPlan {
     int kernel;
     int splits, split_stages;      // of the split kernels: workgroups of the split grid and 128-byte stages of K per workgroup,
@@ -2258,7 +2297,13 @@ struct GemmPlan {
 // mostly empty round and the 256x256 kernel wins (1284 against 978 TOP/s at 2304x4096x4096, 144 tiles).
 // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
 constexpr int64_t kWideMinTiles = 129;
-constexpr int64_t kStagedMaxRows = 32;         // gemv_staged: one or two groups of 16 rows
+constexpr int64_t kStagedMaxRows = 32;         // gemv_staged: one or two groups of 16 rows whatever the shape ...
+// ... and up to four where one round of workgroups covers the columns and a workgroup's pass over all of A stays short: every
+// workgroup streams the whole of A through its LDS, which a split of K divides.  Measured against the split 64x128 tiles,
+// W from HBM, block 128, 48 / 64 rows: 4096 -> 4096 12.8 -> 9.6 / 13.3 -> 10.3 us, but 4096 -> 11008 (2.7 rounds) 17.4 -> 23.8 /
+// 17.9 -> 26.0 and 11008 -> 4096 16.7 -> 19.8 / 17.2 -> 21.8; eight groups (128 rows, three waves) lose everywhere (4096 -> 4096
+// 14.7 -> 17.0, 4096 -> 11008 21.9 -> 45.3).
+constexpr int64_t kStagedWideRows = 64, kStagedWideMaxGroups = 288, kStagedWideMaxCodes = 320 * 1024;
 // `aligned`: A and W 16-byte aligned, the scales 4-byte aligned (the partials entry point has no scales);
 // ws_bytes: scratch memory the split kernels may use (0: none).
 // A last round of 256x256 tiles that is mostly empty costs as much as a full one (1280 x 11008 x 4096: 215 tiles, 69 us;
@@ -2280,6 +2325,27 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     // few tiles and scratch memory: split K over the workgroups, then sum the slabs
     auto try_split = [&]() {
         if (partials || ws_bytes <= 0) return false;
+        // 256x128 tiles on gemm_wide's loop, split evenly, where that puts most of the CUs to work
+        if (block != 32 && M > 128 && wide_addressable(M, N, K, lda, ldw, block)) {
+            const int64_t t = ((M + 255) / 256) * ((N + 127) / 128), nst = K / kStageK;
+            int64_t per = t > 0 && t <= kCus / 2 ? kCus / t : 0;
+            if (per > kSplitMax) per = kSplitMax;
+            if (per > nst / kSplitMinStages) per = nst / kSplitMinStages;
+            if (per >= 2) {
+                int64_t stages = (nst + per - 1) / per;
+                stages += stages & 1;              // even: a piece's padding stage (odd trip count) only at the end of K
+                per = (nst + stages - 1) / stages;
+                const int64_t need = t * per * 256 * 128 * 4;
+                if (per >= kWideSplitMinPer && stages >= kWideSplitMinStages && t * per >= kWideSplitMinGroups && need <= ws_bytes) {
+                    p.kernel = kKSplitWideHalf;
+                    p.splits = (int)(t * per);
+                    p.split_stages = (int)stages;
+                    p.split_per_tile = (int)per;
+                    p.ws_need = need;
+                    return true;
+                }
+            }
+        }
         int kind;
         const SplitGrid sg = plan_split(M, N, K, kind);
         if (sg.groups <= 1) return false;
@@ -2302,8 +2368,9 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             p.kernel = kKRows;
             return p;
         }
-        if (M <= kStagedMaxRows && (block == 64 || block == 128) && (K / block + 16) * N * 4 < 0x3fffffffLL && 16 * ldw + K < 0x3fffffffLL &&
-            32 * lda + K < 0x3fffffffLL && (K / block + 16) * M * 4 < 0x3fffffffLL) {         // (gemv_staged addresses its buffers with 32-bit offsets)
+        const bool staged_rows = M <= kStagedMaxRows || (M <= kStagedWideRows && (N + 15) / 16 <= kStagedWideMaxGroups && M * K <= kStagedWideMaxCodes);
+        if (staged_rows && (block == 64 || block == 128) && (K / block + 16) * N * 4 < 0x3fffffffLL && 16 * ldw + K < 0x3fffffffLL &&
+            128 * lda + K < 0x3fffffffLL && (K / block + 16) * M * 4 < 0x3fffffffLL) {         // (gemv_staged addresses its buffers with 32-bit offsets)
             p.kernel = kKGemv;
             return p;
         }
@@ -2329,7 +2396,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                     if (rest_tiles >= best_rest) continue;
                     const int64_t rm = axis == 1 ? M - lead * 256 : M, rn = axis == 1 ? N : N - lead * 256;
                     const GemmPlan r = plan_gemm(rm, rn, K, lda, ldw, block, aligned, false, ws_bytes, true);
-                    const bool tile_family = r.kernel == kKTile256x128 || r.kernel == kKWideHalf || r.kernel == kKTile128x128 || r.kernel == kKTile64x128 ||
+                    const bool tile_family = r.kernel == kKTile256x128 || r.kernel == kKWideHalf || r.kernel == kKSplitWideHalf || r.kernel == kKTile128x128 || r.kernel == kKTile64x128 ||
                                              r.kernel == kKSplit128x128 || r.kernel == kKSplit64x128;
                     if (!tile_family) continue;
                     best_rest = rest_tiles;
@@ -2390,7 +2457,10 @@ template <int BLK, int CDT> int launch_staged(const GemmArgs &g, hipStream_t st)
     // eight waves per workgroup where four would leave CUs with a single workgroup's loads in flight; up to 16 rows three
     // workgroups of four waves share a CU, up to 32 rows (twice the A ring) two
     if (g.M <= 16) return tn <= 384 ? launch_staged_as<BLK, CDT, 8, 1>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 1>(g, (unsigned)tn, st);
-    return tn <= 384 ? launch_staged_as<BLK, CDT, 8, 2>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 2>(g, (unsigned)tn, st);
+    if (g.M <= 32) return tn <= 384 ? launch_staged_as<BLK, CDT, 8, 2>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 2>(g, (unsigned)tn, st);
+    // up to 64 rows the rings of A leave room for four waves, one workgroup per CU (the plan asks for no more rows)
+    if (g.M <= 64) return launch_staged_as<BLK, CDT, 4, 4>(g, (unsigned)tn, st);
+    return BI8_ERR_UNSUPPORTED;
 }
 
 template <int BLK, int CDT> int launch_rows(const GemmArgs &g, hipStream_t st) {
@@ -2420,7 +2490,8 @@ int launch_kernel(const GemmArgs &g, int kernel, int splits, int split_stages, i
     default: break;
     }
     if constexpr (!PARTIALS) {
-        if (!whole && kernel != kKWide && kernel != kKWideHalf && kernel != kKSplit128x128 && kernel != kKSplit64x128) return BI8_ERR_UNSUPPORTED;
+        if (!whole && kernel != kKWide && kernel != kKWideHalf && kernel != kKSplitWideHalf && kernel != kKSplit128x128 && kernel != kKSplit64x128)
+            return BI8_ERR_UNSUPPORTED;
         switch (kernel) {
         case kKRows:
             if constexpr (BLK != 32) return launch_rows<BLK, CDT>(g, st);
@@ -2435,6 +2506,22 @@ int launch_kernel(const GemmArgs &g, int kernel, int splits, int split_stages, i
             else return launch_wide<BLK, CDT>(g, part, st);
         case kKWideHalf:
             if constexpr (BLK != 32) return launch_wide<BLK, CDT, 4>(g, part, st);
+            break;
+        case kKSplitWideHalf:
+            if constexpr (BLK != 32) {
+                GemmArgs gs = g;
+                gs.splits = splits;
+                gs.split_stages = split_stages;
+                gs.split_per_tile = split_per_tile;
+                const int rc = launch_wide<BLK, BI8_F32, 4, true>(gs, part, st);
+                if (rc != BI8_OK) return rc;
+                gs.tiles_m = (int)((part.rows + 255) / 256);
+                gs.tiles_n = (int)((part.cols + 127) / 128);
+                gs.tile_m0 = (int)(part.row0 / 256);
+                gs.tile_n0 = (int)(part.col0 / 128);
+                hipLaunchKernelGGL((splitk_reduce<CDT, 256, 128>), dim3((unsigned)(gs.tiles_m * gs.tiles_n), 32), dim3(256), 0, st, gs);
+                return bi8_launch_rc();
+            }
             break;
         case kKSplit128x128:
         case kKSplit64x128: {
@@ -2572,6 +2659,7 @@ extern "C" const char *bi8_gemm_kernel_name(int64_t M, int64_t N, int64_t K, int
         switch (p.rest_kernel) {
         case kKTile256x128: return "gemm_wide+gemm_tile_256x128";
         case kKWideHalf: return "gemm_wide+gemm_wide_256x128";
+        case kKSplitWideHalf: return "gemm_wide+gemm_wide_256x128_splitk";
         case kKTile128x128: return "gemm_wide+gemm_tile_128x128";
         case kKTile64x128: return "gemm_wide+gemm_tile_64x128";
         case kKSplit128x128: return "gemm_wide+gemm_tile_128x128_splitk";

@@ -254,17 +254,44 @@ def _int8_matmul(a, b, state_x, state_w, bias=None, a_store=None, w_store=None):
         bias = bias.contiguous()
         bias_ptr, bias_dt = bias.data_ptr(), _DT[bias.dtype]
     lib = _lib.load()
-    # fewer output tiles than compute units: the library splits K over the workgroups if it is given scratch memory
-    # (up to 32 rows at blocks 64 / 128 run the one-pass decode kernels whatever they are given: not asked)
-    ws_bytes = lib.bi8_gemm_workspace_bytes(M, N, K, block) if M > 32 or block == 32 else 0
-    ws = torch.empty(ws_bytes, device=a.device, dtype=torch.uint8) if ws_bytes else None
+    stream = _stream(a)
+    ws, ws_bytes = _workspace(lib, M, N, K, block, a.device, stream)
     with _on_device(a):
         rc = lib.bi8_gemm_nt_dequant_ws(a.data_ptr(), w.data_ptr(), state_x.data_ptr(), state_w.data_ptr(),
                                         bias_ptr, bias_dt, c.data_ptr(), _DT[out_dtype], M, N, K,
                                         _ld(a), _ld(w), max(N, 1), block, ws.data_ptr() if ws is not None else None, ws_bytes,
-                                        _stream(a))
+                                        stream)
     _lib.check(rc, "bi8_gemm_nt_dequant_ws")
     return c
+
+
+_ws_need = {}                       # (M, N, K, block) -> bytes of scratch memory the library's split of K wants (0: none)
+_ws_held = {}                       # (device index, stream) -> uint8 tensor, grown on demand
+
+
+def _workspace(lib, M, N, K, block, device, stream):
+    """Scratch memory for a GEMM of fewer output tiles than compute units (the library then splits K over the
+    workgroups and sums the pieces): (tensor or None, bytes).  What a shape wants is asked once; the memory is one
+    tensor per device and stream, kept for the life of the process (at most 32 MiB each) and shared by the GEMMs of
+    that stream, which run one after the other.  While the stream is being captured into a graph the memory comes from
+    the capture's own pool instead, so that graphs replayed side by side do not share it.
+    (Up to 32 rows at blocks 64 / 128 run the one-pass decode kernels whatever they are given: not asked.)"""
+    if M <= 32 and block != 32:
+        return None, 0
+    key = (M, N, K, block)
+    need = _ws_need.get(key)
+    if need is None:
+        need = _ws_need[key] = lib.bi8_gemm_workspace_bytes(M, N, K, block)
+    if not need:
+        return None, 0
+    if torch.cuda.is_current_stream_capturing():
+        return torch.empty(need, device=device, dtype=torch.uint8), need
+    held = _ws_held.get((device.index, stream))
+    if held is None or held.numel() < need:
+        # (allocated on the current stream, which is `stream`: torch's allocator orders a later reuse of a replaced
+        # tensor's memory behind the work already queued there)
+        held = _ws_held[(device.index, stream)] = torch.empty(need, device=device, dtype=torch.uint8)
+    return held, need
 
 
 _FEW_ROWS = 2
@@ -310,6 +337,46 @@ def linear_few_rows(x, W_int8, state_W, bias=None):
         return None
     _lib.check(rc, "bi8_linear_few_rows")
     return c
+
+
+def few_rows_plan(x, W_int8, state_W, bias):
+    """``linear_few_rows`` with everything that does not change from call to call checked and looked up once: returns
+    ``call(x) -> output or None`` for activations of x's shape and dtype against these weights under the present
+    ``block_linear_config``, or None when the one-launch kernel does not cover the case.  The closure holds the
+    tensors it was made from; make a new one when the weights' buffers, the bias or the configuration change."""
+    block = block_linear_config.GROUP_SIZE
+    dtype = block_linear_config.INPUT_OUTPUT_TORCH_TYPE
+    M, K = x.shape
+    N = W_int8.shape[0]
+    if not (1 <= M <= _FEW_ROWS and block in (64, 128) and K > 0 and K % 128 == 0 and N > 0 and x.dtype == dtype
+            and x.dtype in _DT and W_int8.dtype == torch.int8 and state_W.dtype == torch.float32 and x.is_cuda and W_int8.is_cuda
+            and W_int8.shape[1] == K and tuple(state_W.shape) == (K // block, N) and state_W.is_contiguous()
+            and W_int8.stride(1) == 1 and (bias is None or (bias.is_cuda and bias.numel() == N and bias.dtype in _DT and bias.is_contiguous()))
+            and _few_rows_lds(M, K, block, x.element_size()) <= _FEW_ROWS_LDS):
+        return None
+    fn = _lib.load().bi8_linear_few_rows
+    guard = _on_device(x)
+    dt, ldw, dev, index = _DT[dtype], _ld(W_int8), x.device, x.device.index
+    w_ptr, sw_ptr = W_int8.data_ptr(), state_W.data_ptr()
+    b_ptr, b_dt = (None, 0) if bias is None else (bias.data_ptr(), _DT[bias.dtype])
+    keep = (W_int8, state_W, bias)
+    raw, unsupported, check, empty = _raw_stream, _lib.ERR_UNSUPPORTED, _lib.check, torch.empty
+
+    def call(x):
+        if x.stride(1) != 1:
+            return None
+        c = empty((M, N), device=dev, dtype=dtype)
+        with guard:
+            rc = fn(x.data_ptr(), dt, w_ptr, sw_ptr, b_ptr, b_dt, c.data_ptr(), M, N, K, x.stride(0) if M > 1 else K, ldw, N, block,
+                    raw(index) if raw is not None else torch.cuda.current_stream(dev).cuda_stream)
+        if rc:
+            if rc == unsupported:                   # alignment of a view, for instance
+                return None
+            check(rc, "bi8_linear_few_rows")
+        return c
+
+    call.keep = keep
+    return call
 
 
 def int8_matmul_block_partials(a, b, fblock_size=None):

@@ -168,8 +168,11 @@ def test_llama_decoder_prefill_and_decode(pkg, monkeypatch):
         # the same tokens from a HIP graph replay of the decode step, and with two launches per decode linear
         logits_g, graphed = _greedy(model, tokens, decode, graph=True)
         assert torch.equal(logits_g, logits) and torch.equal(graphed, eager)
-        monkeypatch.setattr(bl, "linear_few_rows", lambda *a, **k: None)
+        monkeypatch.setattr(bl, "few_rows_plan", lambda *a, **k: None)       # no one-launch path: quantize, then multiply
+        for m in linears:
+            m._few_rows = None                                                   # (the modules keep what they were given)
         _, two_launch = _greedy(model, tokens, decode, graph=False)
+        assert all(m._few_rows is not None and m._few_rows[1] is None for m in linears)
         assert torch.equal(two_launch, eager)
         assert len(set(eager.tolist())) > 1         # not stuck on one token
         print(f"[llama decoder] prefill {prefill} + {decode} greedy tokens, eager: {t_eager:.2f} s")

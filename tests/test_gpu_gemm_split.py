@@ -1,5 +1,5 @@
-"""bi8_gemm_nt_dequant_ws: the contraction split over the workgroups in equal runs of (tile, stage of K) pairs, through
-a caller-provided workspace.
+"""bi8_gemm_nt_dequant_ws: the contraction split over the workgroups (equal pieces of every tile, or equal runs of
+(tile, stage of K) pairs) through a caller-provided workspace.
 Against the CPU checker to the GEMM tolerance, and against the one-pass entry point (same numbers up to the fp32
 rounding of a different summation order)."""
 import ctypes
@@ -47,10 +47,13 @@ def _run(lib, A, W, sa, sw, bias, block, out, ws_bytes):
 
 
 @pytest.mark.parametrize("out", ["f32", "bf16", "f16"])
-@pytest.mark.parametrize("M,N,K,block", [(128, 512, 2048, 128), (100, 300, 2048, 64), (48, 700, 2560, 128), (200, 130, 4096, 32),
-                                         (384, 256, 8192, 64), (128, 4096, 4096, 128), (33, 128, 2048, 128),
-                                         # 20 and 25 stages of K in pieces of 8, 8, 4 and 7, 7, 7, 4
-                                         (48, 700, 2560, 128), (60, 4400, 3200, 128), (200, 300, 3200, 64)])
+@pytest.mark.parametrize("M,N,K,block", [(128, 512, 2048, 128), (100, 300, 2048, 64), (80, 700, 2560, 128), (200, 130, 4096, 32),
+                                         (384, 256, 8192, 64), (128, 4096, 4096, 128),
+                                         # up to 64 rows split where the one-pass kernel would stream too much of A or take
+                                         # more than one round of workgroups
+                                         (33, 128, 10240, 128), (48, 700, 7168, 128), (60, 4800, 3200, 128), (40, 700, 2560, 32),
+                                         # 25 stages of K in pieces of 7, 7, 7, 4
+                                         (200, 300, 3200, 64)])
 def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
     want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
@@ -72,14 +75,26 @@ def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
     assert torch.equal(with_bias, split + bias.to(DEV).to(DTYPES[out]))
 
 
-@pytest.mark.parametrize("M,N,K,block", [(3072, 768, 8192, 64), (1700, 1300, 16384, 128), (3000, 700, 8192, 32)])
-def test_more_tiles_than_half_the_chip(lib, M, N, K, block):
-    """129 to 255 tiles of 128x128 and a long K: 256 workgroups, each a run of (tile, stage) pairs that ends inside a tile.
-    The checker on sampled rows (every row of tiles is hit), the one-pass kernel on everything."""
+@pytest.mark.parametrize("M,N,K,block,kernel", [
+    # 129 to 255 tiles of 128x128 and a long K: 256 workgroups, each a run of (tile, stage) pairs that ends inside a tile
+    (2048, 1408, 16384, 64, "gemm_tile_128x128_splitk"), (2000, 1400, 16384, 128, "gemm_tile_128x128_splitk"),
+    (3000, 700, 8192, 32, "gemm_tile_128x128_splitk"),
+    # few tiles of 256x128 and a long K: three or four pieces per tile on the 256x256 kernel's loop (72 tiles x 3 pieces of 22,
+    # 22 and 20 stages; 77 x 3 pieces of 44, 44, 40; 54 x 4 of 16 stages, ragged edges)
+    (3072, 768, 8192, 64, "gemm_wide_256x128_splitk"), (1700, 1300, 16384, 128, "gemm_wide_256x128_splitk"),
+    (2200, 700, 8192, 128, "gemm_wide_256x128_splitk")])
+def test_more_tiles_than_half_the_chip(lib, M, N, K, block, kernel):
+    """The splits of problems that fill more than half of the chip with tiles.  The checker on sampled rows (every row of
+    tiles is hit), the one-pass kernel on everything."""
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
     want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
-    tiles = -(-M // 128) * -(-N // 128)
-    assert want % (128 * 128 * 4) == 0 and 240 + tiles <= want // (128 * 128 * 4) <= 256 + tiles - 1
+    assert lib.bi8_gemm_kernel_name(M, N, K, K, K, block, want).decode() == kernel
+    if "wide" in kernel:
+        tiles = -(-M // 256) * -(-N // 128)
+        assert want % (256 * 128 * 4) == 0 and 160 <= want // (256 * 128 * 4) <= 256 and (want // (256 * 128 * 4)) % tiles == 0
+    else:
+        tiles = -(-M // 128) * -(-N // 128)
+        assert want % (128 * 128 * 4) == 0 and 240 + tiles <= want // (128 * 128 * 4) <= 256 + tiles - 1
     Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
     split = _run(lib, Ad, Wd, sad, swd, bias, block, "f32", want)
     one = _run(lib, Ad, Wd, sad, swd, bias, block, "f32", 0)

@@ -104,7 +104,10 @@ CASES = [
     (300, 500, 512, 128, "gemm_tile_128x128"),
     (300, 500, 512, 32, "gemm_tile_128x128"),
     (2304, 2304, 256, 32, "gemm_tile_128x128"),
-    (48, 700, 640, 64, "gemm_tile_64x128"),
+    (48, 5000, 640, 64, "gemm_tile_64x128"),        # more columns than one round of the one-pass kernel's workgroups covers
+    (48, 700, 640, 64, "gemv_staged"),              # four groups of 16 rows
+    (64, 4096, 1024, 128, "gemv_staged"),
+    (33, 1000, 2048 + 128, 128, "gemv_staged"),
     (1, 384, 512, 128, "gemv_rows"),
     (2, 1000, 4096 + 384, 128, "gemv_rows"),        # more than four runs of 1 KiB per row, the last one partial
     (2, 700, 2048 + 128, 64, "gemv_rows"),
