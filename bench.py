@@ -151,6 +151,16 @@ def bench_extras(pkg, torch):
     g64()
     t = median_ms(g64, 10)
     out["gemm_block64_8192"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1)}
+    del sa, sw
+    sa = torch.rand(S // 32, S, device="cuda") + 0.5
+    sw = torch.rand(S // 32, S, device="cuda") * 0.02
+
+    def g32():
+        assert lib.bi8_gemm_nt_dequant(a.data_ptr(), w.data_ptr(), sa.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
+                                       S, S, S, S, S, S, 32, st) == 0
+    g32()
+    t = median_ms(g32, 10)
+    out["gemm_block32_8192"] = {"ms": round(t, 4), "TOPS": round(2.0 * S ** 3 / t / 1e9, 1)}
     del sa, sw, c
 
     # Context, not part of the path: the vendor library's PLAIN int8 GEMM (int32 out, no scales, no fold) on random
@@ -224,23 +234,29 @@ def bench_extras(pkg, torch):
                 out[f"decode_linear_M1_K{K}_N{N}"] = {"one_kernel_us": round(t1 * 1e3, 2), "two_launches_us": round(t2 * 1e3, 2)}
         del ws
 
-    # Llama-7B prefill shapes at 2048 tokens (the first: 344 tiles of 256x256, run as 256 of them and a second launch)
-    for (M, N, K) in ((2048, 11008, 4096), (2048, 4096, 4096)):
-        x = torch.randint(-127, 128, (M, K), device="cuda", dtype=torch.int8)
-        w = torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8)
-        sx = torch.rand(K // B, M, device="cuda") + 0.5
-        sw = torch.rand(K // B, N, device="cuda") * 0.02
-        c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+    # The Llama-7B GEMM shapes at 2048 and at 128 rows of activations (prefill; a decode batch): through the entry point
+    # that takes scratch memory, as the Python operator calls it (problems of few tiles split K over the workgroups)
+    for M in (2048, 128):
+        for (K, N) in ((4096, 4096), (4096, 11008), (11008, 4096), (4096, 12288)):
+            x = torch.randint(-127, 128, (M, K), device="cuda", dtype=torch.int8)
+            w = torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8)
+            sx = torch.rand(K // B, M, device="cuda") + 0.5
+            sw = torch.rand(K // B, N, device="cuda") * 0.02
+            c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+            need = lib.bi8_gemm_workspace_bytes(M, N, K, B)
+            ws = torch.empty(max(need, 16), device="cuda", dtype=torch.uint8)
 
-        def gp():
-            assert lib.bi8_gemm_nt_dequant(x.data_ptr(), w.data_ptr(), sx.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
-                                           M, N, K, K, K, N, B, st) == 0
-        for _ in range(20):
-            gp()
-        t = median_ms(gp, 30)
-        out[f"prefill_gemm_M{M}_K{K}_N{N}"] = {"us": round(t * 1e3, 1), "TOPS": round(2.0 * M * N * K / t / 1e9, 1),
-                                               "kernel": lib.bi8_gemm_kernel_name(M, N, K, K, K, B, 0).decode()}
-        del x, w, c
+            def gp():
+                assert lib.bi8_gemm_nt_dequant_ws(x.data_ptr(), w.data_ptr(), sx.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
+                                                  M, N, K, K, K, N, B, ws.data_ptr(), need, st) == 0
+            for _ in range(20):
+                gp()
+            t = median_ms(gp, 30)
+            out[f"{'prefill' if M == 2048 else 'batch128'}_gemm_M{M}_K{K}_N{N}"] = {
+                "us": round(t * 1e3, 1), "TOPS": round(2.0 * M * N * K / t / 1e9, 1),
+                "frac_int8_peak": round(2.0 * M * N * K / t / 1e9 / INT8_PEAK_TOPS, 4),
+                "kernel": lib.bi8_gemm_kernel_name(M, N, K, K, K, B, need).decode()}
+            del x, w, c, ws
 
     M = K = 8192
     xs = [torch.randn(M, K, device="cuda", dtype=torch.float32).to(torch.bfloat16) for _ in range(3)]
@@ -375,6 +391,16 @@ def main():
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
 
+    # context: the vendor library's plain int8 GEMM (int32 out, no scales, nothing folded) on the SAME operands, right
+    # after the timed region, with the clocks where the timed launches left them
+    vendor_ms = None
+    try:
+        for _ in range(10):
+            torch._int_mm(xq, wqt)
+        vendor_ms = median_ms(lambda: torch._int_mm(xq, wqt), args.steps)
+    except Exception:                               # not every torch build has it: the figure is context only
+        pass
+
     ops_per_launch = 2.0 * S * S * S
     kern_ms = evs[0].elapsed_time(evs[-1]) / args.steps
     per_launch = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
@@ -400,7 +426,9 @@ def main():
                      "kernel": f"{kernel}<{B},bf16> (the library's choice for this shape: bi8_gemm_kernel_name)",
                      "ops_per_launch": ops_per_launch, "avg_launch_ms": round(kern_ms, 4), "median_launch_ms": round(launch_median, 4),
                      "frac_of_5033_TOPs_at_2p4GHz": round(achieved / 5033.2, 4),
-                     "preroll_launches": preroll_launches, "preroll_last_batch_ms": None if preroll_ms is None else round(preroll_ms, 4)},
+                     "preroll_launches": preroll_launches, "preroll_last_batch_ms": None if preroll_ms is None else round(preroll_ms, 4),
+                     "context_vendor_plain_int8_gemm_same_operands_ms": None if vendor_ms is None else round(vendor_ms, 4),
+                     "time_relative_to_vendor_plain_int8_gemm": None if vendor_ms is None else round(kern_ms / vendor_ms, 3)},
     }
     if not args.no_quantize:
         res["quantize_roundtrip"] = bench_quantize(pkg, torch, 50)

@@ -1376,10 +1376,17 @@ __global__ __launch_bounds__(512) void gemm_wide32(const GemmArgs g) {
     // the 1.5*2^23 offset), then the row scale and the accumulation
     auto fold_slice = [&](const bi8_v16i &pt, int j, int q) {
         const float b = bc[j & 1][0], cm = bc[j & 1][1];
+        // in groups of four: the four products first, so that no instruction reads the result of the one before it
+        // (block 32 at 8192^3: 1.241 -> 1.220 ms)
 #pragma unroll
-        for (int r = q * (16 / KSB); r < (q + 1) * (16 / KSB); ++r) {
-            const float u = __builtin_fmaf(bi8_u2f((uint32_t)pt[r]), b, cm);
-            acc[j][r] = __builtin_fmaf(u, sx[r >> 2][r & 3], acc[j][r]);
+        for (int r0 = q * (16 / KSB); r0 < (q + 1) * (16 / KSB); r0 += 4) {
+            float u[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) u[r] = __builtin_fmaf(bi8_u2f((uint32_t)pt[r0 + r]), b, cm);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[j][r0 + r] = __builtin_fmaf(u[r], sx[(r0 + r) >> 2][r], acc[j][r0 + r]);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto wait_vm = [&](auto pending_c) {
