@@ -375,6 +375,11 @@ def main():
 
     step()
     torch.cuda.synchronize()
+    # For the record, the figure WITHOUT the pre-roll below: `warmup` launches, then `steps` timed ones, straight from an
+    # idle chip, whose shader clock is still ramping (reported as roofline.cold_start_avg_launch_ms; not the headline)
+    for _ in range(args.warmup):
+        step()
+    cold_ms = event_ms(step, args.steps)
     preroll_launches, preroll_ms = (0, None) if args.no_preroll else preroll(step, torch)
     for _ in range(args.warmup):
         step()
@@ -427,6 +432,7 @@ def main():
                      "ops_per_launch": ops_per_launch, "avg_launch_ms": round(kern_ms, 4), "median_launch_ms": round(launch_median, 4),
                      "frac_of_5033_TOPs_at_2p4GHz": round(achieved / 5033.2, 4),
                      "preroll_launches": preroll_launches, "preroll_last_batch_ms": None if preroll_ms is None else round(preroll_ms, 4),
+                     "cold_start_avg_launch_ms": round(cold_ms, 4),
                      "context_vendor_plain_int8_gemm_same_operands_ms": None if vendor_ms is None else round(vendor_ms, 4),
                      "time_relative_to_vendor_plain_int8_gemm": None if vendor_ms is None else round(kern_ms / vendor_ms, 3)},
     }
