@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0          # HBM3E, 8 TB/s
 # WRITE_SIZE of rocprofv3 --pmc runs of this file, scaled by what the same counters read for a 256 MiB copy
 # (x2.0 and x1.0); the runs and figures are in profiles/gemm_wide_8192x8192x8192_block128.md.  Counters cannot be read
 # from inside the process, so this is a constant from those runs, labelled as such in the output ("traffic_source").
-GEMM_8192_TRAFFIC_BYTES = 965859463
+GEMM_8192_TRAFFIC_BYTES = 966812913
 GEMM_8192_TRAFFIC_SOURCE = ("profiles/gemm_wide_8192x8192x8192_block128.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
                             "command, scaled by a 256 MiB copy; a constant, not measured in this run")
 PREROLL_MAX = 400              # launches
@@ -330,6 +330,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--size", type=int, default=8192, help="M = N = K of the GEMM (the metric is quoted at 8192)")
+    ap.add_argument("--shape", type=int, nargs=3, metavar=("M", "N", "K"), default=None,
+                    help="another GEMM shape in place of the headline one (for profiles of the kernels that run other shapes)")
+    ap.add_argument("--block", type=int, default=None, help="block size of the GEMM with --shape (default 128)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-quantize", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the secondary figures (their small launches share kernel names with the round trip)")
@@ -353,6 +356,9 @@ def main():
     B = cfg.GROUP_SIZE
     assert B == 128 and cfg.INPUT_OUTPUT_TORCH_TYPE == torch.bfloat16
     S = args.size
+    M, N, K = args.shape if args.shape else (S, S, S)
+    if args.shape and args.block:
+        B = cfg.GROUP_SIZE = args.block
 
     if args.calibrate_copy:
         src = torch.empty(256 * 1024 * 1024, device="cuda", dtype=torch.uint8).random_(0, 255)
@@ -363,8 +369,8 @@ def main():
         del src, dst
 
     torch.manual_seed(0)
-    x = torch.randn(S, S, device="cuda", dtype=torch.float32).to(torch.bfloat16)
-    w = (torch.randn(S, S, device="cuda", dtype=torch.float32) * 0.02).to(torch.bfloat16)
+    x = torch.randn(M, K, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    w = (torch.randn(N, K, device="cuda", dtype=torch.float32) * 0.02).to(torch.bfloat16)
     xq, sx = pkg.quantize_block_rowwise(x)
     wq, sw = pkg.quantize_block_rowwise(w)
     wqt = wq.t()
@@ -406,13 +412,14 @@ def main():
     except Exception:                               # not every torch build has it: the figure is context only
         pass
 
-    ops_per_launch = 2.0 * S * S * S
+    ops_per_launch = 2.0 * M * N * K
     kern_ms = evs[0].elapsed_time(evs[-1]) / args.steps
     per_launch = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps))
     launch_median = per_launch[len(per_launch) // 2] if len(per_launch) % 2 else 0.5 * (per_launch[len(per_launch) // 2 - 1] + per_launch[len(per_launch) // 2])
     achieved = ops_per_launch / kern_ms / 1e9       # TOPS
     lib = _lib.load()
-    kernel = lib.bi8_gemm_kernel_name(S, S, S, S, S, B, lib.bi8_gemm_workspace_bytes(S, S, S, B)).decode()
+    kernel = lib.bi8_gemm_kernel_name(M, N, K, K, K, B, lib.bi8_gemm_workspace_bytes(M, N, K, B)).decode()
+    headline = (M, N, K, B) == (8192, 8192, 8192, 128)
 
     res = {
         "metric": "int8 block GEMM TOPS (% int8 MFMA peak) at 8192^3; quantize GB/s (% HBM)",
@@ -420,14 +427,14 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
-        "config": {"workload": f"int8 block GEMM + fused dequantize, M=N=K={S}, block {B}, bf16 out; A = quantize(bf16 N(0,1)), "
+        "config": {"workload": f"int8 block GEMM + fused dequantize, M={M} N={N} K={K}, block {B}, bf16 out; A = quantize(bf16 N(0,1)), "
                                f"W = quantize(bf16 0.02*N(0,1)), seed 0; one launch per step via "
                                f"int8_matmul_block64_rowwise_dequantize",
                    "block": B, "out_dtype": "bf16"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                      "frac": round(achieved / INT8_PEAK_TOPS, 4),
-                     "traffic": GEMM_8192_TRAFFIC_BYTES if (S == 8192 and B == 128) else None,
-                     "traffic_source": GEMM_8192_TRAFFIC_SOURCE if (S == 8192 and B == 128) else None,
+                     "traffic": GEMM_8192_TRAFFIC_BYTES if headline else None,
+                     "traffic_source": GEMM_8192_TRAFFIC_SOURCE if headline else None,
                      "kernel": f"{kernel}<{B},bf16> (the library's choice for this shape: bi8_gemm_kernel_name)",
                      "ops_per_launch": ops_per_launch, "avg_launch_ms": round(kern_ms, 4), "median_launch_ms": round(launch_median, 4),
                      "frac_of_5033_TOPs_at_2p4GHz": round(achieved / 5033.2, 4),
