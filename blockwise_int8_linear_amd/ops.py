@@ -228,6 +228,18 @@ def _pad_contraction(a, w, state_x, state_w, block, a_store=None, w_store=None):
     return a, w, state_x, state_w, k_pad
 
 
+def _halve_wide_blocks(state_x, state_w, block, M, N, K):
+    """A K-block of 256, 512, ... codes is two, four, ... runs of 128 codes that share their scales: with every scale row
+    repeated block/128 times the GEMM runs at block 128 on the MFMA kernels, where the library itself has only its
+    general kernel for such blocks (~40x slower).  Same numbers up to fp32 rounding: the int32 partial of the block is
+    folded into the accumulator in pieces of 128 codes, each with the block's scales, instead of in one.  (The
+    reference's kernel takes any power of two as its BLOCK_K, triton_functions.py:30, :43-56.)"""
+    if block <= 128 or block % 128 != 0 or block & (block - 1) or K == 0 or M * N * K < _PAD_MIN_WORK:
+        return state_x, state_w, block
+    rows = ceil_div(K, 128)
+    return (state_x.repeat_interleave(block // 128, dim=0)[:rows], state_w.repeat_interleave(block // 128, dim=0)[:rows], 128)
+
+
 def int8_matmul_block64_rowwise_dequantize(a, b, state_x, state_w, bias=None):
     """a int8 [M,K], b int8 [K,N] (any strides), state_x [K/B, M], state_w [K/B, N], bias [N] or None
     -> [M,N] of INPUT_OUTPUT_TORCH_TYPE; triton_functions.py:142-168.  B = GROUP_SIZE at call time."""
@@ -244,6 +256,7 @@ def _int8_matmul(a, b, state_x, state_w, bias=None, a_store=None, w_store=None):
     nblk = ceil_div(K, block)
     assert tuple(state_x.shape) == (nblk, M) and tuple(state_w.shape) == (nblk, N), "scale shapes must be [ceil(K/block), rows]"
     state_x, state_w = _scales_in(state_x), _scales_in(state_w)
+    state_x, state_w, block = _halve_wide_blocks(state_x, state_w, block, M, N, K)
     a, w, state_x, state_w, K = _pad_contraction(a, w, state_x, state_w, block, a_store, w_store)
     c = torch.empty((M, N), device=a.device, dtype=out_dtype)
     bias_ptr, bias_dt = None, 0

@@ -299,6 +299,44 @@ def test_other_block_sizes_run_the_general_kernel(ops, block):
     assert torch.equal(P.cpu(), P_ref)
 
 
+@pytest.mark.parametrize("block", [256, 512, 1024])
+@pytest.mark.parametrize("shape", [(300, 500, 2048), (2048, 2304, 1024), (2944, 2944, 1536), (40, 700, 1280), (300, 500, 1000)])
+@pytest.mark.parametrize("out", ["f32", "bf16"])
+def test_blocks_above_128_run_the_block_128_kernels(ops, block, shape, out):
+    """Blocks of 256, 512, 1024 codes: the operator repeats every scale row block/128 times and runs the GEMM at block 128
+    (a block's partial is folded in pieces of 128 codes that share its scales).  Against the checker at the real block
+    size, to the GEMM tolerance; K = 1536 and 1280 end in a partial block, K = 1000 also goes through the zero-padded copy.
+    With every scale 1 and small codes the pieces add up exactly: the output is the block partials' sum, rounded once."""
+    M, N, K = shape
+    g = torch.Generator().manual_seed(block + M + K)
+    A, W = _codes(g, M, K), _codes(g, N, K)
+    nblk = -(-K // block)
+    sa = torch.rand(nblk, M, generator=g) + 0.1
+    sw = torch.rand(nblk, N, generator=g) * 0.05 + 1e-3
+    bias = torch.randn(N, generator=g)
+    P_ref, ref, _ = _reference(A, W, sa, sw, block, None, DTYPES[out])
+    # the terms that are rounded and added are those of the pieces of 128 codes: where a block's pieces cancel, the error
+    # scales with the pieces, not with the block's partial (which can be exactly 0)
+    rows = -(-K // 128)
+    _, _, mag = _reference(A, W, sa.repeat_interleave(block // 128, 0)[:rows], sw.repeat_interleave(block // 128, 0)[:rows], 128, None, DTYPES[out])
+    with cfg_as(ops, block, DTYPES[out]):
+        C = ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa.to(DEV), sw.to(DEV))
+        Cb = ops.int8_matmul_block64_rowwise_dequantize(A.to(DEV), W.to(DEV).t(), sa.to(DEV), sw.to(DEV), bias.to(DEV))
+    assert C.dtype == DTYPES[out]
+    _assert_close(C.cpu(), ref, mag, TOL[out])
+    assert torch.equal(Cb, C + bias.to(DEV).to(DTYPES[out]))
+    from blockwise_int8_linear_amd import _lib
+    lib = _lib.load()
+    k128 = -(-K // 128) * 128
+    split = "splitk" in lib.bi8_gemm_kernel_name(M, N, k128, k128, k128, 128, lib.bi8_gemm_workspace_bytes(M, N, k128, 128)).decode()
+    if out == "f32" and not split:                  # (a split of K scales every piece before it adds them)
+        small = torch.randint(-3, 4, (M, K), generator=g, dtype=torch.int32).to(torch.int8)
+        with cfg_as(ops, block, torch.float32):
+            C1 = ops.int8_matmul_block64_rowwise_dequantize(small.to(DEV), W.to(DEV).t(), torch.ones(nblk, M, device=DEV), torch.ones(nblk, N, device=DEV))
+        want = oracle_torch.gemm_nt_partials(small, W, block).sum(0).float() * torch.tensor(1.0 / (127.0 * 127.0), dtype=torch.float32)
+        assert torch.equal(C1.cpu(), want)
+
+
 def test_empty_dimensions(ops):
     """M = 0 and N = 0 give empty outputs; K = 0 gives zeros (plus bias), for few and for many rows"""
     with cfg_as(ops, 128, torch.float32):
