@@ -182,6 +182,13 @@ __device__ __forceinline__ float load_bias(const GemmArgs &g, int64_t n) {
     return bi8_from_f16_bits(((const uint16_t *)g.bias)[n]);
 }
 
+// A slab element of a split contraction (gemm_tile): stored with device scope (cache policy sc1: written through to
+// memory instead of staying in the writing XCD's L2 until the kernel ends, when all of it would be written back at
+// once).  Measured against plain stores, both kernels of the call: 128 x 4096 x 4096 14.7 -> 14.1 us, 128 x 11008 x 4096
+// 22.2 -> 21.6, 256 x 4096 x 4096 20.7 -> 20.1; on the 256x128 slabs of gemm_wide's split +-1 %, not used there.
+__device__ __forceinline__ void slab_store(float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+constexpr int kSplitMax = 8;                   // most slabs per tile
+
 // LDS map of gemm_tile: one region per operand, each a ring of kBufs stage buffers.
 template <int BM, int BN, int BLK, int NBUF> struct TileLds {
     static constexpr int kBufs = NBUF;
@@ -198,7 +205,8 @@ template <int BM, int BN, int BLK, int NBUF> struct TileLds {
 
 // BM x BN output tile per workgroup, WM x WN waves (each TM x TN subtiles of 32x32), BLK = quantization block.
 // One tile (tile_m, tile_n) of the problem `g`, by one workgroup.
-template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS>
+// SLAB: the output is a slab of a split contraction (fp32, no bias), stored with slab_store.
+template <int BM, int BN, int WM, int WN, int NBUF, int BLK, int CDT, bool PARTIALS, bool SLAB = false>
 __device__ __forceinline__ void gemm_tile_body(const GemmArgs g, const int tile_m, const int tile_n) {
     using L = TileLds<BM, BN, BLK, NBUF>;
     constexpr int kBufs = NBUF;
@@ -636,7 +644,11 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs g, const int tile_
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int64_t m = m0 + wm * (BM / WM) + a * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
-                    if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[a][b][r] * div, has_bias, bias);
+                    if constexpr (SLAB) {
+                        if (n_ok && m < g.M) slab_store((float *)g.C + (m * g.ldc + n), acc[a][b][r] * div);
+                    } else {
+                        if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[a][b][r] * div, has_bias, bias);
+                    }
                 }
         }
     }
@@ -691,7 +703,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
             g.C = g.ws + (int64_t)slab * (BM * BN) - ((int64_t)tile_m * BM * BN + (int64_t)tile_n * BN);
             g.ldc = BN;
             g.bias = nullptr;
-            gemm_tile_body<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>(g, tile_m, tile_n);
+            gemm_tile_body<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS, true>(g, tile_m, tile_n);
             __syncthreads();                       // the next piece's loads reuse the stage buffers
         }
     } else {
@@ -701,6 +713,222 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
         // where buffer descriptors have to be)
         gemm_tile_body<BM, BN, WM, WN, NBUF, BLK, CDT, PARTIALS>(g_in, __builtin_amdgcn_readfirstlane(tile_m) + g_in.tile_m0,
                                                                  __builtin_amdgcn_readfirstlane(tile_n) + g_in.tile_n0);
+    }
+}
+
+// ---- 128 x (16 ... 64) tile for 65 ... 128 rows, the whole contraction in one workgroup ---------------------------------
+// A problem of at most 128 rows against a wide W is one pass over W, and it fills the chip only if either the
+// contraction is split (slabs, a second kernel: the split tile kernels) or the tiles are so narrow that there is one
+// for every CU.  This kernel is the second way.  A workgroup streams ALL of A (from L2) next to its few rows of W (from
+// memory), 16 KiB of A per stage of K whatever the tile's width, and that is what bounds its K loop (0.26-0.33 us per
+// stage: about 30 bytes per clock and CU through the path that loads straight into LDS); in exchange nothing is
+// written twice and nothing waits for a second launch, so it wins where K is short: measured against the split or
+// one-pass tile kernels at 128 rows, block 128, W from HBM, us, K = 768 / 2048 / 4096 / 8192: N = 768 8.4 -> 5.0,
+// 10.8 -> 7.8, 11.5 -> 11.8, 13.5 -> 20.1; N = 4096 8.6 -> 5.4, 12.8 -> 8.2, 14.9 -> 13.8, 22.1 -> 24.0; N = 11008
+// 9.2 -> 7.0, 19.3 -> 11.8, 22.5 -> 19.6, 35.3 -> 33.7: taken up to K = 4096.
+// Eight waves, each 16 rows x BN = 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8).  A ring of stage
+// buffers, every wave loads four wave-instructions per stage straight into LDS (two of A, one of W, one scale row);
+// stages past the end of K are loaded from beyond the buffers' ranges (zeros, no memory access), so the count of
+// loads in flight is the same everywhere.  ONE barrier per stage and a software pipeline across it: the MFMAs of stage
+// s are issued, then the wave waits for its loads of stage s + 1 and meets the others, refills the buffer that stage
+// s - 1 has left, reads the operand fragments of stage s + 1 from LDS, folds the partials of stage s - 1 while those
+// reads and the MFMAs are under way, and reads the scales of stage s + 1 into the registers that held those of stage
+// s - 1.  Partials and scales are double-buffered in registers by stage parity.  (Reading the fragments a stage
+// earlier, into a second set of registers, changed nothing: the loop waits for its loads, not for LDS.)
+template <int NBS, int NJ> struct PanelLds {
+    static constexpr int BN = 16 * NJ;
+    static constexpr int kABuf = 128 * kStageK, kWBuf = BN * kStageK;        // 16 KiB, 2 ... 8 KiB
+    static constexpr int kSABuf = NBS * 128 * 4, kSWBuf = NBS * 64 * 4;      // (a scale row is loaded 64 floats at a time)
+    static constexpr int kStage = kABuf + kWBuf + kSABuf + kSWBuf;
+    static constexpr int kBufs = (158 * 1024 / kStage) >= 8 ? 8 : (158 * 1024 / kStage) >= 6 ? (158 * 1024 / kStage) : 4;
+    static constexpr int kAReg = 0;
+    static constexpr int kWReg = kAReg + kBufs * kABuf;
+    static constexpr int kSAReg = kWReg + kBufs * kWBuf;
+    static constexpr int kSWReg = kSAReg + kBufs * kSABuf;
+    static constexpr int kBytes = kSWReg + kBufs * kSWBuf;
+    static_assert(kBytes <= 160 * 1024, "LDS per CU");
+};
+
+template <int BLK, int CDT, int NJ>
+__global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
+    static_assert(BLK == 128 || BLK == 64, "a K-block is one or two MFMAs of 64 bytes of K");
+    static_assert(NJ >= 1 && NJ <= 4, "16 ... 64 columns");
+    constexpr int NBS = kStageK / BLK;
+    constexpr int BM = 128, BN = 16 * NJ;
+    using L = PanelLds<NBS, NJ>;
+    constexpr int kBufs = L::kBufs;
+    constexpr int kLoadsPerStage = 4;              // per wave: rows of A twice, rows of W, a row of scales
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r16 = lane & 15, q = lane >> 4;
+    const uint32_t lds_base = bi8_lds_address(lds);
+    const int tile_m = (int)blockIdx.x / g.tiles_n, tile_n = (int)blockIdx.x - tile_m * g.tiles_n;
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int nst = (int)(g.K / kStageK);
+
+    // ---- loader: wave instruction i covers tile rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which holds
+    // source chunk (lane%8) ^ ((row >> 1) & 7).  A: i = wave and wave + 8; W: i = wave % (BN / 8) (a narrow tile has fewer
+    // instructions than waves: the others repeat one, same bytes to the same place); all of the parity of `wave`.
+    const int ld_row = lane >> 3;
+    const int ld_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+    const int w_i = wave % (BN / 8);
+    const uint32_t a_off = (uint32_t)((wave * 8 + ld_row) * g.lda + ld_chunk * 16), a_step = (uint32_t)(64 * g.lda);
+    const uint32_t w_off = (uint32_t)((w_i * 8 + ld_row) * g.ldw + ld_chunk * 16);
+    // scale rows: instruction idx -> K-block idx / 3 of the stage, and there the row scales of rows 0-63, of rows 64-127
+    // or 64 column scales (those of the tile first)
+    const int s_idx = wave % (3 * NBS), s_kb = s_idx / 3, s_r = s_idx % 3;
+    const bool s_is_a = s_r < 2;
+    const uint32_t s_lane = (uint32_t)((s_is_a ? s_r * 64 + lane : lane) * 4);
+    const uint32_t s_dst = lds_base + (s_is_a ? L::kSAReg + (s_kb * 128 + s_r * 64) * 4 : L::kSWReg + s_kb * 64 * 4);
+    const uint32_t s_bufstep = s_is_a ? L::kSABuf : L::kSWBuf;
+    const uint32_t s_row = (uint32_t)((s_is_a ? g.M : g.N) * 4);             // bytes from one K-block's scales to the next
+    const int64_t nblk = g.K / BLK;
+    const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM, w_rows = g.N - n0 < BN ? g.N - n0 : BN;
+    const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
+    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
+    const bi8_rsrc s_rsrc = s_is_a ? bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4)
+                                   : bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
+    // stage s into buffer `buf` (both wave-uniform); a stage past the end of K loads zeros from beyond the buffers' ranges
+    auto issue_stage = [&](int buf, int s) {
+        const bool real = s < nst;
+        const uint32_t k_pos = real ? (uint32_t)(s * kStageK) : (uint32_t)kBufOut;
+        const uint32_t s_pos = real ? (uint32_t)(s * NBS + s_kb) * s_row : (uint32_t)kBufOut;
+        bi8_buffer_to_lds16(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + wave * 1024, a_off, k_pos);
+        bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + 8) * 1024, a_off, k_pos, a_step);
+        bi8_buffer_to_lds16(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + w_i * 1024, w_off, k_pos);
+        bi8_buffer_to_lds4(s_rsrc, s_dst + buf * s_bufstep, s_lane, s_pos);
+    };
+    // the ring's buffer after `buf`
+    auto next_buf = [](int buf) { return buf + 1 == kBufs ? 0 : buf + 1; };
+
+    // prologue: all buffers but one get a stage; the rest of the set-up runs while they are on their way
+#pragma unroll
+    for (int s = 0; s < kBufs - 1; ++s) issue_stage(s, s);
+
+    // ---- operand fragments: lane -> row r16 of a 16-row subtile, 16-byte chunk 4*kb + q of the stage's eight, stored
+    // at chunk position (4*kb + q) ^ (r16 >> 1): the address of kb = 1 is that of kb = 0 with bit 6 flipped
+    int a_base = L::kAReg + (wave * 16 + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
+    int w_base = L::kWReg + r16 * kStageK + ((q ^ (r16 >> 1)) << 4);
+    // a subtile's outputs: lane -> column r16, rows 4q .. 4q+3
+    int sa_base = L::kSAReg + (wave * 16 + 4 * q) * 4;
+    int sw_base = L::kSWReg + r16 * 4;
+    asm volatile("" : "+v"(a_base), "+v"(w_base), "+v"(sa_base), "+v"(sw_base));
+
+    auto wait_vm = [&](auto pending_c) {
+        constexpr int kPending = decltype(pending_c)::value;
+        static_assert(kPending < 64, "vmcnt is a 6-bit field");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
+    };
+    constexpr int kMagicBits = 0x4B400000;        // bit pattern of 1.5 * 2^23
+    const bi8_v4i magic = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
+
+    float acc[NJ][4];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[j][r] = 0.0f;
+    bi8_v4i A[2], B[NJ][2];                        // [kb], [column subtile][kb]: the current stage's operands
+    bi8_v4i c[2][NBS][NJ];                         // [stage parity][K-block][column subtile]
+    bi8_v4f sx[2][NBS];                            // [stage parity][K-block]: row scales
+    float bw[2][NBS][NJ];                          // ... [column subtile]: column scales
+
+    auto read_frags = [&](int buf) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            A[kb] = *(const bi8_v4i *)(lds + (a_base ^ (kb * 64)) + buf * L::kABuf);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) B[j][kb] = *(const bi8_v4i *)(lds + (w_base ^ (kb * 64)) + buf * L::kWBuf + j * 16 * kStageK);
+        }
+    };
+    auto read_scales = [&](int buf, auto par_c) {
+        constexpr int P = decltype(par_c)::value;
+#pragma unroll
+        for (int kb = 0; kb < NBS; ++kb) {
+            sx[P][kb] = *(const bi8_v4f *)(lds + sa_base + buf * L::kSABuf + kb * 128 * 4);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) bw[P][kb][j] = *(const float *)(lds + sw_base + buf * L::kSWBuf + (kb * 64 + j * 16) * 4);
+        }
+    };
+    auto mfmas = [&](auto par_c) {
+        constexpr int P = decltype(par_c)::value;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int blk = NBS == 2 ? kb : 0;
+                const bool first = NBS == 2 || kb == 0;
+                c[P][blk][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[kb], B[j][kb], first ? magic : c[P][blk][j], 0, 0, 0);
+            }
+    };
+    auto fold = [&](auto par_c) {
+        constexpr int P = decltype(par_c)::value;
+#pragma unroll
+        for (int kb = 0; kb < NBS; ++kb)
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const float b = bi8_u2f((bi8_f2u(bw[P][kb][j]) + 2u) & ~3u);     // 22 significant bits: -(1.5*2^23)*b is exact
+                const float cm = -BI8_MAGIC * b;
+                float t[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) t[r] = __builtin_fmaf(bi8_u2f((uint32_t)c[P][kb][j][r]), b, cm);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[j][r] = __builtin_fmaf(t[r], sx[P][kb][r], acc[j][r]);
+            }
+    };
+    // stage s (parity P, operands in A and B, in buffer `buf`): MFMAs, publish stage s + 1, refill the buffer that stage
+    // s - 1 has left, read the operands of stage s + 1, fold stage s - 1, read the scales of stage s + 1
+    int buf = 0, fill = kBufs - 1;                 // the buffer of the stage being computed; the one the next loads go to
+    auto step = [&](int s, auto par_c, bool fold_prev) {
+        constexpr int P = decltype(par_c)::value;
+        using Q = std::integral_constant<int, 1 - P>;
+        mfmas(par_c);
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vm(std::integral_constant<int, (kBufs - 3) * kLoadsPerStage>{});      // stage s + 1 has landed
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        issue_stage(fill, s + kBufs - 1);
+        fill = next_buf(fill);
+        buf = next_buf(buf);
+        read_frags(buf);
+        __builtin_amdgcn_sched_barrier(0);
+        if (fold_prev) fold(Q{});
+        __builtin_amdgcn_sched_barrier(0);
+        read_scales(buf, Q{});
+    };
+
+    wait_vm(std::integral_constant<int, (kBufs - 2) * kLoadsPerStage>{});
+    __syncthreads();
+    read_frags(0);
+    read_scales(0, std::integral_constant<int, 0>{});
+    step(0, std::integral_constant<int, 0>{}, false);
+    int s = 1;
+    for (; s + 1 < nst; s += 2) {
+        step(s, std::integral_constant<int, 1>{}, true);
+        step(s + 1, std::integral_constant<int, 0>{}, true);
+    }
+    if (s < nst) {                                 // an even number of stages: one more, of odd parity
+        step(s, std::integral_constant<int, 1>{}, true);
+        fold(std::integral_constant<int, 1>{});
+    } else {
+        fold(std::integral_constant<int, 0>{});
+    }
+    wait_vm(std::integral_constant<int, 0>{});     // (the loads past the end of K) nothing may still be writing LDS when the wave ends
+
+    const float div = (float)(1.0 / (127.0 * 127.0));
+    const bool has_bias = g.bias != nullptr;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int64_t n = n0 + j * 16 + r16;
+        const bool n_ok = n < g.N;
+        const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int64_t m = m0 + wave * 16 + 4 * q + r;
+            if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[j][r] * div, has_bias, bias);
+        }
     }
 }
 
@@ -2087,7 +2315,6 @@ __global__ __launch_bounds__(256) void gemm_generic(const GemmArgs g, int block)
 // all loaded before the first addition.  With split_per_tile workgroups per tile, tile t's slabs are
 // t * split_per_tile ... ; with runs, the workgroups whose runs touch tile t are floor(t * nst / S) ...
 // floor(((t + 1) * nst - 1) / S), and workgroup w's slab for it is ws[w + t].
-constexpr int kSplitMax = 8;
 template <int CDT, int BM, int BN>
 __global__ __launch_bounds__(256) void splitk_reduce(const GemmArgs g) {
     static_assert(BN == 128 && BM % 8 == 0, "32 threads x 4 columns per row, 8 rows per workgroup");
@@ -2295,10 +2522,10 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
 
 // ---- which kernel runs a problem ------------------------------------------------------------------------------------
 // One rule, used by the launcher, by bi8_gemm_workspace_bytes and by bi8_gemm_kernel_name.
-enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKWideHalf, kKSplitWideHalf };
+enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKWideHalf, kKSplitWideHalf, kKPanel };
 static const char *const kGemmKernelNames[] = {"gemm_generic", "gemv_staged", "gemm_skinny", "gemm_wide", "gemm_tile_256x128",
                                                 "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk",
-                                                "gemm_tile_64x128_splitk", "gemv_rows", "gemm_wide_256x128", "gemm_wide_256x128_splitk"};
+                                                "gemm_tile_64x128_splitk", "gemv_rows", "gemm_wide_256x128", "gemm_wide_256x128_splitk", "gemm_panel"};
 struct GemmPlan {
     int kernel;
     int splits, split_stages;      // of the split kernels: workgroups of the split grid and 128-byte stages of K per workgroup,
@@ -2315,6 +2542,19 @@ struct GemmPlan {
 // mostly empty round and the 256x256 kernel wins (1284 against 978 TOP/s at 2304x4096x4096, 144 tiles).
 // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
 constexpr int64_t kWideMinTiles = 129;
+// gemm_panel: more than 64 rows, at most one tile of 128 x (16 ... 64) per CU, and a short K: every workgroup streams all
+// 128 rows of A, so its time grows with K faster than that of the kernels that split the contraction.  Measured against
+// what ran these shapes before (one-pass or split 64x128 / 128x128 tiles), W from HBM, block 128, us at K = 768 / 2048 /
+// 4096 / 8192: 128 x 768 8.4 -> 5.0, 10.8 -> 7.8, 11.5 -> 11.8, 13.5 -> 20.1; 128 x 4096 8.6 -> 5.4, 12.8 -> 8.2, 14.9 -> 13.8,
+// 22.1 -> 24.0; 128 x 11008 9.2 -> 7.0, 19.3 -> 11.8, 22.5 -> 19.6, 35.3 -> 33.7; 512 x 2048 8.6 -> 5.9, 15.1 -> 9.1, 22.3 -> 14.2,
+// 25.4 -> 27.2; 1024 x 1024 8.6 -> 5.8, 15.2 -> 9.1, 22.4 -> 14.5, 25.0 -> 25.5; block 64, 128 x 4096 9.6 -> 5.8, 14.8 -> 9.1,
+// 16.6 -> 15.3.  At K = 4096 it needs enough tiles to win (128 x 1024: 11.5 -> 11.9).
+constexpr int64_t kPanelMinRows = 64;          // (up to 64 rows: gemv_staged and the split 64x128 tiles)
+constexpr int64_t kPanelMaxStages = 32;        // K <= 4096 ...
+constexpr int64_t kPanelSureStages = 24;       // ... beyond 3072 only with at least kPanelMinTiles tiles of 16 columns
+constexpr int64_t kPanelMinTiles = 128;
+// the widest tile, in 16-column subtiles (block 64 at 64 columns needs more registers than a wave has)
+constexpr int panel_max_subtiles(int block) { return block == 64 ? 3 : 4; }
 constexpr int64_t kStagedMaxRows = 32;         // gemv_staged: one or two groups of 16 rows whatever the shape ...
 // ... and up to four where one round of workgroups covers the columns and a workgroup's pass over all of A stays short: every
 // workgroup streams the whole of A through its LDS, which a split of K divides.  Measured against the split 64x128 tiles,
@@ -2391,6 +2631,15 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             128 * lda + K < 0x3fffffffLL && (K / block + 16) * M * 4 < 0x3fffffffLL) {         // (gemv_staged addresses its buffers with 32-bit offsets)
             p.kernel = kKGemv;
             return p;
+        }
+        // few tiles and a short K: one narrow tile per CU, no split (gemm_panel)
+        if (M > kPanelMinRows && (block == 64 || block == 128) && (K / block + 1) * max_mn * 4 < kBufOut) {
+            const int64_t rows = (M + 127) / 128, widest = 16 * panel_max_subtiles(block), nst = K / kStageK;
+            const bool one_round = rows * ((N + widest - 1) / widest) <= kCus;
+            if (one_round && (nst <= kPanelSureStages || (nst <= kPanelMaxStages && rows * ((N + 15) / 16) >= kPanelMinTiles))) {
+                p.kernel = kKPanel;
+                return p;
+            }
         }
         if (M <= 32) {
             // (block 32) with scratch memory the split 64x128 tiles are ahead of the kernel that gathers its operands (measured
@@ -2481,6 +2730,28 @@ template <int BLK, int CDT> int launch_staged(const GemmArgs &g, hipStream_t st)
     return BI8_ERR_UNSUPPORTED;
 }
 
+// gemm_panel on the narrowest tiles that give at most one per CU
+template <int BLK, int CDT, int NJ> int launch_panel_as(GemmArgs g, hipStream_t st) {
+    using L = PanelLds<kStageK / BLK, NJ>;
+    g.tiles_m = (int)((g.M + 127) / 128);
+    g.tiles_n = (int)((g.N + 16 * NJ - 1) / (16 * NJ));
+    auto kern = gemm_panel<BLK, CDT, NJ>;
+    static LdsOptIn opted;                         // one per kernel instantiation
+    const int rc = opted.ensure((const void *)kern, L::kBytes);
+    if (rc != BI8_OK) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), L::kBytes, st, g);
+    return bi8_launch_rc();
+}
+template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) {
+    const int64_t rows = (g.M + 127) / 128;
+    if (rows * ((g.N + 15) / 16) <= kCus) return launch_panel_as<BLK, CDT, 1>(g, st);
+    if (rows * ((g.N + 31) / 32) <= kCus) return launch_panel_as<BLK, CDT, 2>(g, st);
+    if (rows * ((g.N + 47) / 48) <= kCus) return launch_panel_as<BLK, CDT, 3>(g, st);
+    if constexpr (panel_max_subtiles(BLK) >= 4)
+        if (rows * ((g.N + 63) / 64) <= kCus) return launch_panel_as<BLK, CDT, 4>(g, st);
+    return BI8_ERR_UNSUPPORTED;                    // (the plan sends no other problem here)
+}
+
 template <int BLK, int CDT> int launch_rows(const GemmArgs &g, hipStream_t st) {
     const int64_t tn = (g.N + 15) / 16;
     if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
@@ -2541,6 +2812,12 @@ int launch_kernel(const GemmArgs &g, int kernel, int splits, int split_stages, i
                 return bi8_launch_rc();
             }
             break;
+        case kKPanel:
+            if constexpr (BLK != 32) {
+                if (!whole) return BI8_ERR_UNSUPPORTED;
+                return launch_panel<BLK, CDT>(g, st);
+            }
+            break;
         case kKSplit128x128:
         case kKSplit64x128: {
             GemmArgs gs = g;
@@ -2548,10 +2825,10 @@ int launch_kernel(const GemmArgs &g, int kernel, int splits, int split_stages, i
             gs.split_stages = split_stages;
             gs.split_per_tile = split_per_tile;
             const bool big = kernel == kKSplit128x128;
+            const int bm = big ? 128 : 64;
             const int rc = big ? launch_tile<128, 128, 4, 2, kRing, BLK, BI8_F32, false, true>(gs, part, st)
                                : launch_tile<64, 128, 2, 2, kRing, BLK, BI8_F32, false, true>(gs, part, st);
             if (rc != BI8_OK) return rc;
-            const int bm = big ? 128 : 64;
             gs.tiles_m = (int)((part.rows + bm - 1) / bm);
             gs.tiles_n = (int)((part.cols + 127) / 128);
             gs.tile_m0 = (int)(part.row0 / bm);
@@ -2644,6 +2921,7 @@ static int scratch_of_current_device(void **out) {
 }
 
 extern "C" int64_t bi8_static_scratch_bytes(void) { return kScratchBytes; }
+
 
 extern "C" int bi8_gemm_nt_dequant_static(const int8_t *A, const int8_t *W, const float *sA, const float *sW, const void *bias,
                                           int bias_dtype, void *C, int c_dtype, int64_t M, int64_t N, int64_t K, int64_t lda,

@@ -240,7 +240,16 @@ def test_kernel_choice_by_shape():
     assert name(2048, 4096, 4096, 128) == "gemm_wide_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
     assert name(2048, 4096, 512, 64) == "gemm_wide_256x128" and name(2048, 2304, 512, 64) == "gemm_wide_256x128"
     assert name(2048, 4096, 4096, 128, 0, 1 << 21, 4096) == "gemm_tile_256x128"     # rows 2 MiB apart: beyond its 32-bit offsets
-    assert name(300, 500, 512, 128) == "gemm_tile_128x128" and name(48, 5000, 640, 128) == "gemm_tile_64x128"
+    assert name(1500, 1500, 512, 128) == "gemm_tile_128x128" and name(48, 5000, 640, 128) == "gemm_tile_64x128"
+    # more than 64 rows, at most one tile of 128 x (16 ... 64) per CU and K up to 4096: narrow tiles, the whole K in one workgroup
+    assert name(300, 500, 512, 128) == "gemm_panel" and name(128, 4096, 4096, 128) == "gemm_panel" and name(65, 64, 128, 64) == "gemm_panel"
+    assert name(128, 4096, 4096, 128, 1 << 30) == "gemm_panel" and name(512, 4096, 4096, 128, 1 << 30) == "gemm_panel"
+    assert name(128, 11008, 4096, 64, 1 << 30) == "gemm_panel" and name(1024, 2048, 4096, 128) == "gemm_panel"
+    assert name(128, 1024, 4096, 128) == "gemm_tile_128x128"         # K = 4096 needs 128 tiles of 16 columns to pay ...
+    assert name(128, 1024, 3072, 128) == "gemm_panel"                # ... up to 3072 any number does
+    assert name(128, 4096, 4224, 128) == "gemm_tile_128x128"         # a longer K: the kernels that split it, given scratch memory
+    assert name(512, 4096, 4096, 64) == "gemm_tile_128x128"          # block 64 stops at 48 columns: 4 x 86 tiles are more than one round
+    assert name(300, 500, 512, 32) == "gemm_tile_128x128" and name(64, 5000, 640, 128) == "gemm_tile_64x128"   # block 32, 64 rows: not its
     assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
     assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 11008, 4096, 64) == "gemv_staged"
     assert name(2, 4096, 32768, 128) == "gemv_staged"                  # 2 x 32768 codes do not fit the few-row kernel's LDS
@@ -250,17 +259,17 @@ def test_kernel_choice_by_shape():
     # 33 to 64 rows: one pass over W where one round of workgroups covers the columns and K is short, else the split tiles
     assert name(33, 4096, 4096, 128, 1 << 30) == "gemv_staged" and name(64, 4096, 4096, 64) == "gemv_staged" and name(48, 700, 640, 128) == "gemv_staged"
     assert name(48, 11008, 4096, 128, 1 << 30) == "gemm_tile_64x128_splitk" and name(48, 4096, 11008, 128, 1 << 30) == "gemm_tile_64x128_splitk"
-    assert name(65, 4096, 4096, 128, 1 << 30) == "gemm_tile_64x128_splitk"
+    assert name(65, 4096, 8192, 128, 1 << 30) == "gemm_tile_128x128_splitk"
     assert name(1, 128, 128 * 1024, 128) == "gemv_staged"            # any K: the scales stream through LDS with the stages
-    assert name(128, 4096, 4096, 128) == "gemm_tile_128x128"         # no scratch memory: one pass
+    assert name(128, 4096, 8192, 128) == "gemm_tile_128x128"         # no scratch memory: one pass
     # few tiles of 256x128 and a long K: pieces of every tile on the 256x256 kernel's loop (the GPT-2 grad-weight GEMMs)
     assert name(3072, 768, 8192, 64, 1 << 25) == "gemm_wide_256x128_splitk" and name(3072, 768, 8192, 64) == "gemm_tile_128x128"
     assert name(1024, 4096, 4096, 128, 1 << 25) == "gemm_tile_128x128"        # two pieces of 16 stages: the slabs would cost more
-    ws = lib.bi8_gemm_workspace_bytes(128, 4096, 4096, 128)
-    # 64 tiles of 64x128, four workgroups each: one fp32 slab of a tile per workgroup
-    assert ws == 4 * 128 * 4096 * 4 and name(128, 4096, 4096, 128, ws) == "gemm_tile_64x128_splitk"
-    assert name(128, 4096, 4096, 128, ws - 1) == "gemm_tile_128x128"     # too small a workspace is not used
-    assert name(512, 4096, 4096, 128, 1 << 30) == "gemm_tile_128x128_splitk"
+    ws = lib.bi8_gemm_workspace_bytes(128, 2048, 8192, 128)
+    # 32 tiles of 64x128, eight workgroups each: one fp32 slab of a tile per workgroup
+    assert ws == 8 * 128 * 2048 * 4 and name(128, 2048, 8192, 128, ws) == "gemm_tile_64x128_splitk"
+    assert name(128, 2048, 8192, 128, ws - 1) == "gemm_tile_128x128"     # too small a workspace is not used
+    assert name(512, 4096, 8192, 128, 1 << 30) == "gemm_wide_256x128_splitk" and name(512, 4096, 4096, 64, 1 << 30) == "gemm_tile_128x128_splitk"
     # 144 tiles of 128x128: runs that end inside tiles fill the chip when K is long enough to pay for the second kernel
     assert name(3072, 768, 8192, 32, 1 << 30) == "gemm_tile_128x128_splitk" and name(3072, 768, 2048, 32, 1 << 30) == "gemm_tile_128x128"
     assert name(2048, 1408, 16384, 64, 1 << 30) == "gemm_tile_128x128_splitk"      # 176 tiles: too many for pieces of 256x128 tiles

@@ -437,7 +437,7 @@ def _run_nonfinite_few_rows(ops, A, W, block, g):
 
 
 # (M, N, K, kernel family)
-NONFINITE_SHAPES = [(300, 500, 512, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (5200, 5100, 256, "gemm_wide"),
+NONFINITE_SHAPES = [(300, 500, 512, "gemm_panel"), (1500, 1500, 256, "gemm_tile_128x128"), (2600, 2900, 256, "gemm_wide"), (5200, 5100, 256, "gemm_wide"),
                     (4400, 4500, 256, "gemm_wide+gemm_tile_128x128"), (2048, 2304, 256, "gemm_wide_256x128"),
                     (8, 256, 512, "gemv_staged"), (24, 256, 512, "gemv_staged_two_row_groups"), (24, 256, 512, "gemm_skinny", 32),
                     (70, 90, 200, "gemm_generic"), (8, 256, 2560, "gemv_staged_long"), (2, 256, 1536, "gemv_rows")]

@@ -47,8 +47,9 @@ def _run(lib, A, W, sa, sw, bias, block, out, ws_bytes):
 
 
 @pytest.mark.parametrize("out", ["f32", "bf16", "f16"])
-@pytest.mark.parametrize("M,N,K,block", [(128, 512, 2048, 128), (100, 300, 2048, 64), (80, 700, 2560, 128), (200, 130, 4096, 32),
-                                         (384, 256, 8192, 64), (128, 4096, 4096, 128),
+@pytest.mark.parametrize("M,N,K,block", [(128, 512, 8192, 128), (100, 300, 5120, 64), (80, 700, 5120, 128), (200, 130, 4096, 32),
+                                         (384, 256, 8192, 64), (128, 4096, 8192, 128),
+                                         # (more than 64 rows split from K = 4096 on; below that they run narrow tiles, one pass)
                                          # up to 64 rows split where the one-pass kernel would stream too much of A or take
                                          # more than one round of workgroups
                                          (33, 128, 10240, 128), (48, 700, 7168, 128), (60, 4800, 3200, 128), (40, 700, 2560, 32),
@@ -115,7 +116,7 @@ def test_more_tiles_than_half_the_chip(lib, M, N, K, block, kernel):
 
 
 def test_workspace_too_small_or_absent_is_the_one_pass_result(lib):
-    M, N, K, block = 128, 512, 2048, 128
+    M, N, K, block = 128, 512, 8192, 128
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=3)
     Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
     want = lib.bi8_gemm_workspace_bytes(M, N, K, block)

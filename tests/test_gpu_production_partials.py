@@ -1,7 +1,7 @@
 """The int32 block partials of the kernels that produce the shipped outputs, recovered bit for bit.
 
 bi8_gemm_nt_partials runs its own kernel instantiations; the kernels behind bi8_gemm_nt_dequant (gemm_wide, the
-software-pipelined gemm_tile, gemv_staged, gemm_skinny, the split of K) and bi8_linear_few_rows fold every partial
+software-pipelined gemm_tile, gemm_panel, gemv_staged, gemm_skinny, the split of K) and bi8_linear_few_rows fold every partial
 into an fp32 accumulator straight away and never store it.  Here each of them is made to hand a partial back through
 its output: column scales all 1, row scales 1 for ONE K-block j and 0 for every other block, so that
 
@@ -101,8 +101,20 @@ CASES = [
     # software-pipelined block-128 instantiation, and its three-buffer form at block 64 (sixth entry: row pitch of A)
     (600, 11008, 256, 128, "gemm_tile_256x128", (1 << 22) - 128),
     (600, 11008, 256, 64, "gemm_tile_256x128", (1 << 22) - 128),
-    (300, 500, 512, 128, "gemm_tile_128x128"),
+    (1500, 1500, 512, 128, "gemm_tile_128x128"),
     (300, 500, 512, 32, "gemm_tile_128x128"),
+    # narrow tiles, the whole K in one workgroup: 16, 32, 48 and 64 columns per tile, one to eight rows of tiles, one stage of
+    # K to thirty-two, odd and even numbers of stages, ragged edges
+    (300, 500, 512, 128, "gemm_panel"),             # 3 x 32 tiles of 16 columns, the last row of tiles 44 rows, the last column 4
+    (128, 4096, 1024, 128, "gemm_panel"),           # 256 tiles of 16 columns
+    (128, 64, 128, 128, "gemm_panel"),              # a single stage
+    (100, 48, 256, 64, "gemm_panel"),
+    (100, 8000, 640, 128, "gemm_panel"),            # 250 tiles of 32 columns, five stages
+    (200, 3000, 1152, 64, "gemm_panel"),            # 2 x 94 tiles of 32 columns, two K-blocks per stage, nine stages
+    (128, 11008, 384, 64, "gemm_panel"),            # 230 tiles of 48 columns
+    (65, 16000, 256, 128, "gemm_panel"),            # 250 tiles of 64 columns
+    (512, 4090, 4096, 128, "gemm_panel"),           # 4 x 64 tiles of 64 columns, 32 stages
+    (1000, 500, 384, 128, "gemm_panel"),            # 8 x 32 tiles
     (2304, 2304, 256, 32, "gemm_tile_128x128"),
     (48, 5000, 640, 64, "gemm_tile_64x128"),        # more columns than one round of the one-pass kernel's workgroups covers
     (48, 700, 640, 64, "gemv_staged"),              # four groups of 16 rows
