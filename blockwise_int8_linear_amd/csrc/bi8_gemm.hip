@@ -727,8 +727,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // 10.8 -> 7.8, 11.5 -> 11.8, 13.5 -> 20.1; N = 4096 8.6 -> 5.4, 12.8 -> 8.2, 14.9 -> 13.8, 22.1 -> 24.0; N = 11008
 // 9.2 -> 7.0, 19.3 -> 11.8, 22.5 -> 19.6, 35.3 -> 33.7: taken up to K = 4096.
 // Eight waves, each 16 rows x BN = 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8).  A ring of stage
-// buffers, every wave loads four wave-instructions per stage straight into LDS (two of A, one of W, one scale row);
-// stages past the end of K are loaded from beyond the buffers' ranges (zeros, no memory access), so the count of
+// buffers, every wave loads three or four wave-instructions per stage straight into LDS (two of A, and its share of the
+// rows of W and the scale rows); stages past the end of K are loaded from beyond the buffers' ranges (zeros, no memory access), so the count of
 // loads in flight is the same everywhere.  ONE barrier per stage and a software pipeline across it: the MFMAs of stage
 // s are issued, then the wave waits for its loads of stage s + 1 and meets the others, refills the buffer that stage
 // s - 1 has left, reads the operand fragments of stage s + 1 from LDS, folds the partials of stage s - 1 while those
@@ -757,7 +757,6 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
     constexpr int BM = 128, BN = 16 * NJ;
     using L = PanelLds<NBS, NJ>;
     constexpr int kBufs = L::kBufs;
-    constexpr int kLoadsPerStage = 4;              // per wave: rows of A twice, rows of W, a row of scales
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     const int tid = threadIdx.x;
@@ -770,43 +769,77 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
     const int nst = (int)(g.K / kStageK);
 
     // ---- loader: wave instruction i covers tile rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which holds
-    // source chunk (lane%8) ^ ((row >> 1) & 7).  A: i = wave and wave + 8; W: i = wave % (BN / 8) (a narrow tile has fewer
-    // instructions than waves: the others repeat one, same bytes to the same place); all of the parity of `wave`.
+    // source chunk (lane%8) ^ ((row >> 1) & 7).  A is 16 instructions per stage: i = wave and wave + 8, both of the parity
+    // of `wave`.  The rest of a stage is BN / 8 instructions of W rows and 3 * NBS of scale rows (per K-block the row
+    // scales of rows 0-63, of rows 64-127, and 64 column scales from the tile's first on): item e * 8 + wave of that list
+    // is wave's instruction of slot e.  The path into LDS takes one wave-instruction per 16 clocks whatever it carries
+    // (a stage of A alone: 0.13 us), so nobody loads anything twice or for show: the waves whose last slot has no item
+    // issue one load less per stage, and wait with a count of their own.
     const int ld_row = lane >> 3;
     const int ld_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
-    const int w_i = wave % (BN / 8);
     const uint32_t a_off = (uint32_t)((wave * 8 + ld_row) * g.lda + ld_chunk * 16), a_step = (uint32_t)(64 * g.lda);
-    const uint32_t w_off = (uint32_t)((w_i * 8 + ld_row) * g.ldw + ld_chunk * 16);
-    // scale rows: instruction idx -> K-block idx / 3 of the stage, and there the row scales of rows 0-63, of rows 64-127
-    // or 64 column scales (those of the tile first)
-    const int s_idx = wave % (3 * NBS), s_kb = s_idx / 3, s_r = s_idx % 3;
-    const bool s_is_a = s_r < 2;
-    const uint32_t s_lane = (uint32_t)((s_is_a ? s_r * 64 + lane : lane) * 4);
-    const uint32_t s_dst = lds_base + (s_is_a ? L::kSAReg + (s_kb * 128 + s_r * 64) * 4 : L::kSWReg + s_kb * 64 * 4);
-    const uint32_t s_bufstep = s_is_a ? L::kSABuf : L::kSWBuf;
-    const uint32_t s_row = (uint32_t)((s_is_a ? g.M : g.N) * 4);             // bytes from one K-block's scales to the next
-    const int64_t nblk = g.K / BLK;
-    const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM, w_rows = g.N - n0 < BN ? g.N - n0 : BN;
+    const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM;
     const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
-    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
-    const bi8_rsrc s_rsrc = s_is_a ? bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4)
-                                   : bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
-    // stage s into buffer `buf` (both wave-uniform); a stage past the end of K loads zeros from beyond the buffers' ranges
-    auto issue_stage = [&](int buf, int s) {
-        const bool real = s < nst;
-        const uint32_t k_pos = real ? (uint32_t)(s * kStageK) : (uint32_t)kBufOut;
-        const uint32_t s_pos = real ? (uint32_t)(s * NBS + s_kb) * s_row : (uint32_t)kBufOut;
+    // stage s into buffer `buf` (both wave-uniform); past the end of K: zeros, no memory access
+    auto issue_a0 = [&](int buf, int s) {
+        const uint32_t k_pos = s < nst ? (uint32_t)(s * kStageK) : (uint32_t)kBufOut;
         bi8_buffer_to_lds16(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + wave * 1024, a_off, k_pos);
-        bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + 8) * 1024, a_off, k_pos, a_step);
-        bi8_buffer_to_lds16(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + w_i * 1024, w_off, k_pos);
-        bi8_buffer_to_lds4(s_rsrc, s_dst + buf * s_bufstep, s_lane, s_pos);
     };
+    auto issue_a1 = [&](int buf, int s) {
+        const uint32_t k_pos = s < nst ? (uint32_t)(s * kStageK) : (uint32_t)kBufOut;
+        bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + 8) * 1024, a_off, k_pos, a_step);
+    };
+    auto issue_a = [&](int buf, int s) {
+        issue_a0(buf, s);
+        issue_a1(buf, s);
+    };
+    // prologue: the first stage's rows of A are on their way before anything else is set up
+    issue_a(0, 0);
+
+    const int64_t nblk = g.K / BLK, w_rows = g.N - n0 < BN ? g.N - n0 : BN;
+    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
+    const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
+    const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
+    constexpr int kWItems = BN / 8, kItems = kWItems + 3 * NBS, kExtra = (kItems + 7) / 8;
+    constexpr int kLoadsFull = 2 + kExtra, kLoadsLess = 1 + kExtra;       // per wave and stage: with an item in every slot / none in the last
+    const bool full = (kExtra - 1) * 8 + wave < kItems;                    // wave-uniform
+    bool x_is_w[kExtra];                           // wave-uniform: rows of W (16 bytes per lane), else a scale row (4 bytes)
+    bi8_rsrc x_rsrc[kExtra];
+    uint32_t x_off[kExtra], x_dst[kExtra], x_bufstep[kExtra], x_kstep[kExtra], x_k0[kExtra];
+#pragma unroll
+    for (int e = 0; e < kExtra; ++e) {
+        const int item = e * 8 + wave;             // (a slot without an item is never issued: what is computed for it is not used)
+        const int sc = item - kWItems, kb = sc / 3, r = sc - 3 * kb;         // (as a scale item)
+        x_is_w[e] = item < kWItems;
+        const bool is_sa = r < 2;
+        x_rsrc[e] = x_is_w[e] ? w_rsrc : is_sa ? sa_rsrc : sw_rsrc;
+        x_off[e] = x_is_w[e] ? (uint32_t)((item * 8 + ld_row) * g.ldw + ld_chunk * 16) : (uint32_t)(((is_sa ? r * 64 : 0) + lane) * 4);
+        x_dst[e] = lds_base + (x_is_w[e] ? L::kWReg + item * 1024 : is_sa ? L::kSAReg + (kb * 128 + r * 64) * 4 : L::kSWReg + kb * 64 * 4);
+        x_bufstep[e] = x_is_w[e] ? L::kWBuf : is_sa ? L::kSABuf : L::kSWBuf;
+        // where stage s of the item starts: x_k0 + s * x_kstep bytes into its buffer
+        x_kstep[e] = x_is_w[e] ? (uint32_t)kStageK : (uint32_t)(NBS * (is_sa ? g.M : g.N) * 4);
+        x_k0[e] = x_is_w[e] ? 0u : (uint32_t)(kb * (is_sa ? g.M : g.N) * 4);
+    }
+    auto issue_rest = [&](int buf, int s) {
+#pragma unroll
+        for (int e = 0; e < kExtra; ++e) {
+            if (e == kExtra - 1 && !full) break;
+            const uint32_t pos = s < nst ? x_k0[e] + (uint32_t)s * x_kstep[e] : (uint32_t)kBufOut;
+            if (x_is_w[e]) bi8_buffer_to_lds16(x_rsrc[e], x_dst[e] + buf * x_bufstep[e], x_off[e], pos);
+            else bi8_buffer_to_lds4(x_rsrc[e], x_dst[e] + buf * x_bufstep[e], x_off[e], pos);
+        }
+    };
+    auto issue_stage = [&](int buf, int s) {
+        issue_a(buf, s);
+        issue_rest(buf, s);
+    };
+    // ... then the rest of it and the stages for all buffers but one
+    issue_rest(0, 0);
+#pragma unroll
+    for (int s = 1; s < kBufs - 1; ++s) issue_stage(s, s);
     // the ring's buffer after `buf`
     auto next_buf = [](int buf) { return buf + 1 == kBufs ? 0 : buf + 1; };
 
-    // prologue: all buffers but one get a stage; the rest of the set-up runs while they are on their way
-#pragma unroll
-    for (int s = 0; s < kBufs - 1; ++s) issue_stage(s, s);
 
     // ---- operand fragments: lane -> row r16 of a 16-row subtile, 16-byte chunk 4*kb + q of the stage's eight, stored
     // at chunk position (4*kb + q) ^ (r16 >> 1): the address of kb = 1 is that of kb = 0 with bit 6 flipped
@@ -821,6 +854,12 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
         constexpr int kPending = decltype(pending_c)::value;
         static_assert(kPending < 64, "vmcnt is a 6-bit field");
         __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
+    };
+    // until at most S stages' worth of this wave's loads are outstanding
+    auto wait_stages = [&](auto stages_c) {
+        constexpr int S = decltype(stages_c)::value;
+        if (full) wait_vm(std::integral_constant<int, S * kLoadsFull>{});
+        else wait_vm(std::integral_constant<int, S * kLoadsLess>{});
     };
     constexpr int kMagicBits = 0x4B400000;        // bit pattern of 1.5 * 2^23
     const bi8_v4i magic = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
@@ -886,20 +925,24 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
         using Q = std::integral_constant<int, 1 - P>;
         mfmas(par_c);
         __builtin_amdgcn_sched_barrier(0);
-        wait_vm(std::integral_constant<int, (kBufs - 3) * kLoadsPerStage>{});      // stage s + 1 has landed
+        wait_stages(std::integral_constant<int, kBufs - 3>{});                   // stage s + 1 has landed
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        issue_stage(fill, s + kBufs - 1);
-        fill = next_buf(fill);
+        // (the stage's loads are spread over the step: the path into LDS takes them one per 16 clocks, and a wave that
+        // offers three at once waits for the other waves' to drain)
         buf = next_buf(buf);
+        issue_a0(fill, s + kBufs - 1);
         read_frags(buf);
         __builtin_amdgcn_sched_barrier(0);
+        issue_a1(fill, s + kBufs - 1);
         if (fold_prev) fold(Q{});
         __builtin_amdgcn_sched_barrier(0);
+        issue_rest(fill, s + kBufs - 1);
         read_scales(buf, Q{});
+        fill = next_buf(fill);
     };
 
-    wait_vm(std::integral_constant<int, (kBufs - 2) * kLoadsPerStage>{});
+    wait_stages(std::integral_constant<int, kBufs - 2>{});                       // stage 0 has landed
     __syncthreads();
     read_frags(0);
     read_scales(0, std::integral_constant<int, 0>{});
