@@ -716,25 +716,29 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
     }
 }
 
-// ---- 128 x (16 ... 64) tile for 65 ... 128 rows, the whole contraction in one workgroup ---------------------------------
-// A problem of at most 128 rows against a wide W is one pass over W, and it fills the chip only if either the
-// contraction is split (slabs, a second kernel: the split tile kernels) or the tiles are so narrow that there is one
-// for every CU.  This kernel is the second way.  A workgroup streams ALL of A (from L2) next to its few rows of W (from
-// memory), 16 KiB of A per stage of K whatever the tile's width, and that is what bounds its K loop (0.26-0.33 us per
-// stage: about 30 bytes per clock and CU through the path that loads straight into LDS); in exchange nothing is
-// written twice and nothing waits for a second launch, so it wins where K is short: measured against the split or
-// one-pass tile kernels at 128 rows, block 128, W from HBM, us, K = 768 / 2048 / 4096 / 8192: N = 768 8.4 -> 5.0,
-// 10.8 -> 7.8, 11.5 -> 11.8, 13.5 -> 20.1; N = 4096 8.6 -> 5.4, 12.8 -> 8.2, 14.9 -> 13.8, 22.1 -> 24.0; N = 11008
-// 9.2 -> 7.0, 19.3 -> 11.8, 22.5 -> 19.6, 35.3 -> 33.7: taken up to K = 4096.
-// Eight waves, each 16 rows x BN = 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8).  A ring of stage
-// buffers, every wave loads three or four wave-instructions per stage straight into LDS (two of A, and its share of the
-// rows of W and the scale rows); stages past the end of K are loaded from beyond the buffers' ranges (zeros, no memory access), so the count of
-// loads in flight is the same everywhere.  ONE barrier per stage and a software pipeline across it: the MFMAs of stage
-// s are issued, then the wave waits for its loads of stage s + 1 and meets the others, refills the buffer that stage
-// s - 1 has left, reads the operand fragments of stage s + 1 from LDS, folds the partials of stage s - 1 while those
-// reads and the MFMAs are under way, and reads the scales of stage s + 1 into the registers that held those of stage
-// s - 1.  Partials and scales are double-buffered in registers by stage parity.  (Reading the fragments a stage
-// earlier, into a second set of registers, changed nothing: the loop waits for its loads, not for LDS.)
+// ---- 128 x (16 ... 64) tiles for problems of few tiles, the whole contraction in one workgroup -------------------------
+// A problem of a few hundred rows against a wide W fills the chip only if either the contraction is split (slabs, a
+// second kernel: the split tile kernels) or the tiles are so narrow that there is one for every CU.  This kernel is
+// the second way.  A workgroup streams ALL 128 rows of A (from L2) next to its few rows of W (from memory), 16 KiB of A
+// per stage of K whatever the tile's width; in exchange nothing is written twice and nothing waits for a second
+// launch, so it wins where K is short (the plan's rule and the measurements behind it: kPanelMaxStages).
+// Eight waves, each 16 rows x BN = 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8).  A ring of
+// six to eight stage buffers, every wave loads two to four wave-instructions per stage straight into LDS (two of A
+// and its share of the rows of W and the scale rows); stages past the end of K are loaded from beyond the buffers'
+// ranges (zeros, no memory access), so a wave's count of loads in flight is the same everywhere.  ONE barrier per stage
+// and a software pipeline across it: the MFMAs of stage s are issued, then the wave waits for its loads of stage s + 1
+// and meets the others, refills the buffer that stage s - 1 has left, reads the operand fragments of stage s + 1 from
+// LDS, folds the partials of stage s - 1 while those reads and the MFMAs are under way, and reads the scales of stage
+// s + 1 into the registers that held those of stage s - 1.  Partials and scales are double-buffered in registers by
+// stage parity.
+// What a stage costs (128 x 4096 x 4096, 32 stages, 0.31 us each; timestamps inside the kernel and parts switched
+// off): without the loop's loads 0.18 us, without the fragment reads 0.24, without the MFMAs 0.23, without the fold
+// 0.26, without the barrier 0.28 -- the parts of a stage run one after the other, in all waves at once, and a stage of
+// A alone streams into LDS in 0.13 us (read-only micro-benchmark, same grid).  Measured and not kept: the fragments
+// read a stage earlier into a second set of registers (the same), the ring filled while the first stages are computed
+// instead of in front of them (the same).  Kept: a stage's loads spread over the step (3-5 %), no load issued twice.
+// The prologue's loads are all issued 1.4 us after the kernel's first instruction, and the first stage has landed
+// 0.9 us later.
 template <int NBS, int NJ> struct PanelLds {
     static constexpr int BN = 16 * NJ;
     static constexpr int kABuf = 128 * kStageK, kWBuf = BN * kStageK;        // 16 KiB, 2 ... 8 KiB
