@@ -252,7 +252,7 @@ def bench_extras(pkg, torch):
             def gp():
                 assert lib.bi8_gemm_nt_dequant_ws(x.data_ptr(), w.data_ptr(), sx.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
                                                   M, N, K, K, K, N, B, ws.data_ptr(), need, st) == 0
-            for _ in range(20):
+            for _ in range(100 if M < 1024 else 20):          # (short kernels: the clock needs a few hundred microseconds of work to settle)
                 gp()
             t = median_ms(gp, 30)
             out[f"{'prefill' if M == 2048 else 'batch128' if M == 128 else 'tokens512'}_gemm_M{M}_K{K}_N{N}"] = {
