@@ -722,7 +722,8 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // the second way.  A workgroup streams ALL 128 rows of A (from L2) next to its few rows of W (from memory), 16 KiB of A
 // per stage of K whatever the tile's width; in exchange nothing is written twice and nothing waits for a second
 // launch, so it wins where K is short (the plan's rule and the measurements behind it: kPanelMaxStages).
-// Eight waves, each 16 rows x BN = 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8).  A ring of
+// Eight waves, each 16 rows x 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8): stacked, a tile of 128
+// rows (described here), or as 4 x 2 a tile of 64 rows x 32 * NJ columns for up to 64 rows (half the bytes of A).  A ring of
 // six to eight stage buffers, every wave loads two to four wave-instructions per stage straight into LDS (two of A
 // and its share of the rows of W and the scale rows); stages past the end of K are loaded from beyond the buffers'
 // ranges (zeros, no memory access), so a wave's count of loads in flight is the same everywhere.  ONE barrier per stage
@@ -739,10 +740,13 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // instead of in front of them (the same).  Kept: a stage's loads spread over the step (3-5 %), no load issued twice.
 // The prologue's loads are all issued 1.4 us after the kernel's first instruction, and the first stage has landed
 // 0.9 us later.
-template <int NBS, int NJ> struct PanelLds {
-    static constexpr int BN = 16 * NJ;
-    static constexpr int kABuf = 128 * kStageK, kWBuf = BN * kStageK;        // 16 KiB, 2 ... 8 KiB
-    static constexpr int kSABuf = NBS * 128 * 4, kSWBuf = NBS * 64 * 4;      // (a scale row is loaded 64 floats at a time)
+// CG = column groups of the eight waves: 1 -> 8 x 1 waves, tiles of 128 rows x 16 * NJ columns; 2 -> 4 x 2 waves, tiles of
+// 64 rows x 32 * NJ columns (for up to 64 rows: half the bytes of A per stage)
+template <int NBS, int NJ, int CG> struct PanelLds {
+    static constexpr int BM = 128 / CG, BN = 16 * NJ * CG;
+    static constexpr int kSWRow = BN > 64 ? 128 : 64;                        // (a scale row is loaded 64 floats at a time)
+    static constexpr int kABuf = BM * kStageK, kWBuf = BN * kStageK;         // 16 or 8 KiB, 2 ... 16 KiB
+    static constexpr int kSABuf = NBS * BM * 4, kSWBuf = NBS * kSWRow * 4;
     static constexpr int kStage = kABuf + kWBuf + kSABuf + kSWBuf;
     static constexpr int kBufs = (158 * 1024 / kStage) >= 8 ? 8 : (158 * 1024 / kStage) >= 6 ? (158 * 1024 / kStage) : 4;
     static constexpr int kAReg = 0;
@@ -753,19 +757,20 @@ template <int NBS, int NJ> struct PanelLds {
     static_assert(kBytes <= 160 * 1024, "LDS per CU");
 };
 
-template <int BLK, int CDT, int NJ>
+template <int BLK, int CDT, int NJ, int CG = 1>
 __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
     static_assert(BLK == 128 || BLK == 64, "a K-block is one or two MFMAs of 64 bytes of K");
-    static_assert(NJ >= 1 && NJ <= 4, "16 ... 64 columns");
+    static_assert(NJ >= 1 && NJ <= 4 && (CG == 1 || CG == 2), "16 ... 64 columns per wave, one or two waves side by side");
     constexpr int NBS = kStageK / BLK;
-    constexpr int BM = 128, BN = 16 * NJ;
-    using L = PanelLds<NBS, NJ>;
+    using L = PanelLds<NBS, NJ, CG>;
+    constexpr int BM = L::BM, BN = L::BN, RG = 8 / CG;                     // RG = row groups of 16 rows
     constexpr int kBufs = L::kBufs;
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rg = wave % RG, cg = wave / RG;                             // the wave's 16 rows, its 16 * NJ columns
     const int r16 = lane & 15, q = lane >> 4;
     const uint32_t lds_base = bi8_lds_address(lds);
     const int tile_m = (int)blockIdx.x / g.tiles_n, tile_n = (int)blockIdx.x - tile_m * g.tiles_n;
@@ -773,10 +778,10 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
     const int nst = (int)(g.K / kStageK);
 
     // ---- loader: wave instruction i covers tile rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which holds
-    // source chunk (lane%8) ^ ((row >> 1) & 7).  A is 16 instructions per stage: i = wave and wave + 8, both of the parity
-    // of `wave`.  The rest of a stage is BN / 8 instructions of W rows and 3 * NBS of scale rows (per K-block the row
-    // scales of rows 0-63, of rows 64-127, and 64 column scales from the tile's first on): item e * 8 + wave of that list
-    // is wave's instruction of slot e.  The path into LDS takes one wave-instruction per 16 clocks whatever it carries
+    // source chunk (lane%8) ^ ((row >> 1) & 7).  A is BM / 8 instructions per stage: i = wave and, of 128 rows, wave + 8, both
+    // of the parity of `wave`.  The rest of a stage is BN / 8 instructions of W rows and the scale rows (per K-block the
+    // row scales, 64 at a time, then the column scales, 64 at a time from the tile's first on): item e * 8 + wave of that
+    // list is wave's instruction of slot e.  The path into LDS takes one wave-instruction per 16 clocks whatever it carries
     // (a stage of A alone: 0.13 us), so nobody loads anything twice or for show: the waves whose last slot has no item
     // issue one load less per stage, and wait with a count of their own.
     const int ld_row = lane >> 3;
@@ -795,7 +800,7 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
     };
     auto issue_a = [&](int buf, int s) {
         issue_a0(buf, s);
-        issue_a1(buf, s);
+        if constexpr (BM == 128) issue_a1(buf, s);
     };
     // prologue: the first stage's rows of A are on their way before anything else is set up
     issue_a(0, 0);
@@ -804,8 +809,10 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
     const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
     const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
     const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
-    constexpr int kWItems = BN / 8, kItems = kWItems + 3 * NBS, kExtra = (kItems + 7) / 8;
-    constexpr int kLoadsFull = 2 + kExtra, kLoadsLess = 1 + kExtra;       // per wave and stage: with an item in every slot / none in the last
+    constexpr int kSAParts = BM / 64, kSWParts = L::kSWRow / 64, kSParts = kSAParts + kSWParts;     // scale rows of a K-block, 64 floats each
+    constexpr int kWItems = BN / 8, kItems = kWItems + kSParts * NBS, kExtra = (kItems + 7) / 8;
+    constexpr int kALoads = BM / 64;
+    constexpr int kLoadsFull = kALoads + kExtra, kLoadsLess = kALoads + kExtra - 1;       // per wave and stage: with an item in every slot / none in the last
     const bool full = (kExtra - 1) * 8 + wave < kItems;                    // wave-uniform
     bool x_is_w[kExtra];                           // wave-uniform: rows of W (16 bytes per lane), else a scale row (4 bytes)
     bi8_rsrc x_rsrc[kExtra];
@@ -813,12 +820,13 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
 #pragma unroll
     for (int e = 0; e < kExtra; ++e) {
         const int item = e * 8 + wave;             // (a slot without an item is never issued: what is computed for it is not used)
-        const int sc = item - kWItems, kb = sc / 3, r = sc - 3 * kb;         // (as a scale item)
+        const int sc = item - kWItems, kb = sc / kSParts, r = sc - kSParts * kb;         // (as a scale item)
         x_is_w[e] = item < kWItems;
-        const bool is_sa = r < 2;
+        const bool is_sa = r < kSAParts;
+        const int part = is_sa ? r : r - kSAParts;                        // which 64 of the row's scales
         x_rsrc[e] = x_is_w[e] ? w_rsrc : is_sa ? sa_rsrc : sw_rsrc;
-        x_off[e] = x_is_w[e] ? (uint32_t)((item * 8 + ld_row) * g.ldw + ld_chunk * 16) : (uint32_t)(((is_sa ? r * 64 : 0) + lane) * 4);
-        x_dst[e] = lds_base + (x_is_w[e] ? L::kWReg + item * 1024 : is_sa ? L::kSAReg + (kb * 128 + r * 64) * 4 : L::kSWReg + kb * 64 * 4);
+        x_off[e] = x_is_w[e] ? (uint32_t)((item * 8 + ld_row) * g.ldw + ld_chunk * 16) : (uint32_t)((part * 64 + lane) * 4);
+        x_dst[e] = lds_base + (x_is_w[e] ? L::kWReg + item * 1024 : is_sa ? L::kSAReg + (kb * BM + part * 64) * 4 : L::kSWReg + (kb * L::kSWRow + part * 64) * 4);
         x_bufstep[e] = x_is_w[e] ? L::kWBuf : is_sa ? L::kSABuf : L::kSWBuf;
         // where stage s of the item starts: x_k0 + s * x_kstep bytes into its buffer
         x_kstep[e] = x_is_w[e] ? (uint32_t)kStageK : (uint32_t)(NBS * (is_sa ? g.M : g.N) * 4);
@@ -847,11 +855,11 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
 
     // ---- operand fragments: lane -> row r16 of a 16-row subtile, 16-byte chunk 4*kb + q of the stage's eight, stored
     // at chunk position (4*kb + q) ^ (r16 >> 1): the address of kb = 1 is that of kb = 0 with bit 6 flipped
-    int a_base = L::kAReg + (wave * 16 + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
-    int w_base = L::kWReg + r16 * kStageK + ((q ^ (r16 >> 1)) << 4);
+    int a_base = L::kAReg + (rg * 16 + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
+    int w_base = L::kWReg + (cg * 16 * NJ + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
     // a subtile's outputs: lane -> column r16, rows 4q .. 4q+3
-    int sa_base = L::kSAReg + (wave * 16 + 4 * q) * 4;
-    int sw_base = L::kSWReg + r16 * 4;
+    int sa_base = L::kSAReg + (rg * 16 + 4 * q) * 4;
+    int sw_base = L::kSWReg + (cg * 16 * NJ + r16) * 4;
     asm volatile("" : "+v"(a_base), "+v"(w_base), "+v"(sa_base), "+v"(sw_base));
 
     auto wait_vm = [&](auto pending_c) {
@@ -890,9 +898,9 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
         constexpr int P = decltype(par_c)::value;
 #pragma unroll
         for (int kb = 0; kb < NBS; ++kb) {
-            sx[P][kb] = *(const bi8_v4f *)(lds + sa_base + buf * L::kSABuf + kb * 128 * 4);
+            sx[P][kb] = *(const bi8_v4f *)(lds + sa_base + buf * L::kSABuf + kb * BM * 4);
 #pragma unroll
-            for (int j = 0; j < NJ; ++j) bw[P][kb][j] = *(const float *)(lds + sw_base + buf * L::kSWBuf + (kb * 64 + j * 16) * 4);
+            for (int j = 0; j < NJ; ++j) bw[P][kb][j] = *(const float *)(lds + sw_base + buf * L::kSWBuf + (kb * L::kSWRow + j * 16) * 4);
         }
     };
     auto mfmas = [&](auto par_c) {
@@ -938,7 +946,7 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
         issue_a0(fill, s + kBufs - 1);
         read_frags(buf);
         __builtin_amdgcn_sched_barrier(0);
-        issue_a1(fill, s + kBufs - 1);
+        if constexpr (BM == 128) issue_a1(fill, s + kBufs - 1);
         if (fold_prev) fold(Q{});
         __builtin_amdgcn_sched_barrier(0);
         issue_rest(fill, s + kBufs - 1);
@@ -968,12 +976,12 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
     const bool has_bias = g.bias != nullptr;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-        const int64_t n = n0 + j * 16 + r16;
+        const int64_t n = n0 + cg * 16 * NJ + j * 16 + r16;
         const bool n_ok = n < g.N;
         const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int64_t m = m0 + wave * 16 + 4 * q + r;
+            const int64_t m = m0 + rg * 16 + 4 * q + r;
             if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[j][r] * div, has_bias, bias);
         }
     }
@@ -2596,10 +2604,11 @@ constexpr int64_t kWideMinTiles = 129;
 // 22.1 -> 24.0; 128 x 11008 9.2 -> 7.0, 19.3 -> 11.8, 22.5 -> 19.6, 35.3 -> 33.7; 512 x 2048 8.6 -> 5.9, 15.1 -> 9.1, 22.3 -> 14.2,
 // 25.4 -> 27.2; 1024 x 1024 8.6 -> 5.8, 15.2 -> 9.1, 22.4 -> 14.5, 25.0 -> 25.5; block 64, 128 x 4096 9.6 -> 5.8, 14.8 -> 9.1,
 // 16.6 -> 15.3.  At K = 4096 it needs enough tiles to win (128 x 1024: 11.5 -> 11.9).
-constexpr int64_t kPanelMinRows = 64;          // (up to 64 rows: gemv_staged and the split 64x128 tiles)
+constexpr int64_t kPanelMinRows = 64;          // more rows: tiles of 128 rows; 33 ... 64: tiles of 64 rows
 constexpr int64_t kPanelMaxStages = 32;        // K <= 4096 ...
 constexpr int64_t kPanelSureStages = 24;       // ... beyond 3072 only with at least kPanelMinTiles tiles of 16 columns
 constexpr int64_t kPanelMinTiles = 128;
+constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024
 // the widest tile, in 16-column subtiles (block 64 at 64 columns needs more registers than a wave has)
 constexpr int panel_max_subtiles(int block) { return block == 64 ? 3 : 4; }
 constexpr int64_t kStagedMaxRows = 32;         // gemv_staged: one or two groups of 16 rows whatever the shape ...
@@ -2673,7 +2682,20 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             p.kernel = kKRows;
             return p;
         }
-        const bool staged_rows = M <= kStagedMaxRows || (M <= kStagedWideRows && (N + 15) / 16 <= kStagedWideMaxGroups && M * K <= kStagedWideMaxCodes);
+        // 33 ... 64 rows: gemm_panel on tiles of 64 rows where the columns fit one round of them and K is at most 4096 --
+        // unless gemv_staged's four groups of rows apply, which are ahead from K = 1152 on (measured, 64 rows, block 128, W from
+        // HBM, us, gemv_staged or the split 64x128 tiles -> gemm_panel, K = 768 / 2048 / 4096 / 8192: N = 4096 5.7 -> 4.7,
+        // 6.0 -> 7.2, 10.1 -> 11.6, 16.9 -> 19.6; N = 8192 7.1 -> 5.0, 12.4 -> 7.9, 15.5 -> 13.1, 21.1 -> 23.1; N = 11008 7.5 -> 5.9,
+        // 13.6 -> 10.2, 17.4 -> 16.2, 29.4 -> 28.0; N = 16384 8.0 -> 6.6, 15.5 -> 12.5, 22.4 -> 19.4, 39.4 -> 33.5)
+        const bool staged_band = M <= kStagedWideRows && (N + 15) / 16 <= kStagedWideMaxGroups && M * K <= kStagedWideMaxCodes;
+        if (M > kStagedMaxRows && M <= kPanelMinRows && (block == 64 || block == 128) && (K / block + 1) * max_mn * 4 < kBufOut) {
+            const int64_t widest = 32 * panel_max_subtiles(block), nst = K / kStageK;
+            if ((N + widest - 1) / widest <= kCus && nst <= kPanelMaxStages && (!staged_band || nst <= kPanelOverStagedStages)) {
+                p.kernel = kKPanel;
+                return p;
+            }
+        }
+        const bool staged_rows = M <= kStagedMaxRows || staged_band;
         if (staged_rows && (block == 64 || block == 128) && (K / block + 16) * N * 4 < 0x3fffffffLL && 16 * ldw + K < 0x3fffffffLL &&
             128 * lda + K < 0x3fffffffLL && (K / block + 16) * M * 4 < 0x3fffffffLL) {         // (gemv_staged addresses its buffers with 32-bit offsets)
             p.kernel = kKGemv;
@@ -2778,25 +2800,28 @@ template <int BLK, int CDT> int launch_staged(const GemmArgs &g, hipStream_t st)
 }
 
 // gemm_panel on the narrowest tiles that give at most one per CU
-template <int BLK, int CDT, int NJ> int launch_panel_as(GemmArgs g, hipStream_t st) {
-    using L = PanelLds<kStageK / BLK, NJ>;
-    g.tiles_m = (int)((g.M + 127) / 128);
-    g.tiles_n = (int)((g.N + 16 * NJ - 1) / (16 * NJ));
-    auto kern = gemm_panel<BLK, CDT, NJ>;
+template <int BLK, int CDT, int NJ, int CG> int launch_panel_as(GemmArgs g, hipStream_t st) {
+    using L = PanelLds<kStageK / BLK, NJ, CG>;
+    g.tiles_m = (int)((g.M + L::BM - 1) / L::BM);
+    g.tiles_n = (int)((g.N + L::BN - 1) / L::BN);
+    auto kern = gemm_panel<BLK, CDT, NJ, CG>;
     static LdsOptIn opted;                         // one per kernel instantiation
     const int rc = opted.ensure((const void *)kern, L::kBytes);
     if (rc != BI8_OK) return rc;
     hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), L::kBytes, st, g);
     return bi8_launch_rc();
 }
-template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) {
-    const int64_t rows = (g.M + 127) / 128;
-    if (rows * ((g.N + 15) / 16) <= kCus) return launch_panel_as<BLK, CDT, 1>(g, st);
-    if (rows * ((g.N + 31) / 32) <= kCus) return launch_panel_as<BLK, CDT, 2>(g, st);
-    if (rows * ((g.N + 47) / 48) <= kCus) return launch_panel_as<BLK, CDT, 3>(g, st);
+template <int BLK, int CDT, int CG> int launch_panel_cg(const GemmArgs &g, hipStream_t st) {
+    const int64_t rows = (g.M + 128 / CG - 1) / (128 / CG), w = 16 * CG;       // rows of tiles; columns of a tile per subtile of a wave
+    if (rows * ((g.N + w - 1) / w) <= kCus) return launch_panel_as<BLK, CDT, 1, CG>(g, st);
+    if (rows * ((g.N + 2 * w - 1) / (2 * w)) <= kCus) return launch_panel_as<BLK, CDT, 2, CG>(g, st);
+    if (rows * ((g.N + 3 * w - 1) / (3 * w)) <= kCus) return launch_panel_as<BLK, CDT, 3, CG>(g, st);
     if constexpr (panel_max_subtiles(BLK) >= 4)
-        if (rows * ((g.N + 63) / 64) <= kCus) return launch_panel_as<BLK, CDT, 4>(g, st);
+        if (rows * ((g.N + 4 * w - 1) / (4 * w)) <= kCus) return launch_panel_as<BLK, CDT, 4, CG>(g, st);
     return BI8_ERR_UNSUPPORTED;                    // (the plan sends no other problem here)
+}
+template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) {
+    return g.M <= 64 ? launch_panel_cg<BLK, CDT, 2>(g, st) : launch_panel_cg<BLK, CDT, 1>(g, st);
 }
 
 template <int BLK, int CDT> int launch_rows(const GemmArgs &g, hipStream_t st) {

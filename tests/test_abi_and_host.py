@@ -240,7 +240,7 @@ def test_kernel_choice_by_shape():
     assert name(2048, 4096, 4096, 128) == "gemm_wide_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
     assert name(2048, 4096, 512, 64) == "gemm_wide_256x128" and name(2048, 2304, 512, 64) == "gemm_wide_256x128"
     assert name(2048, 4096, 4096, 128, 0, 1 << 21, 4096) == "gemm_tile_256x128"     # rows 2 MiB apart: beyond its 32-bit offsets
-    assert name(1500, 1500, 512, 128) == "gemm_tile_128x128" and name(48, 5000, 640, 128) == "gemm_tile_64x128"
+    assert name(1500, 1500, 512, 128) == "gemm_tile_128x128" and name(48, 5000, 640, 32) == "gemm_tile_64x128"
     # more than 64 rows, at most one tile of 128 x (16 ... 64) per CU and K up to 4096: narrow tiles, the whole K in one workgroup
     assert name(300, 500, 512, 128) == "gemm_panel" and name(128, 4096, 4096, 128) == "gemm_panel" and name(65, 64, 128, 64) == "gemm_panel"
     assert name(128, 4096, 4096, 128, 1 << 30) == "gemm_panel" and name(512, 4096, 4096, 128, 1 << 30) == "gemm_panel"
@@ -249,7 +249,11 @@ def test_kernel_choice_by_shape():
     assert name(128, 1024, 3072, 128) == "gemm_panel"                # ... up to 3072 any number does
     assert name(128, 4096, 4224, 128) == "gemm_tile_128x128"         # a longer K: the kernels that split it, given scratch memory
     assert name(512, 4096, 4096, 64) == "gemm_tile_128x128"          # block 64 stops at 48 columns: 4 x 86 tiles are more than one round
-    assert name(300, 500, 512, 32) == "gemm_tile_128x128" and name(64, 5000, 640, 128) == "gemm_tile_64x128"   # block 32, 64 rows: not its
+    assert name(300, 500, 512, 32) == "gemm_tile_128x128"            # block 32: not its
+    # 33 to 64 rows: the same on tiles of 64 rows x 32 ... 128 columns, where gemv_staged (below) does not apply or K is at most 1024
+    assert name(64, 5000, 640, 128) == "gemm_panel" and name(48, 11008, 4096, 128, 1 << 30) == "gemm_panel" and name(33, 16384, 4096, 64) == "gemm_panel"
+    assert name(48, 700, 640, 128) == "gemm_panel" and name(64, 4096, 1024, 64) == "gemm_panel" and name(64, 4096, 1152, 64) == "gemv_staged"
+    assert name(64, 33000, 768, 128) == "gemm_wide" and name(32, 11008, 768, 128) == "gemv_staged"    # too many columns for one round; 32 rows
     assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
     assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 11008, 4096, 64) == "gemv_staged"
     assert name(2, 4096, 32768, 128) == "gemv_staged"                  # 2 x 32768 codes do not fit the few-row kernel's LDS
@@ -257,8 +261,8 @@ def test_kernel_choice_by_shape():
     assert name(24, 4096, 4096, 128) == "gemv_staged" and name(32, 11008, 4096, 64, 1 << 30) == "gemv_staged"   # two groups of 16 rows
     assert name(24, 4096, 4096, 32, 1 << 30) == "gemm_tile_64x128_splitk"      # block 32 with scratch memory: the split tiles are ahead
     # 33 to 64 rows: one pass over W where one round of workgroups covers the columns and K is short, else the split tiles
-    assert name(33, 4096, 4096, 128, 1 << 30) == "gemv_staged" and name(64, 4096, 4096, 64) == "gemv_staged" and name(48, 700, 640, 128) == "gemv_staged"
-    assert name(48, 11008, 4096, 128, 1 << 30) == "gemm_tile_64x128_splitk" and name(48, 4096, 11008, 128, 1 << 30) == "gemm_tile_64x128_splitk"
+    assert name(33, 4096, 4096, 128, 1 << 30) == "gemv_staged" and name(64, 4096, 4096, 64) == "gemv_staged" and name(48, 700, 1280, 128) == "gemv_staged"
+    assert name(48, 11008, 8192, 128, 1 << 30) == "gemm_tile_64x128_splitk" and name(48, 4096, 11008, 128, 1 << 30) == "gemm_tile_64x128_splitk"
     assert name(65, 4096, 8192, 128, 1 << 30) == "gemm_tile_128x128_splitk"
     assert name(1, 128, 128 * 1024, 128) == "gemv_staged"            # any K: the scales stream through LDS with the stages
     assert name(128, 4096, 8192, 128) == "gemm_tile_128x128"         # no scratch memory: one pass

@@ -52,7 +52,7 @@ def _run(lib, A, W, sa, sw, bias, block, out, ws_bytes):
                                          # (more than 64 rows split from K = 4096 on; below that they run narrow tiles, one pass)
                                          # up to 64 rows split where the one-pass kernel would stream too much of A or take
                                          # more than one round of workgroups
-                                         (33, 128, 10240, 128), (48, 700, 7168, 128), (60, 4800, 3200, 128), (40, 700, 2560, 32),
+                                         (33, 128, 10240, 128), (48, 700, 7168, 128), (60, 4800, 4224, 128), (40, 700, 2560, 32),
                                          # 25 stages of K in pieces of 7, 7, 7, 4
                                          (200, 300, 3200, 64)])
 def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):

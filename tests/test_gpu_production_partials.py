@@ -115,10 +115,19 @@ CASES = [
     (65, 16000, 256, 128, "gemm_panel"),            # 250 tiles of 64 columns
     (512, 4090, 4096, 128, "gemm_panel"),           # 4 x 64 tiles of 64 columns, 32 stages
     (1000, 500, 384, 128, "gemm_panel"),            # 8 x 32 tiles
+    # ... and for 33 to 64 rows tiles of 64 rows, the waves as 4 x 2: 32, 64, 96 and 128 columns per tile
+    (48, 5000, 640, 64, "gemm_panel"),              # 157 tiles of 32 columns, the last 8 columns wide
+    (48, 700, 640, 64, "gemm_panel"),
+    (64, 4096, 1024, 128, "gemm_panel"),            # 128 tiles of 32 columns
+    (33, 64, 128, 128, "gemm_panel"),               # one stage, one tile of which the second wave column is empty
+    (64, 11008, 4096, 128, "gemm_panel"),           # 172 tiles of 64 columns, 32 stages
+    (50, 24000, 256, 128, "gemm_panel"),            # 250 tiles of 96 columns
+    (40, 24000, 384, 64, "gemm_panel"),             # ... two K-blocks per stage
+    (64, 32000, 384, 128, "gemm_panel"),            # 250 tiles of 128 columns
     (2304, 2304, 256, 32, "gemm_tile_128x128"),
-    (48, 5000, 640, 64, "gemm_tile_64x128"),        # more columns than one round of the one-pass kernel's workgroups covers
-    (48, 700, 640, 64, "gemv_staged"),              # four groups of 16 rows
-    (64, 4096, 1024, 128, "gemv_staged"),
+    (48, 5000, 640, 32, "gemm_tile_64x128"),
+    (48, 700, 1280, 64, "gemv_staged"),             # four groups of 16 rows
+    (64, 4096, 2048, 128, "gemv_staged"),
     (33, 1000, 2048 + 128, 128, "gemv_staged"),
     (1, 384, 512, 128, "gemv_rows"),
     (2, 1000, 4096 + 384, 128, "gemv_rows"),        # more than four runs of 1 KiB per row, the last one partial
