@@ -722,24 +722,29 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // the second way.  A workgroup streams ALL 128 rows of A (from L2) next to its few rows of W (from memory), 16 KiB of A
 // per stage of K whatever the tile's width; in exchange nothing is written twice and nothing waits for a second
 // launch, so it wins where K is short (the plan's rule and the measurements behind it: kPanelMaxStages).
-// Eight waves, each 16 rows x 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8): stacked, a tile of 128
-// rows (described here), or as 4 x 2 a tile of 64 rows x 32 * NJ columns for up to 64 rows (half the bytes of A).  A ring of
-// six to eight stage buffers, every wave loads two to four wave-instructions per stage straight into LDS (two of A
-// and its share of the rows of W and the scale rows); stages past the end of K are loaded from beyond the buffers'
-// ranges (zeros, no memory access), so a wave's count of loads in flight is the same everywhere.  ONE barrier per stage
-// and a software pipeline across it: the MFMAs of stage s are issued, then the wave waits for its loads of stage s + 1
-// and meets the others, refills the buffer that stage s - 1 has left, reads the operand fragments of stage s + 1 from
-// LDS, folds the partials of stage s - 1 while those reads and the MFMAs are under way, and reads the scales of stage
-// s + 1 into the registers that held those of stage s - 1.  Partials and scales are double-buffered in registers by
-// stage parity.
-// What a stage costs (128 x 4096 x 4096, 32 stages, 0.31 us each; timestamps inside the kernel and parts switched
-// off): without the loop's loads 0.18 us, without the fragment reads 0.24, without the MFMAs 0.23, without the fold
-// 0.26, without the barrier 0.28 -- the parts of a stage run one after the other, in all waves at once, and a stage of
-// A alone streams into LDS in 0.13 us (read-only micro-benchmark, same grid).  Measured and not kept: the fragments
-// read a stage earlier into a second set of registers (the same), the ring filled while the first stages are computed
-// instead of in front of them (the same).  Kept: a stage's loads spread over the step (3-5 %), no load issued twice.
-// The prologue's loads are all issued 1.4 us after the kernel's first instruction, and the first stage has landed
-// 0.9 us later.
+// Twelve waves.  Eight compute, each 16 rows x 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8): stacked,
+// a tile of 128 rows (described here), or as 4 x 2 a tile of 64 rows x 32 * NJ columns for up to 64 rows (half the bytes
+// of A).  Four only load: a ring of six to eight stage buffers is filled by their `buffer_load ... lds`, each loader its
+// share of a stage's wave-instructions (rows of A, rows of W, scale rows); stages past the end of K are loaded from
+// beyond the buffers' ranges (zeros, no memory access), so a loader's count of loads in flight is the same everywhere.
+// ONE barrier per stage, which all twelve waves meet: a loader arrives when its loads of stage s + 1 have landed, and
+// behind the barrier asks for the stage that goes into the buffer stage s - 1 has left; a computing wave arrives when
+// the MFMAs of stage s are issued, and behind the barrier reads the operand fragments of stage s + 1 from LDS, folds
+// the partials of stage s - 1 while those reads and the MFMAs are under way, and reads the scales of stage s + 1 into
+// the registers that held those of stage s - 1.  Partials and scales are double-buffered in registers by stage parity.
+// Why waves that only load.  In the first form of this kernel the eight computing waves loaded as well (three or four
+// wave-instructions each per stage).  Timestamps inside that kernel and parts switched off (128 x 4096 x 4096, 32
+// stages of 0.31 us each): without the loop's loads 0.18 us per stage, without the fragment reads 0.24, without the MFMAs
+// 0.23, without the fold 0.26, without the barrier 0.28 -- the parts of a stage ran one after the other, in all waves at
+// once, and a wave that offers a load to a busy path into LDS (one wave-instruction per 16-19 clocks, whoever issues it:
+// a stage of A alone streams in 0.13-0.15 us from one, two, four, eight or sixteen waves alike) stands still.  With the
+// loads in waves of their own the two run side by side: 128 x 4096 x 2048 8.1 -> 6.6 us, 512 x 1024 x 4096 12.5 -> 9.6,
+// 128 x 11008 x 4096 20.1 -> 18.5, 128 x 4096 x 4096 13.4 -> 12.6 (256 workgroups reading the same lines of A: the L2 is the
+// limit there).  The loaders' code is specialised per loader at compile time (which item of the stage is of which kind);
+// as one copy with a four-way branch per load it ran at 0.6 us per stage.  Measured and not kept in the first form: the
+// fragments read a stage earlier into a second set of registers, the ring filled while the first stages are computed
+// instead of in front of them (both the same), every wave repeating somebody else's W or scale row to keep the waves'
+// counts equal (0.26 against 0.25 us).
 // CG = column groups of the eight waves: 1 -> 8 x 1 waves, tiles of 128 rows x 16 * NJ columns; 2 -> 4 x 2 waves, tiles of
 // 64 rows x 32 * NJ columns (for up to 64 rows: half the bytes of A per stage)
 template <int NBS, int NJ, int CG> struct PanelLds {
@@ -757,8 +762,10 @@ template <int NBS, int NJ, int CG> struct PanelLds {
     static_assert(kBytes <= 160 * 1024, "LDS per CU");
 };
 
+constexpr int kPanelLoaders = 4;               // waves of a gemm_panel workgroup that only load
+constexpr int kPanelThreads = (8 + kPanelLoaders) * 64;
 template <int BLK, int CDT, int NJ, int CG = 1>
-__global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
+__global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
     static_assert(BLK == 128 || BLK == 64, "a K-block is one or two MFMAs of 64 bytes of K");
     static_assert(NJ >= 1 && NJ <= 4 && (CG == 1 || CG == 2), "16 ... 64 columns per wave, one or two waves side by side");
     constexpr int NBS = kStageK / BLK;
@@ -770,109 +777,100 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int rg = wave % RG, cg = wave / RG;                             // the wave's 16 rows, its 16 * NJ columns
-    const int r16 = lane & 15, q = lane >> 4;
     const uint32_t lds_base = bi8_lds_address(lds);
     const int tile_m = (int)blockIdx.x / g.tiles_n, tile_n = (int)blockIdx.x - tile_m * g.tiles_n;
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
     const int nst = (int)(g.K / kStageK);
+    auto wait_vm = [&](auto pending_c) {
+        constexpr int kPending = decltype(pending_c)::value;
+        static_assert(kPending < 64, "vmcnt is a 6-bit field");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
+    };
+    auto next_buf = [](int buf) { return buf + 1 == kBufs ? 0 : buf + 1; };      // the ring's buffer after `buf`
 
-    // ---- loader: wave instruction i covers tile rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which holds
-    // source chunk (lane%8) ^ ((row >> 1) & 7).  A is BM / 8 instructions per stage: i = wave and, of 128 rows, wave + 8, both
-    // of the parity of `wave`.  The rest of a stage is BN / 8 instructions of W rows and the scale rows (per K-block the
-    // row scales, 64 at a time, then the column scales, 64 at a time from the tile's first on): item e * 8 + wave of that
-    // list is wave's instruction of slot e.  The path into LDS takes one wave-instruction per 16 clocks whatever it carries
-    // (a stage of A alone: 0.13 us), so nobody loads anything twice or for show: the waves whose last slot has no item
-    // issue one load less per stage, and wait with a count of their own.
-    const int ld_row = lane >> 3;
-    const int ld_chunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
-    const uint32_t a_off = (uint32_t)((wave * 8 + ld_row) * g.lda + ld_chunk * 16), a_step = (uint32_t)(64 * g.lda);
-    const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM;
-    const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
-    // stage s into buffer `buf` (both wave-uniform); past the end of K: zeros, no memory access
-    auto issue_a0 = [&](int buf, int s) {
-        const uint32_t k_pos = s < nst ? (uint32_t)(s * kStageK) : (uint32_t)kBufOut;
-        bi8_buffer_to_lds16(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + wave * 1024, a_off, k_pos);
-    };
-    auto issue_a1 = [&](int buf, int s) {
-        const uint32_t k_pos = s < nst ? (uint32_t)(s * kStageK) : (uint32_t)kBufOut;
-        bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + (wave + 8) * 1024, a_off, k_pos, a_step);
-    };
-    auto issue_a = [&](int buf, int s) {
-        issue_a0(buf, s);
-        if constexpr (BM == 128) issue_a1(buf, s);
-    };
-    // prologue: the first stage's rows of A are on their way before anything else is set up
-    issue_a(0, 0);
-
-    const int64_t nblk = g.K / BLK, w_rows = g.N - n0 < BN ? g.N - n0 : BN;
-    const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
-    const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
-    const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
-    constexpr int kSAParts = BM / 64, kSWParts = L::kSWRow / 64, kSParts = kSAParts + kSWParts;     // scale rows of a K-block, 64 floats each
-    constexpr int kWItems = BN / 8, kItems = kWItems + kSParts * NBS, kExtra = (kItems + 7) / 8;
-    constexpr int kALoads = BM / 64;
-    constexpr int kLoadsFull = kALoads + kExtra, kLoadsLess = kALoads + kExtra - 1;       // per wave and stage: with an item in every slot / none in the last
-    const bool full = (kExtra - 1) * 8 + wave < kItems;                    // wave-uniform
-    bool x_is_w[kExtra];                           // wave-uniform: rows of W (16 bytes per lane), else a scale row (4 bytes)
-    bi8_rsrc x_rsrc[kExtra];
-    uint32_t x_off[kExtra], x_dst[kExtra], x_bufstep[kExtra], x_kstep[kExtra], x_k0[kExtra];
+    if (wave >= 8) {
+        // ---- the loading waves.  A stage is a list of wave-instructions: BM / 8 of rows of A and BN / 8 of rows of W (an
+        // instruction covers tile rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which holds source chunk
+        // (lane%8) ^ ((row >> 1) & 7)), then per K-block the row scales and the column scales, 64 floats per instruction.
+        // Loader P takes items P, P + 4, ... (all its row items have the parity of P); which item is of which kind is known
+        // at compile time, one copy of the code per loader.  Stages past the end of K are loaded from beyond the buffers'
+        // ranges (zeros, no memory access), so a loader's count of loads in flight never changes.
+        constexpr int kAItems = BM / 8, kWItems = BN / 8;
+        constexpr int kSAParts = BM / 64, kSWParts = L::kSWRow / 64, kSParts = kSAParts + kSWParts;
+        constexpr int kItems = kAItems + kWItems + kSParts * NBS, kSlots = (kItems + kPanelLoaders - 1) / kPanelLoaders;
+        static_assert(kAItems % 2 == 0 && kPanelLoaders % 2 == 0, "the swizzle term of a loader's row items does not depend on the slot");
+        static_assert((kBufs - 1) * kSlots < 64, "a loader's loads in flight fit the counter");
+        const int64_t nblk = g.K / BLK;
+        const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM, w_rows = g.N - n0 < BN ? g.N - n0 : BN;
+        const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
+        const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
+        const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
+        const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
+        const uint32_t sa_row = (uint32_t)(g.M * 4), sw_row = (uint32_t)(g.N * 4);          // bytes from one K-block's scales to the next
+        auto loader = [&](auto p_c) {
+            constexpr int P = decltype(p_c)::value;
+            constexpr int kMine = (kItems - P + kPanelLoaders - 1) / kPanelLoaders;          // this loader's items per stage
+            const int ld_row = lane >> 3;
+            const int ld_chunk = (lane & 7) ^ ((4 * (P & 1) + (lane >> 4)) & 7);
+            const uint32_t a_lane = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_lane = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
+            const uint32_t a_item = (uint32_t)(8 * g.lda), w_item = (uint32_t)(8 * g.ldw);  // from one row item to the next
+            const uint32_t s_lane = (uint32_t)(lane * 4);
+            auto issue_stage = [&](int buf, int s) {   // both wave-uniform
+                const bool real = s < nst;
+                const uint32_t k_pos = real ? (uint32_t)(s * kStageK) : (uint32_t)kBufOut;
+                const uint32_t kb0 = (uint32_t)(s * NBS);
 #pragma unroll
-    for (int e = 0; e < kExtra; ++e) {
-        const int item = e * 8 + wave;             // (a slot without an item is never issued: what is computed for it is not used)
-        const int sc = item - kWItems, kb = sc / kSParts, r = sc - kSParts * kb;         // (as a scale item)
-        x_is_w[e] = item < kWItems;
-        const bool is_sa = r < kSAParts;
-        const int part = is_sa ? r : r - kSAParts;                        // which 64 of the row's scales
-        x_rsrc[e] = x_is_w[e] ? w_rsrc : is_sa ? sa_rsrc : sw_rsrc;
-        x_off[e] = x_is_w[e] ? (uint32_t)((item * 8 + ld_row) * g.ldw + ld_chunk * 16) : (uint32_t)((part * 64 + lane) * 4);
-        x_dst[e] = lds_base + (x_is_w[e] ? L::kWReg + item * 1024 : is_sa ? L::kSAReg + (kb * BM + part * 64) * 4 : L::kSWReg + (kb * L::kSWRow + part * 64) * 4);
-        x_bufstep[e] = x_is_w[e] ? L::kWBuf : is_sa ? L::kSABuf : L::kSWBuf;
-        // where stage s of the item starts: x_k0 + s * x_kstep bytes into its buffer
-        x_kstep[e] = x_is_w[e] ? (uint32_t)kStageK : (uint32_t)(NBS * (is_sa ? g.M : g.N) * 4);
-        x_k0[e] = x_is_w[e] ? 0u : (uint32_t)(kb * (is_sa ? g.M : g.N) * 4);
+                for (int e = 0; e < kMine; ++e) {
+                    constexpr int kA = kAItems, kW = kWItems;
+                    const int item = e * kPanelLoaders + P;            // a constant after unrolling
+                    if (item < kA) {
+                        bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + item * 1024, a_lane, k_pos, (uint32_t)item * a_item);
+                    } else if (item < kA + kW) {
+                        bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (item - kA) * 1024, w_lane, k_pos, (uint32_t)(item - kA) * w_item);
+                    } else {
+                        const int sc = item - kA - kW, kb = sc / kSParts, r = sc % kSParts;
+                        if (r < kSAParts) {
+                            const uint32_t pos = real ? (kb0 + kb) * sa_row + r * 256 : (uint32_t)kBufOut;
+                            bi8_buffer_to_lds4(sa_rsrc, lds_base + L::kSAReg + buf * L::kSABuf + (kb * BM + r * 64) * 4, s_lane, pos);
+                        } else {
+                            const uint32_t pos = real ? (kb0 + kb) * sw_row + (r - kSAParts) * 256 : (uint32_t)kBufOut;
+                            bi8_buffer_to_lds4(sw_rsrc, lds_base + L::kSWReg + buf * L::kSWBuf + (kb * L::kSWRow + (r - kSAParts) * 64) * 4, s_lane, pos);
+                        }
+                    }
+                }
+            };
+#pragma unroll
+            for (int s = 0; s < kBufs - 1; ++s) issue_stage(s, s);
+            wait_vm(std::integral_constant<int, (kBufs - 2) * kMine>{});                 // stage 0 has landed
+            __syncthreads();
+            int fill = kBufs - 1;
+            for (int s = 0; s < nst; ++s) {
+                wait_vm(std::integral_constant<int, (kBufs - 3) * kMine>{});             // stage s + 1 has landed
+                __syncthreads();                   // ... for every loader: published; and the computing waves have left stage s - 1
+                issue_stage(fill, s + kBufs - 1);
+                fill = next_buf(fill);
+            }
+            wait_vm(std::integral_constant<int, 0>{});     // (the loads past the end of K) nothing may still be writing LDS when the wave ends
+        };
+        static_assert(kPanelLoaders == 4, "one copy of the loader per loading wave");
+        if (wave == 8) loader(std::integral_constant<int, 0>{});
+        else if (wave == 9) loader(std::integral_constant<int, 1>{});
+        else if (wave == 10) loader(std::integral_constant<int, 2>{});
+        else loader(std::integral_constant<int, 3>{});
+        return;
     }
-    auto issue_rest = [&](int buf, int s) {
-#pragma unroll
-        for (int e = 0; e < kExtra; ++e) {
-            if (e == kExtra - 1 && !full) break;
-            const uint32_t pos = s < nst ? x_k0[e] + (uint32_t)s * x_kstep[e] : (uint32_t)kBufOut;
-            if (x_is_w[e]) bi8_buffer_to_lds16(x_rsrc[e], x_dst[e] + buf * x_bufstep[e], x_off[e], pos);
-            else bi8_buffer_to_lds4(x_rsrc[e], x_dst[e] + buf * x_bufstep[e], x_off[e], pos);
-        }
-    };
-    auto issue_stage = [&](int buf, int s) {
-        issue_a(buf, s);
-        issue_rest(buf, s);
-    };
-    // ... then the rest of it and the stages for all buffers but one
-    issue_rest(0, 0);
-#pragma unroll
-    for (int s = 1; s < kBufs - 1; ++s) issue_stage(s, s);
-    // the ring's buffer after `buf`
-    auto next_buf = [](int buf) { return buf + 1 == kBufs ? 0 : buf + 1; };
 
-
-    // ---- operand fragments: lane -> row r16 of a 16-row subtile, 16-byte chunk 4*kb + q of the stage's eight, stored
-    // at chunk position (4*kb + q) ^ (r16 >> 1): the address of kb = 1 is that of kb = 0 with bit 6 flipped
+    // ---- the computing waves: `wave` = row group rg (16 rows), column group cg (16 * NJ columns)
+    const int rg = wave % RG, cg = wave / RG;
+    const int r16 = lane & 15, q = lane >> 4;
+    // operand fragments: lane -> row r16 of a 16-row subtile, 16-byte chunk 4*kb + q of the stage's eight, stored at chunk
+    // position (4*kb + q) ^ (r16 >> 1): the address of kb = 1 is that of kb = 0 with bit 6 flipped
     int a_base = L::kAReg + (rg * 16 + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
     int w_base = L::kWReg + (cg * 16 * NJ + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
     // a subtile's outputs: lane -> column r16, rows 4q .. 4q+3
     int sa_base = L::kSAReg + (rg * 16 + 4 * q) * 4;
     int sw_base = L::kSWReg + (cg * 16 * NJ + r16) * 4;
     asm volatile("" : "+v"(a_base), "+v"(w_base), "+v"(sa_base), "+v"(sw_base));
-
-    auto wait_vm = [&](auto pending_c) {
-        constexpr int kPending = decltype(pending_c)::value;
-        static_assert(kPending < 64, "vmcnt is a 6-bit field");
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
-    };
-    // until at most S stages' worth of this wave's loads are outstanding
-    auto wait_stages = [&](auto stages_c) {
-        constexpr int S = decltype(stages_c)::value;
-        if (full) wait_vm(std::integral_constant<int, S * kLoadsFull>{});
-        else wait_vm(std::integral_constant<int, S * kLoadsLess>{});
-    };
     constexpr int kMagicBits = 0x4B400000;        // bit pattern of 1.5 * 2^23
     const bi8_v4i magic = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
 
@@ -914,6 +912,7 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
                 c[P][blk][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[kb], B[j][kb], first ? magic : c[P][blk][j], 0, 0, 0);
             }
     };
+    // a stage's partials into the accumulators: per K-block and subtile four products, then four accumulations
     auto fold = [&](auto par_c) {
         constexpr int P = decltype(par_c)::value;
 #pragma unroll
@@ -929,48 +928,39 @@ __global__ __launch_bounds__(512) void gemm_panel(const GemmArgs g) {
                 for (int r = 0; r < 4; ++r) acc[j][r] = __builtin_fmaf(t[r], sx[P][kb][r], acc[j][r]);
             }
     };
-    // stage s (parity P, operands in A and B, in buffer `buf`): MFMAs, publish stage s + 1, refill the buffer that stage
-    // s - 1 has left, read the operands of stage s + 1, fold stage s - 1, read the scales of stage s + 1
-    int buf = 0, fill = kBufs - 1;                 // the buffer of the stage being computed; the one the next loads go to
-    auto step = [&](int s, auto par_c, bool fold_prev) {
+    // stage s (parity P, its operands in A and B): MFMAs; the barrier that publishes stage s + 1; its operands from LDS; the
+    // fold of stage s - 1; the scales of stage s + 1 into the registers that held those of stage s - 1
+    int buf = 0;
+    auto step = [&](auto par_c, bool fold_prev) {
         constexpr int P = decltype(par_c)::value;
         using Q = std::integral_constant<int, 1 - P>;
         mfmas(par_c);
         __builtin_amdgcn_sched_barrier(0);
-        wait_stages(std::integral_constant<int, kBufs - 3>{});                   // stage s + 1 has landed
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        // (the stage's loads are spread over the step: the path into LDS takes them one per 16 clocks, and a wave that
-        // offers three at once waits for the other waves' to drain)
         buf = next_buf(buf);
-        issue_a0(fill, s + kBufs - 1);
         read_frags(buf);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (BM == 128) issue_a1(fill, s + kBufs - 1);
         if (fold_prev) fold(Q{});
         __builtin_amdgcn_sched_barrier(0);
-        issue_rest(fill, s + kBufs - 1);
         read_scales(buf, Q{});
-        fill = next_buf(fill);
     };
 
-    wait_stages(std::integral_constant<int, kBufs - 2>{});                       // stage 0 has landed
-    __syncthreads();
+    __syncthreads();                               // stage 0 is published
     read_frags(0);
     read_scales(0, std::integral_constant<int, 0>{});
-    step(0, std::integral_constant<int, 0>{}, false);
+    step(std::integral_constant<int, 0>{}, false);
     int s = 1;
     for (; s + 1 < nst; s += 2) {
-        step(s, std::integral_constant<int, 1>{}, true);
-        step(s + 1, std::integral_constant<int, 0>{}, true);
+        step(std::integral_constant<int, 1>{}, true);
+        step(std::integral_constant<int, 0>{}, true);
     }
     if (s < nst) {                                 // an even number of stages: one more, of odd parity
-        step(s, std::integral_constant<int, 1>{}, true);
+        step(std::integral_constant<int, 1>{}, true);
         fold(std::integral_constant<int, 1>{});
     } else {
         fold(std::integral_constant<int, 0>{});
     }
-    wait_vm(std::integral_constant<int, 0>{});     // (the loads past the end of K) nothing may still be writing LDS when the wave ends
 
     const float div = (float)(1.0 / (127.0 * 127.0));
     const bool has_bias = g.bias != nullptr;
@@ -2597,17 +2587,15 @@ struct GemmPlan {
 // mostly empty round and the 256x256 kernel wins (1284 against 978 TOP/s at 2304x4096x4096, 144 tiles).
 // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
 constexpr int64_t kWideMinTiles = 129;
-// gemm_panel: more than 64 rows, at most one tile of 128 x (16 ... 64) per CU, and a short K: every workgroup streams all
-// 128 rows of A, so its time grows with K faster than that of the kernels that split the contraction.  Measured against
-// what ran these shapes before (one-pass or split 64x128 / 128x128 tiles), W from HBM, block 128, us at K = 768 / 2048 /
-// 4096 / 8192: 128 x 768 8.4 -> 5.0, 10.8 -> 7.8, 11.5 -> 11.8, 13.5 -> 20.1; 128 x 4096 8.6 -> 5.4, 12.8 -> 8.2, 14.9 -> 13.8,
-// 22.1 -> 24.0; 128 x 11008 9.2 -> 7.0, 19.3 -> 11.8, 22.5 -> 19.6, 35.3 -> 33.7; 512 x 2048 8.6 -> 5.9, 15.1 -> 9.1, 22.3 -> 14.2,
-// 25.4 -> 27.2; 1024 x 1024 8.6 -> 5.8, 15.2 -> 9.1, 22.4 -> 14.5, 25.0 -> 25.5; block 64, 128 x 4096 9.6 -> 5.8, 14.8 -> 9.1,
-// 16.6 -> 15.3.  At K = 4096 it needs enough tiles to win (128 x 1024: 11.5 -> 11.9).
+// gemm_panel: more than 32 rows, at most one tile of 128 x (16 ... 64) -- up to 64 rows: 64 x (32 ... 128) -- per CU, and a
+// short K: every workgroup streams all rows of A, so its time grows with K faster than that of the kernels that split the
+// contraction.  Measured against what ran these shapes before (one-pass or split 64x128 / 128x128 tiles), W from HBM,
+// block 128, us at K = 768 / 2048 / 4096 / 8192: 128 x 768 8.4 -> 4.3, 10.8 -> 6.0, 11.0 -> 8.7, 12.7 -> 13.8; 128 x 4096
+// 8.6 -> 4.9, 12.8 -> 6.6, 14.9 -> 12.3, 21.7 -> 21.8; 128 x 11008 9.2 -> 6.5, 19.3 -> 10.9, 22.5 -> 18.2, 35.0 -> 35.2;
+// 512 x 2048 8.6 -> 5.3, 15.1 -> 8.0, 22.3 -> 12.0, 24.7 -> 23.6; 1024 x 1024 (512 x 1024: the same tiles) 8.6 -> 4.7,
+// 15.2 -> 6.5, 22.4 -> 9.6; block 64, 128 x 4096 (first form of the kernel) 9.6 -> 5.8, 14.8 -> 9.1, 16.6 -> 15.3.
 constexpr int64_t kPanelMinRows = 64;          // more rows: tiles of 128 rows; 33 ... 64: tiles of 64 rows
-constexpr int64_t kPanelMaxStages = 32;        // K <= 4096 ...
-constexpr int64_t kPanelSureStages = 24;       // ... beyond 3072 only with at least kPanelMinTiles tiles of 16 columns
-constexpr int64_t kPanelMinTiles = 128;
+constexpr int64_t kPanelMaxStages = 32;        // K <= 4096
 constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024
 // the widest tile, in 16-column subtiles (block 64 at 64 columns needs more registers than a wave has)
 constexpr int panel_max_subtiles(int block) { return block == 64 ? 3 : 4; }
@@ -2705,7 +2693,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
         if (M > kPanelMinRows && (block == 64 || block == 128) && (K / block + 1) * max_mn * 4 < kBufOut) {
             const int64_t rows = (M + 127) / 128, widest = 16 * panel_max_subtiles(block), nst = K / kStageK;
             const bool one_round = rows * ((N + widest - 1) / widest) <= kCus;
-            if (one_round && (nst <= kPanelSureStages || (nst <= kPanelMaxStages && rows * ((N + 15) / 16) >= kPanelMinTiles))) {
+            if (one_round && nst <= kPanelMaxStages) {
                 p.kernel = kKPanel;
                 return p;
             }
@@ -2808,7 +2796,7 @@ template <int BLK, int CDT, int NJ, int CG> int launch_panel_as(GemmArgs g, hipS
     static LdsOptIn opted;                         // one per kernel instantiation
     const int rc = opted.ensure((const void *)kern, L::kBytes);
     if (rc != BI8_OK) return rc;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), L::kBytes, st, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(kPanelThreads), L::kBytes, st, g);
     return bi8_launch_rc();
 }
 template <int BLK, int CDT, int CG> int launch_panel_cg(const GemmArgs &g, hipStream_t st) {

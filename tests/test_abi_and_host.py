@@ -245,8 +245,7 @@ def test_kernel_choice_by_shape():
     assert name(300, 500, 512, 128) == "gemm_panel" and name(128, 4096, 4096, 128) == "gemm_panel" and name(65, 64, 128, 64) == "gemm_panel"
     assert name(128, 4096, 4096, 128, 1 << 30) == "gemm_panel" and name(512, 4096, 4096, 128, 1 << 30) == "gemm_panel"
     assert name(128, 11008, 4096, 64, 1 << 30) == "gemm_panel" and name(1024, 2048, 4096, 128) == "gemm_panel"
-    assert name(128, 1024, 4096, 128) == "gemm_tile_128x128"         # K = 4096 needs 128 tiles of 16 columns to pay ...
-    assert name(128, 1024, 3072, 128) == "gemm_panel"                # ... up to 3072 any number does
+    assert name(128, 1024, 4096, 128) == "gemm_panel" and name(128, 16, 4096, 128, 1 << 30) == "gemm_panel"      # however few the tiles
     assert name(128, 4096, 4224, 128) == "gemm_tile_128x128"         # a longer K: the kernels that split it, given scratch memory
     assert name(512, 4096, 4096, 64) == "gemm_tile_128x128"          # block 64 stops at 48 columns: 4 x 86 tiles are more than one round
     assert name(300, 500, 512, 32) == "gemm_tile_128x128"            # block 32: not its

@@ -53,8 +53,8 @@ def _run(lib, A, W, sa, sw, bias, block, out, ws_bytes):
                                          # up to 64 rows split where the one-pass kernel would stream too much of A or take
                                          # more than one round of workgroups
                                          (33, 128, 10240, 128), (48, 700, 7168, 128), (60, 4800, 4224, 128), (40, 700, 2560, 32),
-                                         # 25 stages of K in pieces of 7, 7, 7, 4
-                                         (200, 300, 3200, 64)])
+                                         # 35 stages of K in pieces of 9, 9, 9, 8
+                                         (200, 300, 4480, 64)])
 def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
     want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
@@ -140,7 +140,7 @@ def test_no_workspace_wanted_where_nothing_would_split(lib):
 def test_operator_uses_the_split(lib):
     """through the Python operator (which allocates the workspace): same tolerance, and deterministic from call to call"""
     import blockwise_int8_linear_amd as pkg
-    M, N, K, block = 128, 1024, 4096, 128
+    M, N, K, block = 128, 1024, 8192, 128
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=9)
     cfg = pkg.block_linear_config
     old = (cfg.GROUP_SIZE, cfg.INPUT_OUTPUT_TORCH_TYPE)

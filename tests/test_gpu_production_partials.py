@@ -146,7 +146,7 @@ CASES = [
     (24, 500, 640, 32, "gemm_skinny"),              # block 32, five stages of K: nothing to split
     (24, 500, 2048, 32, "gemm_tile_64x128_splitk"),
     (16, 300, 1024, 32, "gemm_skinny"),
-    (128, 1024, 4096, 128, "gemm_tile_64x128_splitk"),
+    (128, 1024, 8192, 128, "gemm_tile_64x128_splitk"),
     (512, 4096, 4096, 64, "gemm_tile_128x128_splitk"),
 ]
 
