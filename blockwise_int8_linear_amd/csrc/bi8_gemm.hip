@@ -764,8 +764,11 @@ template <int NBS, int NJ, int CG> struct PanelLds {
 
 constexpr int kPanelLoaders = 4;               // waves of a gemm_panel workgroup that only load
 constexpr int kPanelThreads = (8 + kPanelLoaders) * 64;
-template <int BLK, int CDT, int NJ, int CG = 1>
+// SPLIT: K in gridDim.y pieces of GemmArgs::split_stages stages; workgroup (t, y) writes the fp32 sums of its piece, scaled,
+// without bias, to slab t * gridDim.y + y of the workspace ([BM][BN] each), and splitk_reduce adds a tile's slabs.
+template <int BLK, int CDT, int NJ, int CG = 1, bool SPLIT = false>
 __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
+    static_assert(!SPLIT || CDT == BI8_F32, "the slabs are fp32 sums");
     static_assert(BLK == 128 || BLK == 64, "a K-block is one or two MFMAs of 64 bytes of K");
     static_assert(NJ >= 1 && NJ <= 4 && (CG == 1 || CG == 2), "16 ... 64 columns per wave, one or two waves side by side");
     constexpr int NBS = kStageK / BLK;
@@ -780,7 +783,9 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
     const uint32_t lds_base = bi8_lds_address(lds);
     const int tile_m = (int)blockIdx.x / g.tiles_n, tile_n = (int)blockIdx.x - tile_m * g.tiles_n;
     const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
-    const int nst = (int)(g.K / kStageK);
+    const int stage_lo = SPLIT ? (int)blockIdx.y * g.split_stages : 0;          // this workgroup's first stage of K, and how many
+    const int nst = SPLIT ? ((int)(g.K / kStageK) - stage_lo < g.split_stages ? (int)(g.K / kStageK) - stage_lo : g.split_stages)
+                          : (int)(g.K / kStageK);
     auto wait_vm = [&](auto pending_c) {
         constexpr int kPending = decltype(pending_c)::value;
         static_assert(kPending < 64, "vmcnt is a 6-bit field");
@@ -817,8 +822,8 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
             const uint32_t s_lane = (uint32_t)(lane * 4);
             auto issue_stage = [&](int buf, int s) {   // both wave-uniform
                 const bool real = s < nst;
-                const uint32_t k_pos = real ? (uint32_t)(s * kStageK) : (uint32_t)kBufOut;
-                const uint32_t kb0 = (uint32_t)(s * NBS);
+                const uint32_t k_pos = real ? (uint32_t)((stage_lo + s) * kStageK) : (uint32_t)kBufOut;
+                const uint32_t kb0 = (uint32_t)((stage_lo + s) * NBS);
 #pragma unroll
                 for (int e = 0; e < kMine; ++e) {
                     constexpr int kA = kAItems, kW = kWItems;
@@ -963,7 +968,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
     }
 
     const float div = (float)(1.0 / (127.0 * 127.0));
-    const bool has_bias = g.bias != nullptr;
+    const bool has_bias = !SPLIT && g.bias != nullptr;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const int64_t n = n0 + cg * 16 * NJ + j * 16 + r16;
@@ -972,7 +977,12 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int64_t m = m0 + rg * 16 + 4 * q + r;
-            if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[j][r] * div, has_bias, bias);
+            if constexpr (SPLIT) {
+                float *slab = g.ws + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * (BM * BN);
+                if (n_ok && m < g.M) slab_store(slab + (rg * 16 + 4 * q + r) * BN + cg * 16 * NJ + j * 16 + r16, acc[j][r] * div);
+            } else {
+                if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[j][r] * div, has_bias, bias);
+            }
         }
     }
 }
@@ -2356,13 +2366,14 @@ __global__ __launch_bounds__(256) void gemm_generic(const GemmArgs g, int block)
 }
 
 // Sum of a tile's slabs in ascending workgroup order (deterministic), then the cast and the bias of the one-pass
-// epilogue.  One workgroup = 8 rows of one tile, a thread = four consecutive columns; a tile has at most kSplitMax slabs,
+// epilogue.  One workgroup = 8 rows of one tile (16 or 32 of a tile of 64 or 32 columns), a thread = four consecutive columns; a tile has at most kSplitMax slabs,
 // all loaded before the first addition.  With split_per_tile workgroups per tile, tile t's slabs are
 // t * split_per_tile ... ; with runs, the workgroups whose runs touch tile t are floor(t * nst / S) ...
 // floor(((t + 1) * nst - 1) / S), and workgroup w's slab for it is ws[w + t].
 template <int CDT, int BM, int BN>
 __global__ __launch_bounds__(256) void splitk_reduce(const GemmArgs g) {
-    static_assert(BN == 128 && BM % 8 == 0, "32 threads x 4 columns per row, 8 rows per workgroup");
+    constexpr int kCols4 = BN / 4, kRowsPerGroup = 256 / kCols4;     // BN = 128: 32 threads per row, 8 rows per workgroup; 64: 16 and 16; 32: 8 and 32
+    static_assert((BN == 128 || BN == 64 || BN == 32) && BM % kRowsPerGroup == 0, "whole rows per workgroup (grid y = BM / rows per workgroup)");
     const int t = blockIdx.x, tile_m = t / g.tiles_n, tile_n = t - tile_m * g.tiles_n;
     const int nst = (int)(g.K / kStageK), S = g.split_stages;
     int first, count;
@@ -2374,7 +2385,7 @@ __global__ __launch_bounds__(256) void splitk_reduce(const GemmArgs g) {
         first = w0 + t;
         count = w1 - w0 + 1;
     }
-    const int i = blockIdx.y * 8 + (threadIdx.x >> 5), j = (threadIdx.x & 31) * 4;
+    const int i = blockIdx.y * kRowsPerGroup + (int)threadIdx.x / kCols4, j = ((int)threadIdx.x % kCols4) * 4;
     const int64_t m = (int64_t)(tile_m + g.tile_m0) * BM + i;
     if (m >= g.M) return;
     const float *src = g.ws + (int64_t)first * (BM * BN) + i * BN + j;
@@ -2567,10 +2578,10 @@ template <int CDT, bool PARTIALS> int launch_generic(GemmArgs g, int block, hipS
 
 // ---- which kernel runs a problem ------------------------------------------------------------------------------------
 // One rule, used by the launcher, by bi8_gemm_workspace_bytes and by bi8_gemm_kernel_name.
-enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKWideHalf, kKSplitWideHalf, kKPanel };
+enum GemmKernel { kKGeneric = 0, kKGemv, kKSkinny, kKWide, kKTile256x128, kKTile128x128, kKTile64x128, kKSplit128x128, kKSplit64x128, kKRows, kKWideHalf, kKSplitWideHalf, kKPanel, kKSplitPanel };
 static const char *const kGemmKernelNames[] = {"gemm_generic", "gemv_staged", "gemm_skinny", "gemm_wide", "gemm_tile_256x128",
                                                 "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk",
-                                                "gemm_tile_64x128_splitk", "gemv_rows", "gemm_wide_256x128", "gemm_wide_256x128_splitk", "gemm_panel"};
+                                                "gemm_tile_64x128_splitk", "gemv_rows", "gemm_wide_256x128", "gemm_wide_256x128_splitk", "gemm_panel", "gemm_panel_splitk"};
 struct GemmPlan {
     int kernel;
     int splits, split_stages;      // of the split kernels: workgroups of the split grid and 128-byte stages of K per workgroup,
@@ -2596,6 +2607,8 @@ constexpr int64_t kWideMinTiles = 129;
 // 15.2 -> 6.5, 22.4 -> 9.6; block 64, 128 x 4096 (first form of the kernel) 9.6 -> 5.8, 14.8 -> 9.1, 16.6 -> 15.3.
 constexpr int64_t kPanelMinRows = 64;          // more rows: tiles of 128 rows; 33 ... 64: tiles of 64 rows
 constexpr int64_t kPanelMaxStages = 32;        // K <= 4096
+constexpr int64_t kPanelSplitMinStages = 8;    // the split form: the least stages of K per piece ...
+constexpr int64_t kPanelSplitMaxStages = 96;   // ... and the longest K (12288)
 constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024
 // the widest tile, in 16-column subtiles (block 64 at 64 columns needs more registers than a wave has)
 constexpr int panel_max_subtiles(int block) { return block == 64 ? 3 : 4; }
@@ -2627,6 +2640,30 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     // few tiles and scratch memory: split K over the workgroups, then sum the slabs
     auto try_split = [&]() {
         if (partials || ws_bytes <= 0) return false;
+        // 65 ... 128 rows and K up to 12288: gemm_panel on pieces of K, tiles of 128 rows x 64 columns (block 64: 32).  Measured
+        // against the split 64x128 / 128x128 tiles, block 128, W from HBM, us at K = 8192 / 11008 / 16384: 128 x 768 12.9 -> 11.1,
+        // 13.7 -> 11.8, 17.4 -> 14.1; 128 x 4096 21.7 -> 18.8, 24.8 -> 20.1, 25.8 -> 31.2; 128 x 8192 28.4 -> 26.3, 35.4 -> 32.9,
+        // 43.7 -> 46.7; 512 x 768 18.7 -> 15.1, 19.9 -> 20.3; 512 x 2048 25.8 -> 23.6, 28.5 -> 28.8; 1024 x 768 21.8 -> 23.0
+        // (256 workgroups that each stream all of A: the longer the pieces and the more rows of tiles, the less it pays).
+        if (block != 32 && M > kPanelMinRows && M <= 128 && K / kStageK <= kPanelSplitMaxStages && !rest_of_cut && (K / block + 1) * max_mn * 4 < kBufOut) {
+            const int64_t bn = block == 64 ? 32 : 64, t = ((M + 127) / 128) * ((N + bn - 1) / bn), nst = K / kStageK;
+            int64_t per = t > 0 && t <= kCus / 2 ? kCus / t : 0;
+            if (per > kSplitMax) per = kSplitMax;
+            if (per > nst / kPanelSplitMinStages) per = nst / kPanelSplitMinStages;
+            if (per >= 2) {
+                const int64_t stages = (nst + per - 1) / per;
+                per = (nst + stages - 1) / stages;
+                const int64_t need = t * per * 128 * bn * 4;
+                if (per >= 2 && need <= ws_bytes) {
+                    p.kernel = kKSplitPanel;
+                    p.splits = (int)(t * per);
+                    p.split_stages = (int)stages;
+                    p.split_per_tile = (int)per;
+                    p.ws_need = need;
+                    return true;
+                }
+            }
+        }
         // 256x128 tiles on gemm_wide's loop, split evenly, where that puts most of the CUs to work
         if (block != 32 && M > 128 && wide_addressable(M, N, K, lda, ldw, block)) {
             const int64_t t = ((M + 255) / 256) * ((N + 127) / 128), nst = K / kStageK;
@@ -2808,6 +2845,24 @@ template <int BLK, int CDT, int CG> int launch_panel_cg(const GemmArgs &g, hipSt
         if (rows * ((g.N + 4 * w - 1) / (4 * w)) <= kCus) return launch_panel_as<BLK, CDT, 4, CG>(g, st);
     return BI8_ERR_UNSUPPORTED;                    // (the plan sends no other problem here)
 }
+// the split form: tiles of 128 rows x 64 columns (block 64: 32), split_per_tile pieces of split_stages stages each, then the sum
+template <int BLK, int CDT> int launch_panel_split(GemmArgs g, hipStream_t st) {
+    constexpr int NJ = BLK == 64 ? 2 : 4;
+    using L = PanelLds<kStageK / BLK, NJ, 1>;
+    g.tiles_m = (int)((g.M + L::BM - 1) / L::BM);
+    g.tiles_n = (int)((g.N + L::BN - 1) / L::BN);
+    g.tile_m0 = g.tile_n0 = 0;
+    if (g.split_per_tile < 2 || g.split_per_tile > kSplitMax || (int64_t)g.tiles_m * g.tiles_n * g.split_per_tile > 2 * kCus) return BI8_ERR_UNSUPPORTED;
+    auto kern = gemm_panel<BLK, BI8_F32, NJ, 1, true>;
+    static LdsOptIn opted;                         // one per kernel instantiation
+    const int rc = opted.ensure((const void *)kern, L::kBytes);
+    if (rc != BI8_OK) return rc;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), (unsigned)g.split_per_tile), dim3(kPanelThreads), L::kBytes, st, g);
+    const int rc_launch = bi8_launch_rc();
+    if (rc_launch != BI8_OK) return rc_launch;
+    hipLaunchKernelGGL((splitk_reduce<CDT, L::BM, L::BN>), dim3((unsigned)(g.tiles_m * g.tiles_n), L::BM / (256 / (L::BN / 4))), dim3(256), 0, st, g);
+    return bi8_launch_rc();
+}
 template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) {
     return g.M <= 64 ? launch_panel_cg<BLK, CDT, 2>(g, st) : launch_panel_cg<BLK, CDT, 1>(g, st);
 }
@@ -2876,6 +2931,16 @@ int launch_kernel(const GemmArgs &g, int kernel, int splits, int split_stages, i
             if constexpr (BLK != 32) {
                 if (!whole) return BI8_ERR_UNSUPPORTED;
                 return launch_panel<BLK, CDT>(g, st);
+            }
+            break;
+        case kKSplitPanel:
+            if constexpr (BLK != 32) {
+                if (!whole) return BI8_ERR_UNSUPPORTED;
+                GemmArgs gs = g;
+                gs.splits = splits;
+                gs.split_stages = split_stages;
+                gs.split_per_tile = split_per_tile;
+                return launch_panel_split<BLK, CDT>(gs, st);
             }
             break;
         case kKSplit128x128:

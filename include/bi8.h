@@ -164,7 +164,7 @@ int bi8_gemm_nt_dequant_static(const int8_t *A, const int8_t *W, const float *sA
 /*
  * Name of the kernel family that bi8_gemm_nt_dequant_ws runs on a problem with 16-byte aligned operands and
  * `workspace_bytes` of scratch memory ("gemm_wide", "gemm_wide_256x128", "gemm_wide_256x128_splitk", "gemm_tile_256x128",
- * "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk", "gemm_tile_64x128_splitk", "gemm_panel", "gemv_rows",
+ * "gemm_tile_128x128", "gemm_tile_64x128", "gemm_tile_128x128_splitk", "gemm_tile_64x128_splitk", "gemm_panel", "gemm_panel_splitk", "gemv_rows",
  * "gemv_staged", "gemm_skinny", "gemm_generic"; "gemm_wide+<tile kernel>" for a problem that runs as two launches, the 256x256 kernel on the leading
  * rows or columns that fill whole rounds of workgroups and a tile kernel on the rest; "none" for an empty problem).
  * Static string.  The reference picks its kernel configuration with Triton's autotuner

@@ -58,7 +58,7 @@ def _run(lib, A, W, sa, sw, bias, block, out, ws_bytes):
 def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
     want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
-    assert 0 < want <= lib.bi8_static_scratch_bytes() and want % (64 * 128 * 4) == 0     # fp32 slabs of one tile (64x128 or 128x128) each
+    assert 0 < want <= lib.bi8_static_scratch_bytes() and want % (128 * 32 * 4) == 0     # fp32 slabs of one tile (128x32 ... 128x128) each
     Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
     split = _run(lib, Ad, Wd, sad, swd, None, block, out, want)
     one = _run(lib, Ad, Wd, sad, swd, None, block, out, 0)

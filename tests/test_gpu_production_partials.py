@@ -146,7 +146,11 @@ CASES = [
     (24, 500, 640, 32, "gemm_skinny"),              # block 32, five stages of K: nothing to split
     (24, 500, 2048, 32, "gemm_tile_64x128_splitk"),
     (16, 300, 1024, 32, "gemm_skinny"),
-    (128, 1024, 8192, 128, "gemm_tile_64x128_splitk"),
+    (128, 1024, 16384, 128, "gemm_tile_64x128_splitk"),
+    # narrow tiles on pieces of K (65 to 128 rows, K from 4224 to 12288): 128 x 64 tiles, at block 64 128 x 32
+    (128, 1024, 8192, 128, "gemm_panel_splitk"),    # 16 tiles, eight pieces of eight stages
+    (65, 4100, 4224, 128, "gemm_panel_splitk"),     # 65 tiles (the last 4 columns wide), three pieces of 11 stages
+    (100, 300, 5120, 64, "gemm_panel_splitk"),      # ten tiles of 32 columns, five pieces of eight stages, two K-blocks per stage
     (512, 4096, 4096, 64, "gemm_tile_128x128_splitk"),
 ]
 
