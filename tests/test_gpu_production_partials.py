@@ -115,6 +115,7 @@ CASES = [
     (65, 16000, 256, 128, "gemm_panel"),            # 250 tiles of 64 columns
     (512, 4090, 4096, 128, "gemm_panel"),           # 4 x 64 tiles of 64 columns, 32 stages
     (1000, 500, 384, 128, "gemm_panel"),            # 8 x 32 tiles
+    (30000, 16, 256, 128, "gemm_panel"),            # 235 x 1 tiles: tall and one tile wide
     # ... and for 33 to 64 rows tiles of 64 rows, the waves as 4 x 2: 32, 64, 96 and 128 columns per tile
     (48, 5000, 640, 64, "gemm_panel"),              # 157 tiles of 32 columns, the last 8 columns wide
     (48, 700, 640, 64, "gemm_panel"),
