@@ -2638,6 +2638,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                          (block == 32 || block == 64 || block == 128);
     if (!tile_ok) return p;
     // few tiles and scratch memory: split K over the workgroups, then sum the slabs
+    bool panel_if_no_split = false;                // gemm_panel's tiles would give one round, but K is beyond what it is given outright
     auto try_split = [&]() {
         if (partials || ws_bytes <= 0) return false;
         // 65 ... 128 rows and K up to 12288: gemm_panel on pieces of K, tiles of 128 rows x 64 columns (block 64: 32).  Measured
@@ -2719,6 +2720,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                 p.kernel = kKPanel;
                 return p;
             }
+            panel_if_no_split = (N + widest - 1) / widest <= kCus && !staged_band;
         }
         const bool staged_rows = M <= kStagedMaxRows || staged_band;
         if (staged_rows && (block == 64 || block == 128) && (K / block + 16) * N * 4 < 0x3fffffffLL && 16 * ldw + K < 0x3fffffffLL &&
@@ -2734,6 +2736,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                 p.kernel = kKPanel;
                 return p;
             }
+            panel_if_no_split = one_round;
         }
         if (M <= 32) {
             // (block 32) with scratch memory the split 64x128 tiles are ahead of the kernel that gathers its operands (measured
@@ -2789,6 +2792,13 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     // small grids: one workgroup per CU at best, so the tile is spread over as many waves as its shape allows
     // (measured 25-37 % faster than 2x2 waves of 64x64 at M = 96 ... 1024)
     if (try_split()) return p;
+    // a long K and nothing to split it with (no scratch memory, or too little): one round of narrow tiles is still ahead of a
+    // few 128x128 tiles (measured without scratch memory, block 128, us, K = 8192 / 16384: 128 x 768 45.0 -> 13.9, 88.6 -> 35.9;
+    // 128 x 11008 48.7 -> 32.2, 90.3 -> 57.6; 512 x 4096 49.7 -> 34.9, 88.5 -> 63.2; 1024 x 256 at K = 32768 167 -> 53)
+    if (panel_if_no_split) {
+        p.kernel = kKPanel;
+        return p;
+    }
     // (64x128 tiles for problems of 129-255 tiles of 128x128 measured 5-10 % slower than the half-empty 128x128 grid)
     p.kernel = M > 64 ? kKTile128x128 : kKTile64x128;
     return p;

@@ -246,7 +246,7 @@ def test_kernel_choice_by_shape():
     assert name(128, 4096, 4096, 128, 1 << 30) == "gemm_panel" and name(512, 4096, 4096, 128, 1 << 30) == "gemm_panel"
     assert name(128, 11008, 4096, 64, 1 << 30) == "gemm_panel" and name(1024, 2048, 4096, 128) == "gemm_panel"
     assert name(128, 1024, 4096, 128) == "gemm_panel" and name(128, 16, 4096, 128, 1 << 30) == "gemm_panel"      # however few the tiles
-    assert name(128, 4096, 4224, 128) == "gemm_tile_128x128"         # a longer K: the kernels that split it, given scratch memory
+    assert name(128, 4096, 4224, 128, 1 << 30) == "gemm_panel_splitk" and name(256, 4096, 4224, 128, 1 << 30) == "gemm_tile_128x128_splitk"   # a longer K: split, given scratch memory
     assert name(512, 4096, 4096, 64) == "gemm_tile_128x128"          # block 64 stops at 48 columns: 4 x 86 tiles are more than one round
     assert name(300, 500, 512, 32) == "gemm_tile_128x128"            # block 32: not its
     # 33 to 64 rows: the same on tiles of 64 rows x 32 ... 128 columns, where gemv_staged (below) does not apply or K is at most 1024
@@ -267,14 +267,14 @@ def test_kernel_choice_by_shape():
     assert name(65, 4096, 8192, 128, 1 << 30) == "gemm_panel_splitk" and name(128, 4096, 11008, 64, 1 << 30) == "gemm_panel_splitk"
     assert name(128, 4096, 12416, 128, 1 << 30) == "gemm_tile_128x128_splitk" and name(129, 4096, 8192, 128, 1 << 30) != "gemm_panel_splitk"
     assert name(1, 128, 128 * 1024, 128) == "gemv_staged"            # any K: the scales stream through LDS with the stages
-    assert name(128, 4096, 8192, 128) == "gemm_tile_128x128"         # no scratch memory: one pass
+    assert name(128, 4096, 8192, 128) == "gemm_panel" and name(128, 32768, 8192, 128) == "gemm_tile_128x128"   # no scratch memory: one pass
     # few tiles of 256x128 and a long K: pieces of every tile on the 256x256 kernel's loop (the GPT-2 grad-weight GEMMs)
     assert name(3072, 768, 8192, 64, 1 << 25) == "gemm_wide_256x128_splitk" and name(3072, 768, 8192, 64) == "gemm_tile_128x128"
     assert name(1024, 4096, 4096, 128, 1 << 25) == "gemm_tile_128x128"        # two pieces of 16 stages: the slabs would cost more
     ws = lib.bi8_gemm_workspace_bytes(128, 2048, 16384, 128)
     # 32 tiles of 64x128, eight workgroups each: one fp32 slab of a tile per workgroup
     assert ws == 8 * 128 * 2048 * 4 and name(128, 2048, 16384, 128, ws) == "gemm_tile_64x128_splitk"
-    assert name(128, 2048, 16384, 128, ws - 1) == "gemm_tile_128x128"     # too small a workspace is not used
+    assert name(128, 2048, 16384, 128, ws - 1) == "gemm_panel"            # too small a workspace is not used: one pass on narrow tiles
     assert name(512, 4096, 8192, 128, 1 << 30) == "gemm_wide_256x128_splitk" and name(512, 4096, 4096, 64, 1 << 30) == "gemm_tile_128x128_splitk"
     # 144 tiles of 128x128: runs that end inside tiles fill the chip when K is long enough to pay for the second kernel
     assert name(3072, 768, 8192, 32, 1 << 30) == "gemm_tile_128x128_splitk" and name(3072, 768, 2048, 32, 1 << 30) == "gemm_tile_128x128"
