@@ -724,7 +724,7 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // launch, so it wins where K is short (the plan's rule and the measurements behind it: kPanelMaxStages).
 // Twelve waves.  Eight compute, each 16 rows x 16 * NJ columns (NJ subtiles of 16 x 16 on v_mfma_i32_16x16x64_i8): stacked,
 // a tile of 128 rows (described here), or as 4 x 2 a tile of 64 rows x 32 * NJ columns for up to 64 rows (half the bytes
-// of A).  Four only load: a ring of six to eight stage buffers is filled by their `buffer_load ... lds`, each loader its
+// of A), or as 2 x 4 a tile of 32 rows x 64 * NJ columns for up to 32.  Four only load: a ring of six to eight stage buffers is filled by their `buffer_load ... lds`, each loader its
 // share of a stage's wave-instructions (rows of A, rows of W, scale rows); stages past the end of K are loaded from
 // beyond the buffers' ranges (zeros, no memory access), so a loader's count of loads in flight is the same everywhere.
 // ONE barrier per stage, which all twelve waves meet: a loader arrives when its loads of stage s + 1 have landed, and
@@ -746,12 +746,14 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // instead of in front of them (both the same), every wave repeating somebody else's W or scale row to keep the waves'
 // counts equal (0.26 against 0.25 us).
 // CG = column groups of the eight waves: 1 -> 8 x 1 waves, tiles of 128 rows x 16 * NJ columns; 2 -> 4 x 2 waves, tiles of
-// 64 rows x 32 * NJ columns (for up to 64 rows: half the bytes of A per stage)
+// 64 rows x 32 * NJ columns (for up to 64 rows: half the bytes of A per stage); 4 -> 2 x 4 waves, tiles of 32 rows x 64 * NJ
+// columns (for up to 32 rows: a quarter)
 template <int NBS, int NJ, int CG> struct PanelLds {
     static constexpr int BM = 128 / CG, BN = 16 * NJ * CG;
-    static constexpr int kSWRow = BN > 64 ? 128 : 64;                        // (a scale row is loaded 64 floats at a time)
-    static constexpr int kABuf = BM * kStageK, kWBuf = BN * kStageK;         // 16 or 8 KiB, 2 ... 16 KiB
-    static constexpr int kSABuf = NBS * BM * 4, kSWBuf = NBS * kSWRow * 4;
+    static constexpr int kSWRow = (BN + 63) / 64 * 64;                       // (a scale row is loaded 64 floats at a time)
+    static constexpr int kABuf = BM * kStageK, kWBuf = BN * kStageK;         // 16, 8 or 4 KiB; 2 ... 32 KiB
+    static constexpr int kSARow = BM > 64 ? BM : 64;                         // (... and so is a row of row scales)
+    static constexpr int kSABuf = NBS * kSARow * 4, kSWBuf = NBS * kSWRow * 4;
     static constexpr int kStage = kABuf + kWBuf + kSABuf + kSWBuf;
     static constexpr int kBufs = (158 * 1024 / kStage) >= 8 ? 8 : (158 * 1024 / kStage) >= 6 ? (158 * 1024 / kStage) : 4;
     static constexpr int kAReg = 0;
@@ -770,7 +772,7 @@ template <int BLK, int CDT, int NJ, int CG = 1, bool SPLIT = false>
 __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
     static_assert(!SPLIT || CDT == BI8_F32, "the slabs are fp32 sums");
     static_assert(BLK == 128 || BLK == 64, "a K-block is one or two MFMAs of 64 bytes of K");
-    static_assert(NJ >= 1 && NJ <= 4 && (CG == 1 || CG == 2), "16 ... 64 columns per wave, one or two waves side by side");
+    static_assert(NJ >= 1 && NJ <= 4 && (CG == 1 || CG == 2 || CG == 4), "16 ... 64 columns per wave, one, two or four waves side by side");
     constexpr int NBS = kStageK / BLK;
     using L = PanelLds<NBS, NJ, CG>;
     constexpr int BM = L::BM, BN = L::BN, RG = 8 / CG;                     // RG = row groups of 16 rows
@@ -801,7 +803,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
         // at compile time, one copy of the code per loader.  Stages past the end of K are loaded from beyond the buffers'
         // ranges (zeros, no memory access), so a loader's count of loads in flight never changes.
         constexpr int kAItems = BM / 8, kWItems = BN / 8;
-        constexpr int kSAParts = BM / 64, kSWParts = L::kSWRow / 64, kSParts = kSAParts + kSWParts;
+        constexpr int kSAParts = L::kSARow / 64, kSWParts = L::kSWRow / 64, kSParts = kSAParts + kSWParts;
         constexpr int kItems = kAItems + kWItems + kSParts * NBS, kSlots = (kItems + kPanelLoaders - 1) / kPanelLoaders;
         static_assert(kAItems % 2 == 0 && kPanelLoaders % 2 == 0, "the swizzle term of a loader's row items does not depend on the slot");
         static_assert((kBufs - 1) * kSlots < 64, "a loader's loads in flight fit the counter");
@@ -836,7 +838,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
                         const int sc = item - kA - kW, kb = sc / kSParts, r = sc % kSParts;
                         if (r < kSAParts) {
                             const uint32_t pos = real ? (kb0 + kb) * sa_row + r * 256 : (uint32_t)kBufOut;
-                            bi8_buffer_to_lds4(sa_rsrc, lds_base + L::kSAReg + buf * L::kSABuf + (kb * BM + r * 64) * 4, s_lane, pos);
+                            bi8_buffer_to_lds4(sa_rsrc, lds_base + L::kSAReg + buf * L::kSABuf + (kb * L::kSARow + r * 64) * 4, s_lane, pos);
                         } else {
                             const uint32_t pos = real ? (kb0 + kb) * sw_row + (r - kSAParts) * 256 : (uint32_t)kBufOut;
                             bi8_buffer_to_lds4(sw_rsrc, lds_base + L::kSWReg + buf * L::kSWBuf + (kb * L::kSWRow + (r - kSAParts) * 64) * 4, s_lane, pos);
@@ -901,7 +903,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
         constexpr int P = decltype(par_c)::value;
 #pragma unroll
         for (int kb = 0; kb < NBS; ++kb) {
-            sx[P][kb] = *(const bi8_v4f *)(lds + sa_base + buf * L::kSABuf + kb * BM * 4);
+            sx[P][kb] = *(const bi8_v4f *)(lds + sa_base + buf * L::kSABuf + kb * L::kSARow * 4);
 #pragma unroll
             for (int j = 0; j < NJ; ++j) bw[P][kb][j] = *(const float *)(lds + sw_base + buf * L::kSWBuf + (kb * L::kSWRow + j * 16) * 4);
         }
@@ -2598,7 +2600,7 @@ struct GemmPlan {
 // mostly empty round and the 256x256 kernel wins (1284 against 978 TOP/s at 2304x4096x4096, 144 tiles).
 // (choosing between the two by the fill of the last round of workgroups changed nothing measurable)
 constexpr int64_t kWideMinTiles = 129;
-// gemm_panel: more than 32 rows, at most one tile of 128 x (16 ... 64) -- up to 64 rows: 64 x (32 ... 128) -- per CU, and a
+// gemm_panel: at most one tile of 128 x (16 ... 64) -- up to 64 rows: 64 x (32 ... 128), up to 32: 32 x (64 ... 256) -- per CU, and a
 // short K: every workgroup streams all rows of A, so its time grows with K faster than that of the kernels that split the
 // contraction.  Measured against what ran these shapes before (one-pass or split 64x128 / 128x128 tiles), W from HBM,
 // block 128, us at K = 768 / 2048 / 4096 / 8192: 128 x 768 8.4 -> 4.3, 10.8 -> 6.0, 11.0 -> 8.7, 12.7 -> 13.8; 128 x 4096
@@ -2610,6 +2612,8 @@ constexpr int64_t kPanelMaxStages = 32;        // K <= 4096
 constexpr int64_t kPanelSplitMinStages = 8;    // the split form: the least stages of K per piece ...
 constexpr int64_t kPanelSplitMaxStages = 96;   // ... and the longest K (12288)
 constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024
+constexpr int64_t kPanelFewRows = 32;          // up to 32 rows: tiles of 32 rows x (64 ... 256) columns ...
+constexpr int64_t kPanelFewRowsMinCols = 6144; // ... from this many columns on (fewer leave most CUs without a tile)
 // the widest tile, in 16-column subtiles (block 64 at 64 columns needs more registers than a wave has)
 constexpr int panel_max_subtiles(int block) { return block == 64 ? 3 : 4; }
 constexpr int64_t kStagedMaxRows = 32;         // gemv_staged: one or two groups of 16 rows whatever the shape ...
@@ -2721,6 +2725,19 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                 return p;
             }
             panel_if_no_split = (N + widest - 1) / widest <= kCus && !staged_band;
+        }
+        // 3 ... 32 rows against many columns: gemm_panel on tiles of 32 rows x 64 ... 256 columns, one per CU, where gemv_staged's
+        // workgroups of 16 columns run in several rounds (measured, block 128, W from HBM, us, gemv_staged -> gemm_panel at
+        // K = 1024 / 4096: 16 rows N = 6144 7.2 -> 4.2, 10.4 -> 9.4; N = 11008 6.1 -> 4.7, 13.6 -> 11.9; N = 32000 13.8 -> 9.1, 31.8 -> 29.8;
+        // 32 rows N = 8192 5.7 -> 4.1, 12.3 -> 11.4; N = 11008 7.8 -> 4.3, 16.4 -> 12.5; N = 16384 10.1 -> 5.0, 21.6 -> 16.3; N = 32000
+        // 17.9 -> 8.1, 37.3 -> 30.0; at N = 4096 the 64 tiles leave most CUs idle: 16 rows 6.5 -> 9.1, 32 rows 7.9 -> 9.9 at K = 4096)
+        if (M > kRowsMax && M <= kPanelFewRows && N >= kPanelFewRowsMinCols && (block == 64 || block == 128) &&
+            (K / block + 1) * max_mn * 4 < kBufOut && K / kStageK <= kPanelMaxStages) {
+            const int64_t widest = 64 * panel_max_subtiles(block);
+            if ((N + widest - 1) / widest <= kCus) {
+                p.kernel = kKPanel;
+                return p;
+            }
         }
         const bool staged_rows = M <= kStagedMaxRows || staged_band;
         if (staged_rows && (block == 64 || block == 128) && (K / block + 16) * N * 4 < 0x3fffffffLL && 16 * ldw + K < 0x3fffffffLL &&
@@ -2874,6 +2891,7 @@ template <int BLK, int CDT> int launch_panel_split(GemmArgs g, hipStream_t st) {
     return bi8_launch_rc();
 }
 template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) {
+    if (g.M <= kPanelFewRows) return launch_panel_cg<BLK, CDT, 4>(g, st);
     return g.M <= 64 ? launch_panel_cg<BLK, CDT, 2>(g, st) : launch_panel_cg<BLK, CDT, 1>(g, st);
 }
 

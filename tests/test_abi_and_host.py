@@ -252,12 +252,17 @@ def test_kernel_choice_by_shape():
     # 33 to 64 rows: the same on tiles of 64 rows x 32 ... 128 columns, where gemv_staged (below) does not apply or K is at most 1024
     assert name(64, 5000, 640, 128) == "gemm_panel" and name(48, 11008, 4096, 128, 1 << 30) == "gemm_panel" and name(33, 16384, 4096, 64) == "gemm_panel"
     assert name(48, 700, 640, 128) == "gemm_panel" and name(64, 4096, 1024, 64) == "gemm_panel" and name(64, 4096, 1152, 64) == "gemv_staged"
-    assert name(64, 33000, 768, 128) == "gemm_wide" and name(32, 11008, 768, 128) == "gemv_staged"    # too many columns for one round; 32 rows
+    assert name(64, 33000, 768, 128) == "gemm_wide"                  # too many columns for one round
+    # 3 to 32 rows against 6144 columns or more: the same on tiles of 32 rows x 64 ... 256 columns
+    assert name(32, 11008, 768, 128) == "gemm_panel" and name(16, 11008, 4096, 64) == "gemm_panel" and name(3, 6144, 4096, 128, 1 << 30) == "gemm_panel"
+    assert name(32, 11008, 4096, 64, 1 << 30) == "gemm_panel" and name(16, 32000, 4096, 128) == "gemm_panel" and name(8, 50257, 768, 128) == "gemm_panel"
+    assert name(16, 6143, 4096, 128) == "gemv_staged" and name(16, 11008, 4224, 128) == "gemv_staged" and name(2, 11008, 4096, 128) == "gemv_rows"
+    assert name(16, 50257, 768, 64) == "gemv_staged" and name(16, 65537, 768, 128) == "gemv_staged"      # 262 tiles of 192 / 257 of 256 columns
     assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
-    assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 11008, 4096, 64) == "gemv_staged"
+    assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 4096, 11008, 64) == "gemv_staged"
     assert name(2, 4096, 32768, 128) == "gemv_staged"                  # 2 x 32768 codes do not fit the few-row kernel's LDS
     assert name(16, 4096, 4096, 32) == "gemm_skinny" and name(24, 4096, 4096, 32) == "gemm_skinny"     # block 32, few rows
-    assert name(24, 4096, 4096, 128) == "gemv_staged" and name(32, 11008, 4096, 64, 1 << 30) == "gemv_staged"   # two groups of 16 rows
+    assert name(24, 4096, 4096, 128) == "gemv_staged" and name(32, 4096, 11008, 64, 1 << 30) == "gemv_staged"   # two groups of 16 rows
     assert name(24, 4096, 4096, 32, 1 << 30) == "gemm_tile_64x128_splitk"      # block 32 with scratch memory: the split tiles are ahead
     # 33 to 64 rows: one pass over W where one round of workgroups covers the columns and K is short, else the split tiles
     assert name(33, 4096, 4096, 128, 1 << 30) == "gemv_staged" and name(64, 4096, 4096, 64) == "gemv_staged" and name(48, 700, 1280, 128) == "gemv_staged"

@@ -76,7 +76,7 @@ def test_llama_shaped_gemm_sweep(pkg, KN_, M):
         assert torch.equal(y, y2)                   # the one-kernel path and the two launches give the same bits
         ws = _lib.load().bi8_gemm_workspace_bytes(M, N, K, block)
         kernel = _lib.load().bi8_gemm_kernel_name(M, N, K, K, K, block, ws).decode()
-        want = {1: "gemv_rows", 16: "gemv_staged", 128: "gemm_panel" if K <= 4096 else "splitk",
+        want = {1: "gemv_rows", 16: "gemm_panel" if N >= 6144 and K <= 4096 else "gemv_staged", 128: "gemm_panel" if K <= 4096 else "splitk",
                 2048: "gemm_wide_256x128" if N == 4096 else "gemm_wide", 8192: "gemm_wide"}[M]
         assert want in kernel, kernel
         rows = torch.arange(M) if M <= 128 else torch.randperm(M, generator=g)[:64]

@@ -162,9 +162,9 @@ def test_bias_dtypes_on_the_persistent_kernel(ops, out, block):
             assert torch.equal(Cb, C + bias.to(DTYPES[out]))             # added after the cast, in the output dtype
 
 
-@pytest.mark.parametrize("M,N,K", [(7, 11008, 2048), (16, 11008, 4096), (3, 8192, 2048), (17, 11008, 2048), (32, 8192, 4096), (25, 4096, 2048)])
+@pytest.mark.parametrize("M,N,K", [(7, 11008, 4224), (16, 11008, 4608), (3, 8192, 4224), (17, 11008, 4224), (32, 8192, 4352), (25, 4096, 2048)])
 def test_small_batches_against_many_columns_call_after_call(ops, M, N, K):
-    """3 to 32 rows against more than 6144 columns run gemv_staged with four waves per workgroup, two or three workgroups
+    """3 to 32 rows against more than 6144 columns and a K beyond 4096 run gemv_staged with four waves per workgroup, two or three workgroups
     per CU (the last shape: eight waves, one workgroup per CU).  Every wave streams W and A through a private LDS ring with direct-to-LDS loads; a load that overwrites a slot
     must not be issued while the stage before is still reading it (a load of A, which the CU's L1 holds for the younger
     workgroups, can land within an LDS read's latency: such workgroups used to return wrong sums now and then).  Ten calls

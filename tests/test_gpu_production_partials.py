@@ -125,6 +125,16 @@ CASES = [
     (50, 24000, 256, 128, "gemm_panel"),            # 250 tiles of 96 columns
     (40, 24000, 384, 64, "gemm_panel"),             # ... two K-blocks per stage
     (64, 32000, 384, 128, "gemm_panel"),            # 250 tiles of 128 columns
+    # ... and for 3 to 32 rows against 6144 columns or more tiles of 32 rows, the waves as 2 x 4: 64, 128, 192 and 256 columns per tile
+    (7, 8192, 2048, 128, "gemm_panel"),             # 128 tiles of 64 columns, the second row group empty
+    (12, 11008, 2048, 64, "gemm_panel"),            # 172 tiles
+    (17, 8192, 2048, 128, "gemm_panel"),
+    (29, 11008, 1024, 64, "gemm_panel"),
+    (32, 6144, 4096, 128, "gemm_panel"),            # 96 tiles, 32 stages
+    (5, 6150, 256, 128, "gemm_panel"),              # the last tile 6 columns wide
+    (24, 30000, 384, 128, "gemm_panel"),            # 235 tiles of 128 columns
+    (20, 40000, 384, 64, "gemm_panel"),             # 209 tiles of 192 columns, two K-blocks per stage
+    (3, 50000, 128, 128, "gemm_panel"),             # 196 tiles of 256 columns, one stage
     (2304, 2304, 256, 32, "gemm_tile_128x128"),
     (48, 5000, 640, 32, "gemm_tile_64x128"),
     (48, 700, 1280, 64, "gemv_staged"),             # four groups of 16 rows
@@ -138,12 +148,12 @@ CASES = [
     (3, 384, 512, 128, "gemv_staged"),
     (16, 1000, 4096, 128, "gemv_staged"),           # eight stages per wave
     (7, 1000, 1152, 64, "gemv_staged"),
-    (7, 8192, 2048, 128, "gemv_staged"),            # more than 6144 columns: four waves per workgroup, several workgroups per CU
-    (12, 11008, 2048, 64, "gemv_staged"),
+    (7, 8192, 4224, 128, "gemv_staged"),            # more than 6144 columns: four waves per workgroup, several workgroups per CU
+    (12, 11008, 4224, 64, "gemv_staged"),
     (24, 500, 640, 128, "gemv_staged"),             # two groups of 16 rows
     (32, 1000, 2048 + 128, 64, "gemv_staged"),
-    (17, 8192, 2048, 128, "gemv_staged"),           # ... four waves per workgroup, two workgroups per CU
-    (29, 11008, 1024, 64, "gemv_staged"),
+    (17, 8192, 4224, 128, "gemv_staged"),           # ... four waves per workgroup, two workgroups per CU
+    (29, 11008, 4224, 64, "gemv_staged"),
     (24, 500, 640, 32, "gemm_skinny"),              # block 32, five stages of K: nothing to split
     (24, 500, 2048, 32, "gemm_tile_64x128_splitk"),
     (16, 300, 1024, 32, "gemm_skinny"),
