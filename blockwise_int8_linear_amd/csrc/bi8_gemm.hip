@@ -2611,6 +2611,10 @@ constexpr int64_t kPanelMinRows = 64;          // more rows: tiles of 128 rows; 
 constexpr int64_t kPanelMaxStages = 32;        // K <= 4096
 constexpr int64_t kPanelSplitMinStages = 8;    // the split form: the least stages of K per piece ...
 constexpr int64_t kPanelSplitMaxStages = 96;   // ... and the longest K (12288)
+constexpr int64_t kPanelSplitFewRowsMin = 16;  // the split form on tiles of 32 rows: more rows than this, ...
+constexpr int64_t kPanelSplitFewRowsMinStages = 64, kPanelSplitFewRowsTwoStages = 80;      // ... K from 8192 on; two pieces per tile from 10240 on, ...
+constexpr int64_t kPanelSplitFewRowsMinGroups = 192;                                       // ... and this many workgroups
+constexpr int64_t kPanelSplit64RowsMinStages = 40, kPanelSplit64RowsMaxTiles = 32;         // on tiles of 64 rows: K from 5120 on, up to 2048 columns
 constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024
 constexpr int64_t kPanelFewRows = 32;          // up to 32 rows: tiles of 32 rows x (64 ... 256) columns ...
 constexpr int64_t kPanelFewRowsMinCols = 6144; // ... from this many columns on (fewer leave most CUs without a tile)
@@ -2643,23 +2647,38 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     if (!tile_ok) return p;
     // few tiles and scratch memory: split K over the workgroups, then sum the slabs
     bool panel_if_no_split = false;                // gemm_panel's tiles would give one round, but K is beyond what it is given outright
-    auto try_split = [&]() {
+    auto try_split = [&](bool few_rows_split = false) {
         if (partials || ws_bytes <= 0) return false;
         // 65 ... 128 rows and K up to 12288: gemm_panel on pieces of K, tiles of 128 rows x 64 columns (block 64: 32).  Measured
         // against the split 64x128 / 128x128 tiles, block 128, W from HBM, us at K = 8192 / 11008 / 16384: 128 x 768 12.9 -> 11.1,
         // 13.7 -> 11.8, 17.4 -> 14.1; 128 x 4096 21.7 -> 18.8, 24.8 -> 20.1, 25.8 -> 31.2; 128 x 8192 28.4 -> 26.3, 35.4 -> 32.9,
         // 43.7 -> 46.7; 512 x 768 18.7 -> 15.1, 19.9 -> 20.3; 512 x 2048 25.8 -> 23.6, 28.5 -> 28.8; 1024 x 768 21.8 -> 23.0
         // (256 workgroups that each stream all of A: the longer the pieces and the more rows of tiles, the less it pays).
-        if (block != 32 && M > kPanelMinRows && M <= 128 && K / kStageK <= kPanelSplitMaxStages && !rest_of_cut && (K / block + 1) * max_mn * 4 < kBufOut) {
-            const int64_t bn = block == 64 ? 32 : 64, t = ((M + 127) / 128) * ((N + bn - 1) / bn), nst = K / kStageK;
+        // 17 ... 32 rows and K from 8192 on: the same on tiles of 32 x 64 where the columns leave three pieces of K or more per tile,
+        // or two of 40 stages, and 192 workgroups or more; 33 ... 64 rows and K from 5120 on: tiles of 64 x 64 where there are at most
+        // 32 of them.  Measured against gemv_staged and the split 64x128 tiles, block 128, W from HBM, us at K = 8192 / 11008 / 12288:
+        // 32 x 1024 7.3 -> 7.7; 32 x 2048 10.0 -> 8.8, 13.6 -> 10.0, 15.0 -> 10.4; 32 x 4096 11.8 -> 11.5, 16.5 -> 14.2, 16.3 -> 15.0;
+        // 32 x 5120 17.5 -> 13.1, 25.4 -> 18.0; 32 x 8192 19.3 -> 20.3, 28.1 -> 23.0, 30.2 -> 23.2; at K = 5120 / 7168 32 x 2048 7.4 -> 8.0,
+        // 9.2 -> 8.3, 32 x 4096 9.9 -> 9.6, 10.9 -> 11.1; 16 rows stay with gemv_staged: 16 x 4096 9.7 -> 11.3, 13.8 -> 13.9, 13.0 -> 14.6.
+        // 64 x 1024 at K = 5120 / 7168 / 8192 9.2 -> 8.6, 11.1 -> 8.4, 11.2 -> 8.4; 64 x 2048 9.9 -> 8.6, 12.1 -> 9.4, 12.6 -> 10.0, at
+        // K = 11008 14.0 -> 11.2; 40 x 2048 8.6 -> 8.4, 11.6 -> 9.0; 64 x 4096 (two runs) 12.2 -> 11.2, 15.5 -> 14.2, 14.0 -> 12.7 and 14.5 -> 15.4,
+        // block 64 16.2 -> 16.4, at K = 11008 18.8 -> 19.8: not taken.
+        const bool few = M <= kPanelMinRows;
+        const int64_t ps_bm = M <= kPanelFewRows ? 32 : few ? 64 : 128, ps_nst = K / kStageK;
+        if (block != 32 && M > (few_rows_split ? kPanelSplitFewRowsMin : kPanelMinRows) && M <= 128 && ps_nst <= kPanelSplitMaxStages &&
+            (!few || ps_nst >= (ps_bm == 32 ? kPanelSplitFewRowsMinStages : kPanelSplit64RowsMinStages)) && !rest_of_cut &&
+            (K / block + 1) * max_mn * 4 < kBufOut) {
+            const int64_t bm = ps_bm, nst = ps_nst, bn = block == 64 && bm == 128 ? 32 : 64, t = (N + bn - 1) / bn;
             int64_t per = t > 0 && t <= kCus / 2 ? kCus / t : 0;
             if (per > kSplitMax) per = kSplitMax;
             if (per > nst / kPanelSplitMinStages) per = nst / kPanelSplitMinStages;
-            if (per >= 2) {
+            const int64_t least = bm == 128 ? 2 : bm == 64 ? 4 : nst >= kPanelSplitFewRowsTwoStages ? 2 : 3;
+            const bool enough = bm == 128 || (bm == 64 ? t <= kPanelSplit64RowsMaxTiles : t * per >= kPanelSplitFewRowsMinGroups);
+            if (per >= least && enough) {
                 const int64_t stages = (nst + per - 1) / per;
                 per = (nst + stages - 1) / stages;
-                const int64_t need = t * per * 128 * bn * 4;
-                if (per >= 2 && need <= ws_bytes) {
+                const int64_t need = t * per * bm * bn * 4;
+                if (per >= least && need <= ws_bytes) {
                     p.kernel = kKSplitPanel;
                     p.splits = (int)(t * per);
                     p.split_stages = (int)stages;
@@ -2669,6 +2688,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                 }
             }
         }
+        if (few_rows_split) return false;          // (asked ahead of gemv_staged: only for that rule)
         // 256x128 tiles on gemm_wide's loop, split evenly, where that puts most of the CUs to work
         if (block != 32 && M > 128 && wide_addressable(M, N, K, lda, ldw, block)) {
             const int64_t t = ((M + 255) / 256) * ((N + 127) / 128), nst = K / kStageK;
@@ -2712,6 +2732,8 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             p.kernel = kKRows;
             return p;
         }
+        // 17 ... 64 rows against a long K, given scratch memory: gemm_panel on pieces of K where the rule in try_split has it
+        if (M > kPanelSplitFewRowsMin && M <= kPanelMinRows && try_split(true)) return p;
         // 33 ... 64 rows: gemm_panel on tiles of 64 rows where the columns fit one round of them and K is at most 4096 --
         // unless gemv_staged's four groups of rows apply, which are ahead from K = 1152 on (measured, 64 rows, block 128, W from
         // HBM, us, gemv_staged or the split 64x128 tiles -> gemm_panel, K = 768 / 2048 / 4096 / 8192: N = 4096 5.7 -> 4.7,
@@ -2842,10 +2864,12 @@ template <int BLK, int CDT, int NW, int MT> int launch_staged_as(const GemmArgs 
 template <int BLK, int CDT> int launch_staged(const GemmArgs &g, hipStream_t st) {
     const int64_t tn = (g.N + 15) / 16;
     if (tn > 0x7fffffffLL) return BI8_ERR_TOO_LARGE;
-    // eight waves per workgroup where four would leave CUs with a single workgroup's loads in flight; up to 16 rows three
-    // workgroups of four waves share a CU, up to 32 rows (twice the A ring) two
-    if (g.M <= 16) return tn <= 384 ? launch_staged_as<BLK, CDT, 8, 1>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 1>(g, (unsigned)tn, st);
-    if (g.M <= 32) return tn <= 384 ? launch_staged_as<BLK, CDT, 8, 2>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 2>(g, (unsigned)tn, st);
+    // eight waves per workgroup (one workgroup per CU) where that is one round of workgroups; else four: up to 16 rows three
+    // workgroups of four waves share a CU, up to 32 rows (twice the A ring) two (measured, 16 rows, block 128, W from HBM, eight
+    // waves -> four: N = 4112, K = 1024 / 4096 / 11008 6.7 -> 4.3, 9.6 -> 8.7, 19.5 -> 18.9 us; N = 5120 6.9 -> 4.5, 10.1 -> 9.2,
+    // 21.4 -> 20.5; 32 rows N = 5120 8.9 -> 5.6, 12.7 -> 11.0, 27.0 -> 25.4)
+    if (g.M <= 16) return tn <= kCus ? launch_staged_as<BLK, CDT, 8, 1>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 1>(g, (unsigned)tn, st);
+    if (g.M <= 32) return tn <= kCus ? launch_staged_as<BLK, CDT, 8, 2>(g, (unsigned)tn, st) : launch_staged_as<BLK, CDT, 4, 2>(g, (unsigned)tn, st);
     // up to 64 rows the rings of A leave room for four waves, one workgroup per CU (the plan asks for no more rows)
     if (g.M <= 64) return launch_staged_as<BLK, CDT, 4, 4>(g, (unsigned)tn, st);
     return BI8_ERR_UNSUPPORTED;
@@ -2873,14 +2897,13 @@ template <int BLK, int CDT, int CG> int launch_panel_cg(const GemmArgs &g, hipSt
     return BI8_ERR_UNSUPPORTED;                    // (the plan sends no other problem here)
 }
 // the split form: tiles of 128 rows x 64 columns (block 64: 32), split_per_tile pieces of split_stages stages each, then the sum
-template <int BLK, int CDT> int launch_panel_split(GemmArgs g, hipStream_t st) {
-    constexpr int NJ = BLK == 64 ? 2 : 4;
-    using L = PanelLds<kStageK / BLK, NJ, 1>;
+template <int BLK, int CDT, int NJ, int CG> int launch_panel_split_as(GemmArgs g, hipStream_t st) {
+    using L = PanelLds<kStageK / BLK, NJ, CG>;
     g.tiles_m = (int)((g.M + L::BM - 1) / L::BM);
     g.tiles_n = (int)((g.N + L::BN - 1) / L::BN);
     g.tile_m0 = g.tile_n0 = 0;
     if (g.split_per_tile < 2 || g.split_per_tile > kSplitMax || (int64_t)g.tiles_m * g.tiles_n * g.split_per_tile > 2 * kCus) return BI8_ERR_UNSUPPORTED;
-    auto kern = gemm_panel<BLK, BI8_F32, NJ, 1, true>;
+    auto kern = gemm_panel<BLK, BI8_F32, NJ, CG, true>;
     static LdsOptIn opted;                         // one per kernel instantiation
     const int rc = opted.ensure((const void *)kern, L::kBytes);
     if (rc != BI8_OK) return rc;
@@ -2889,6 +2912,12 @@ template <int BLK, int CDT> int launch_panel_split(GemmArgs g, hipStream_t st) {
     if (rc_launch != BI8_OK) return rc_launch;
     hipLaunchKernelGGL((splitk_reduce<CDT, L::BM, L::BN>), dim3((unsigned)(g.tiles_m * g.tiles_n), L::BM / (256 / (L::BN / 4))), dim3(256), 0, st, g);
     return bi8_launch_rc();
+}
+// (the tiles the plan has counted: 32 rows x 64 columns up to 32 rows, 64 x 64 up to 64, else 128 x 64, at block 64 128 x 32)
+template <int BLK, int CDT> int launch_panel_split(const GemmArgs &g, hipStream_t st) {
+    if (g.M <= kPanelFewRows) return launch_panel_split_as<BLK, CDT, 1, 4>(g, st);
+    if (g.M <= kPanelMinRows) return launch_panel_split_as<BLK, CDT, 2, 2>(g, st);
+    return launch_panel_split_as<BLK, CDT, BLK == 64 ? 2 : 4, 1>(g, st);
 }
 template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) {
     if (g.M <= kPanelFewRows) return launch_panel_cg<BLK, CDT, 4>(g, st);

@@ -262,11 +262,21 @@ def test_kernel_choice_by_shape():
     assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 4096, 11008, 64) == "gemv_staged"
     assert name(2, 4096, 32768, 128) == "gemv_staged"                  # 2 x 32768 codes do not fit the few-row kernel's LDS
     assert name(16, 4096, 4096, 32) == "gemm_skinny" and name(24, 4096, 4096, 32) == "gemm_skinny"     # block 32, few rows
-    assert name(24, 4096, 4096, 128) == "gemv_staged" and name(32, 4096, 11008, 64, 1 << 30) == "gemv_staged"   # two groups of 16 rows
+    assert name(24, 4096, 4096, 128) == "gemv_staged" and name(32, 4096, 11008, 64) == "gemv_staged"   # two groups of 16 rows
     assert name(24, 4096, 4096, 32, 1 << 30) == "gemm_tile_64x128_splitk"      # block 32 with scratch memory: the split tiles are ahead
     # 33 to 64 rows: one pass over W where one round of workgroups covers the columns and K is short, else the split tiles
     assert name(33, 4096, 4096, 128, 1 << 30) == "gemv_staged" and name(64, 4096, 4096, 64) == "gemv_staged" and name(48, 700, 1280, 128) == "gemv_staged"
     assert name(48, 11008, 8192, 128, 1 << 30) == "gemm_tile_64x128_splitk" and name(48, 4096, 11008, 128, 1 << 30) == "gemm_tile_64x128_splitk"
+    # 33 to 64 rows, K from 5120 to 12288, up to 2048 columns: narrow tiles of 64 rows on pieces of K
+    assert name(48, 2048, 11008, 128, 1 << 30) == "gemm_panel_splitk" and name(64, 1024, 5120, 64, 1 << 30) == "gemm_panel_splitk"
+    assert name(64, 2049, 8192, 128, 1 << 30) == "gemm_tile_64x128_splitk" and name(64, 2048, 4992, 128, 1 << 30) != "gemm_panel_splitk"
+    assert name(64, 2048, 12416, 128, 1 << 30) == "gemm_tile_64x128_splitk"
+    # 17 to 32 rows, K from 8192: tiles of 32 rows where that gives 192 workgroups of three pieces per tile or more, or two of 40 stages
+    assert name(32, 4096, 8192, 128, 1 << 30) == "gemm_panel_splitk" and name(17, 2048, 11008, 64, 1 << 30) == "gemm_panel_splitk"
+    assert name(32, 5120, 8192, 128, 1 << 30) == "gemm_panel_splitk" and name(17, 8192, 11008, 128, 1 << 30) == "gemm_panel_splitk"
+    assert name(32, 8192, 8192, 128, 1 << 30) == "gemv_staged" and name(16, 4096, 11008, 128, 1 << 30) == "gemv_staged" and name(32, 4096, 8064, 128, 1 << 30) == "gemv_staged"
+    assert name(32, 1024, 8192, 128, 1 << 30) == "gemv_staged"       # 16 tiles in eight pieces: 128 workgroups
+    assert name(32, 4096, 11008, 128) == "gemv_staged" and name(32, 4096, 11008, 32, 1 << 30) != "gemm_panel_splitk"      # no scratch memory; block 32
     assert name(65, 4096, 16384, 128, 1 << 30) == "gemm_tile_128x128_splitk"
     # 65 to 128 rows and K up to 12288: narrow tiles on pieces of K
     assert name(65, 4096, 8192, 128, 1 << 30) == "gemm_panel_splitk" and name(128, 4096, 11008, 64, 1 << 30) == "gemm_panel_splitk"

@@ -54,11 +54,14 @@ def _run(lib, A, W, sa, sw, bias, block, out, ws_bytes):
                                          # more than one round of workgroups
                                          (33, 128, 10240, 128), (48, 700, 7168, 128), (60, 4800, 4224, 128), (40, 700, 2560, 32),
                                          # 35 stages of K in pieces of 9, 9, 9, 8
-                                         (200, 300, 4480, 64)])
+                                         (200, 300, 4480, 64),
+                                         # 17 to 64 rows and a long K: narrow tiles of 32 x 64 or 64 x 64 on pieces of K
+                                         (24, 2000, 8320, 64), (32, 5000, 8192, 128), (20, 8192, 10240, 128), (64, 2000, 5120, 128),
+                                         (50, 1000, 12288, 64)])
 def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
     want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
-    assert 0 < want <= lib.bi8_static_scratch_bytes() and want % (128 * 32 * 4) == 0     # fp32 slabs of one tile (128x32 ... 128x128) each
+    assert 0 < want <= lib.bi8_static_scratch_bytes() and want % (32 * 64 * 4) == 0      # fp32 slabs of one tile (32x64 ... 128x128) each
     Ad, Wd, sad, swd = A.to(DEV), W.to(DEV), sa.to(DEV), sw.to(DEV)
     split = _run(lib, Ad, Wd, sad, swd, None, block, out, want)
     one = _run(lib, Ad, Wd, sad, swd, None, block, out, 0)

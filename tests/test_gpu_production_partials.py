@@ -162,6 +162,12 @@ CASES = [
     (128, 1024, 8192, 128, "gemm_panel_splitk"),    # 16 tiles, eight pieces of eight stages
     (65, 4100, 4224, 128, "gemm_panel_splitk"),     # 65 tiles (the last 4 columns wide), three pieces of 11 stages
     (100, 300, 5120, 64, "gemm_panel_splitk"),      # ten tiles of 32 columns, five pieces of eight stages, two K-blocks per stage
+    # ... and for 17 to 64 rows against a long K: tiles of 32 x 64 or 64 x 64
+    (32, 4096, 8192, 128, "gemm_panel_splitk"),     # 64 tiles, four pieces of 16 stages
+    (17, 5000, 8320, 64, "gemm_panel_splitk"),      # 79 tiles (the last 8 columns wide), three pieces of 22, 22 and 21 stages
+    (30, 8192, 10240, 128, "gemm_panel_splitk"),    # 128 tiles, two pieces of 40 stages
+    (64, 2048, 11008, 128, "gemm_panel_splitk"),    # 32 tiles of 64 x 64, eight pieces of 11 stages
+    (33, 2000, 5120, 64, "gemm_panel_splitk"),      # 32 tiles (the last 16 columns wide), five pieces of eight stages
     (512, 4096, 4096, 64, "gemm_tile_128x128_splitk"),
 ]
 
