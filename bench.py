@@ -201,17 +201,20 @@ def bench_extras(pkg, torch):
             sx = torch.rand(K // B, M, device="cuda") + 0.5
             c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
             turn = [0]
+            need = lib.bi8_gemm_workspace_bytes(M, N, K, B)          # scratch memory, as the Python operator passes it
+            scratch = torch.empty(max(need, 16), device="cuda", dtype=torch.uint8)
 
             def gv():
                 i = turn[0] = (turn[0] + 1) % nset
-                assert lib.bi8_gemm_nt_dequant(x.data_ptr(), ws[i].data_ptr(), sx.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
-                                               M, N, K, K, K, N, B, st) == 0
+                assert lib.bi8_gemm_nt_dequant_ws(x.data_ptr(), ws[i].data_ptr(), sx.data_ptr(), sw.data_ptr(), None, 0, c.data_ptr(), 1,
+                                                  M, N, K, K, K, N, B, scratch.data_ptr(), need, st) == 0
             for _ in range(5):
                 gv()
             t = median_ms(gv, 50)
             nbytes = N * K + 4 * (K // B) * (N + M) + M * K + 2 * M * N
             out[f"decode_gemm_M{M}_K{K}_N{N}"] = {"us": round(t * 1e3, 2), "GBps": round(nbytes / t / 1e6, 1),
-                                                  "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4)}
+                                                  "frac_hbm": round(nbytes / t / 1e6 / HBM_PEAK_GBS, 4),
+                                                  "kernel": lib.bi8_gemm_kernel_name(M, N, K, K, K, B, need).decode()}
             if M == 1:
                 # the whole eval-path linear for one token: row quantizer + GEMM as two launches, and as the one kernel
                 xf = torch.randn(M, K, device="cuda").to(torch.bfloat16)
