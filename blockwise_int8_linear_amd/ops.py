@@ -288,8 +288,8 @@ def _workspace(lib, M, N, K, block, device, stream):
     tensor per device and stream, kept for the life of the process (at most 32 MiB each) and shared by the GEMMs of
     that stream, which run one after the other.  While the stream is being captured into a graph the memory comes from
     the capture's own pool instead, so that graphs replayed side by side do not share it.
-    (Up to 32 rows at blocks 64 / 128 run the one-pass decode kernels whatever they are given: not asked.)"""
-    if M <= 32 and block != 32:
+    (Up to 16 rows at blocks 64 / 128 run the one-pass decode kernels whatever they are given: not asked.)"""
+    if M <= 16 and block != 32:
         return None, 0
     key = (M, N, K, block)
     need = _ws_need.get(key)

@@ -303,3 +303,23 @@ def test_kernel_choice_by_shape():
             for K in (1024, 4096, 11008 , 8192 * 4):
                 for block in (32, 64, 128):
                     assert lib.bi8_gemm_workspace_bytes(M, N, K, block) <= lib.bi8_static_scratch_bytes(), (M, N, K, block)
+    # up to 16 rows at blocks 64 / 128 no plan wants scratch memory (the Python launcher does not ask for such shapes) ...
+    for M in (1, 2, 3, 8, 16):
+        for N in (128, 1024, 2048, 4096, 5120, 11008, 50257):
+            for K in (1024, 4096, 8192, 11008, 8192 * 4):
+                for block in (64, 128):
+                    assert lib.bi8_gemm_workspace_bytes(M, N, K, block) == 0, (M, N, K, block)
+    # ... and from 17 on some do, and the launcher asks
+    from blockwise_int8_linear_amd import ops
+    assert lib.bi8_gemm_workspace_bytes(17, 4096, 11008, 128) > 0
+    asked = []
+
+    class _Probe:
+        def bi8_gemm_workspace_bytes(self, *a):
+            asked.append(a)
+            return 0
+    for M in (16, 17):
+        ops._ws_need.pop((M, 4096, 11008, 128), None)
+        ops._workspace(_Probe(), M, 4096, 11008, 128, None, None)
+        ops._ws_need.pop((M, 4096, 11008, 128), None)
+    assert asked == [(17, 4096, 11008, 128)]
