@@ -748,8 +748,9 @@ __global__ __launch_bounds__(WM *WN * 64) void gemm_tile(const GemmArgs g_in) {
 // CG = column groups of the eight waves: 1 -> 8 x 1 waves, tiles of 128 rows x 16 * NJ columns; 2 -> 4 x 2 waves, tiles of
 // 64 rows x 32 * NJ columns (for up to 64 rows: half the bytes of A per stage); 4 -> 2 x 4 waves, tiles of 32 rows x 64 * NJ
 // columns (for up to 32 rows: a quarter)
-template <int NBS, int NJ, int CG> struct PanelLds {
-    static constexpr int BM = 128 / CG, BN = 16 * NJ * CG;
+// NI = 16-row subtiles per wave (1 or 2): with two, 4 x 2 waves make a tile of 128 rows x 32 * NJ columns (the square form below)
+template <int NBS, int NJ, int CG, int NI = 1> struct PanelLds {
+    static constexpr int BM = 128 * NI / CG, BN = 16 * NJ * CG;
     static constexpr int kSWRow = (BN + 63) / 64 * 64;                       // (a scale row is loaded 64 floats at a time)
     static constexpr int kABuf = BM * kStageK, kWBuf = BN * kStageK;         // 16, 8 or 4 KiB; 2 ... 32 KiB
     static constexpr int kSARow = BM > 64 ? BM : 64;                         // (... and so is a row of row scales)
@@ -766,108 +767,14 @@ template <int NBS, int NJ, int CG> struct PanelLds {
 
 constexpr int kPanelLoaders = 4;               // waves of a gemm_panel workgroup that only load
 constexpr int kPanelThreads = (8 + kPanelLoaders) * 64;
-// SPLIT: K in gridDim.y pieces of GemmArgs::split_stages stages; workgroup (t, y) writes the fp32 sums of its piece, scaled,
-// without bias, to slab t * gridDim.y + y of the workspace ([BM][BN] each), and splitk_reduce adds a tile's slabs.
-template <int BLK, int CDT, int NJ, int CG = 1, bool SPLIT = false>
-__global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
-    static_assert(!SPLIT || CDT == BI8_F32, "the slabs are fp32 sums");
-    static_assert(BLK == 128 || BLK == 64, "a K-block is one or two MFMAs of 64 bytes of K");
-    static_assert(NJ >= 1 && NJ <= 4 && (CG == 1 || CG == 2 || CG == 4), "16 ... 64 columns per wave, one, two or four waves side by side");
+// The computing waves of the forms with one 16-row subtile per wave: `wave` = row group rg (16 rows), column group cg
+// (16 * NJ columns).
+template <int BLK, int CDT, int NJ, int CG, bool SPLIT>
+__device__ __forceinline__ void panel_compute_rows(const GemmArgs &g, uint8_t *lds, int wave, int lane, int64_t m0, int64_t n0, int nst) {
     constexpr int NBS = kStageK / BLK;
     using L = PanelLds<NBS, NJ, CG>;
-    constexpr int BM = L::BM, BN = L::BN, RG = 8 / CG;                     // RG = row groups of 16 rows
-    constexpr int kBufs = L::kBufs;
-    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t lds_base = bi8_lds_address(lds);
-    const int tile_m = (int)blockIdx.x / g.tiles_n, tile_n = (int)blockIdx.x - tile_m * g.tiles_n;
-    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
-    const int stage_lo = SPLIT ? (int)blockIdx.y * g.split_stages : 0;          // this workgroup's first stage of K, and how many
-    const int nst = SPLIT ? ((int)(g.K / kStageK) - stage_lo < g.split_stages ? (int)(g.K / kStageK) - stage_lo : g.split_stages)
-                          : (int)(g.K / kStageK);
-    auto wait_vm = [&](auto pending_c) {
-        constexpr int kPending = decltype(pending_c)::value;
-        static_assert(kPending < 64, "vmcnt is a 6-bit field");
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
-    };
+    constexpr int BM = L::BM, BN = L::BN, RG = 8 / CG, kBufs = L::kBufs;     // RG = row groups of 16 rows
     auto next_buf = [](int buf) { return buf + 1 == kBufs ? 0 : buf + 1; };      // the ring's buffer after `buf`
-
-    if (wave >= 8) {
-        // ---- the loading waves.  A stage is a list of wave-instructions: BM / 8 of rows of A and BN / 8 of rows of W (an
-        // instruction covers tile rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which holds source chunk
-        // (lane%8) ^ ((row >> 1) & 7)), then per K-block the row scales and the column scales, 64 floats per instruction.
-        // Loader P takes items P, P + 4, ... (all its row items have the parity of P); which item is of which kind is known
-        // at compile time, one copy of the code per loader.  Stages past the end of K are loaded from beyond the buffers'
-        // ranges (zeros, no memory access), so a loader's count of loads in flight never changes.
-        constexpr int kAItems = BM / 8, kWItems = BN / 8;
-        constexpr int kSAParts = L::kSARow / 64, kSWParts = L::kSWRow / 64, kSParts = kSAParts + kSWParts;
-        constexpr int kItems = kAItems + kWItems + kSParts * NBS, kSlots = (kItems + kPanelLoaders - 1) / kPanelLoaders;
-        static_assert(kAItems % 2 == 0 && kPanelLoaders % 2 == 0, "the swizzle term of a loader's row items does not depend on the slot");
-        static_assert((kBufs - 1) * kSlots < 64, "a loader's loads in flight fit the counter");
-        const int64_t nblk = g.K / BLK;
-        const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM, w_rows = g.N - n0 < BN ? g.N - n0 : BN;
-        const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
-        const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
-        const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
-        const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
-        const uint32_t sa_row = (uint32_t)(g.M * 4), sw_row = (uint32_t)(g.N * 4);          // bytes from one K-block's scales to the next
-        auto loader = [&](auto p_c) {
-            constexpr int P = decltype(p_c)::value;
-            constexpr int kMine = (kItems - P + kPanelLoaders - 1) / kPanelLoaders;          // this loader's items per stage
-            const int ld_row = lane >> 3;
-            const int ld_chunk = (lane & 7) ^ ((4 * (P & 1) + (lane >> 4)) & 7);
-            const uint32_t a_lane = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_lane = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
-            const uint32_t a_item = (uint32_t)(8 * g.lda), w_item = (uint32_t)(8 * g.ldw);  // from one row item to the next
-            const uint32_t s_lane = (uint32_t)(lane * 4);
-            auto issue_stage = [&](int buf, int s) {   // both wave-uniform
-                const bool real = s < nst;
-                const uint32_t k_pos = real ? (uint32_t)((stage_lo + s) * kStageK) : (uint32_t)kBufOut;
-                const uint32_t kb0 = (uint32_t)((stage_lo + s) * NBS);
-#pragma unroll
-                for (int e = 0; e < kMine; ++e) {
-                    constexpr int kA = kAItems, kW = kWItems;
-                    const int item = e * kPanelLoaders + P;            // a constant after unrolling
-                    if (item < kA) {
-                        bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + item * 1024, a_lane, k_pos, (uint32_t)item * a_item);
-                    } else if (item < kA + kW) {
-                        bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (item - kA) * 1024, w_lane, k_pos, (uint32_t)(item - kA) * w_item);
-                    } else {
-                        const int sc = item - kA - kW, kb = sc / kSParts, r = sc % kSParts;
-                        if (r < kSAParts) {
-                            const uint32_t pos = real ? (kb0 + kb) * sa_row + r * 256 : (uint32_t)kBufOut;
-                            bi8_buffer_to_lds4(sa_rsrc, lds_base + L::kSAReg + buf * L::kSABuf + (kb * L::kSARow + r * 64) * 4, s_lane, pos);
-                        } else {
-                            const uint32_t pos = real ? (kb0 + kb) * sw_row + (r - kSAParts) * 256 : (uint32_t)kBufOut;
-                            bi8_buffer_to_lds4(sw_rsrc, lds_base + L::kSWReg + buf * L::kSWBuf + (kb * L::kSWRow + (r - kSAParts) * 64) * 4, s_lane, pos);
-                        }
-                    }
-                }
-            };
-#pragma unroll
-            for (int s = 0; s < kBufs - 1; ++s) issue_stage(s, s);
-            wait_vm(std::integral_constant<int, (kBufs - 2) * kMine>{});                 // stage 0 has landed
-            __syncthreads();
-            int fill = kBufs - 1;
-            for (int s = 0; s < nst; ++s) {
-                wait_vm(std::integral_constant<int, (kBufs - 3) * kMine>{});             // stage s + 1 has landed
-                __syncthreads();                   // ... for every loader: published; and the computing waves have left stage s - 1
-                issue_stage(fill, s + kBufs - 1);
-                fill = next_buf(fill);
-            }
-            wait_vm(std::integral_constant<int, 0>{});     // (the loads past the end of K) nothing may still be writing LDS when the wave ends
-        };
-        static_assert(kPanelLoaders == 4, "one copy of the loader per loading wave");
-        if (wave == 8) loader(std::integral_constant<int, 0>{});
-        else if (wave == 9) loader(std::integral_constant<int, 1>{});
-        else if (wave == 10) loader(std::integral_constant<int, 2>{});
-        else loader(std::integral_constant<int, 3>{});
-        return;
-    }
-
-    // ---- the computing waves: `wave` = row group rg (16 rows), column group cg (16 * NJ columns)
     const int rg = wave % RG, cg = wave / RG;
     const int r16 = lane & 15, q = lane >> 4;
     // operand fragments: lane -> row r16 of a 16-row subtile, 16-byte chunk 4*kb + q of the stage's eight, stored at chunk
@@ -987,6 +894,272 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
             }
         }
     }
+}
+
+// The computing waves of the square form (NI = 2): 4 x 2 waves, each 32 rows x 16 * NJ columns as 2 x NJ subtiles, a tile of
+// 128 rows x 32 * NJ columns.  Per byte read from LDS a wave does twice the MFMAs of the one-subtile-high forms (a stage's
+// fragment reads are what bounds those at 64 columns per wave).  To stay within the 168 registers that twelve waves leave
+// each lane, the int32 partials are double-buffered by HALF stages, and the next stage's fragments are read in two parts, each
+// right behind the MFMAs that were the last to read the registers it goes into, so that the LDS reads run under MFMAs and
+// folds (the order of a stage: at `step` below).
+template <int BLK, int CDT, int NJ, bool SPLIT>
+__device__ __forceinline__ void panel_compute_square(const GemmArgs &g, uint8_t *lds, int wave, int lane, int64_t m0, int64_t n0, int nst) {
+    constexpr int NBS = kStageK / BLK, NI = 2, CG = 2, RG = 4, NH = NJ / 2;
+    using L = PanelLds<NBS, NJ, CG, NI>;
+    constexpr int BM = L::BM, BN = L::BN, kBufs = L::kBufs;
+    auto next_buf = [](int buf) { return buf + 1 == kBufs ? 0 : buf + 1; };
+    const int rg = wave % RG, cg = wave / RG;
+    const int r16 = lane & 15, q = lane >> 4;
+    int a_base = L::kAReg + (rg * 16 * NI + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
+    int w_base = L::kWReg + (cg * 16 * NJ + r16) * kStageK + ((q ^ (r16 >> 1)) << 4);
+    int sa_base = L::kSAReg + (rg * 16 * NI + 4 * q) * 4;
+    int sw_base = L::kSWReg + (cg * 16 * NJ + r16) * 4;
+    asm volatile("" : "+v"(a_base), "+v"(w_base), "+v"(sa_base), "+v"(sw_base));
+    constexpr int kMagicBits = 0x4B400000;        // bit pattern of 1.5 * 2^23
+    const bi8_v4i magic = {kMagicBits, kMagicBits, kMagicBits, kMagicBits};
+
+    float acc[NI][NJ][4];
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.0f;
+    bi8_v4i A[NI][2], B[NJ][2];                    // [subtile][kb]: the current stage's operands
+    bi8_v4i c[2][NBS][NI][NH];                     // [half of the columns][K-block][row subtile][column subtile of the half]
+    bi8_v4f sx[2][NBS][NI];                        // [stage parity][K-block][row subtile]: row scales
+    float bw[2][NBS][NJ];                          // ... [column subtile]: column scales
+
+    auto read_a = [&](int buf) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < NI; ++i) A[i][kb] = *(const bi8_v4i *)(lds + (a_base ^ (kb * 64)) + buf * L::kABuf + i * 16 * kStageK);
+    };
+    auto read_b = [&](int buf, auto half_c) {      // the W fragments of one half of the columns
+        constexpr int H = decltype(half_c)::value;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int jj = 0; jj < NH; ++jj)
+                B[H * NH + jj][kb] = *(const bi8_v4i *)(lds + (w_base ^ (kb * 64)) + buf * L::kWBuf + (H * NH + jj) * 16 * kStageK);
+    };
+    auto read_scales = [&](int buf, auto par_c) {
+        constexpr int P = decltype(par_c)::value;
+#pragma unroll
+        for (int kb = 0; kb < NBS; ++kb) {
+#pragma unroll
+            for (int i = 0; i < NI; ++i) sx[P][kb][i] = *(const bi8_v4f *)(lds + sa_base + buf * L::kSABuf + (kb * L::kSARow + i * 16) * 4);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) bw[P][kb][j] = *(const float *)(lds + sw_base + buf * L::kSWBuf + (kb * L::kSWRow + j * 16) * 4);
+        }
+    };
+    auto mfmas = [&](auto half_c) {
+        constexpr int H = decltype(half_c)::value;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+                for (int jj = 0; jj < NH; ++jj) {
+                    const int blk = NBS == 2 ? kb : 0;
+                    const bool first = NBS == 2 || kb == 0;
+                    c[H][blk][i][jj] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[i][kb], B[H * NH + jj][kb], first ? magic : c[H][blk][i][jj], 0, 0, 0);
+                }
+    };
+    // half H of a stage (its scales in parity P) into the accumulators: per K-block and subtile four products, then four accumulations
+    auto fold = [&](auto half_c, auto par_c) {
+        constexpr int H = decltype(half_c)::value, P = decltype(par_c)::value;
+#pragma unroll
+        for (int kb = 0; kb < NBS; ++kb)
+#pragma unroll
+            for (int jj = 0; jj < NH; ++jj) {
+                const float b = bi8_u2f((bi8_f2u(bw[P][kb][H * NH + jj]) + 2u) & ~3u);      // 22 significant bits: -(1.5*2^23)*b is exact
+                const float cm = -BI8_MAGIC * b;
+#pragma unroll
+                for (int i = 0; i < NI; ++i) {
+                    float t[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) t[r] = __builtin_fmaf(bi8_u2f((uint32_t)c[H][kb][i][jj][r]), b, cm);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[i][H * NH + jj][r] = __builtin_fmaf(t[r], sx[P][kb][i][r], acc[i][H * NH + jj][r]);
+                }
+            }
+    };
+    using H0 = std::integral_constant<int, 0>;
+    using H1 = std::integral_constant<int, 1>;
+    // stage s (its operands in A and B, its scales in parity P): the barrier that publishes stage s + 1; the MFMAs of the left
+    // columns, behind them the left W fragments of stage s + 1 into the registers they have just read; the fold of the right
+    // columns of stage s - 1; the MFMAs of the right columns, behind them the A and the right W fragments of stage s + 1; the
+    // fold of the left columns; the scales of stage s + 1 into the registers that held those of stage s - 1
+    int buf = 0;
+    auto step = [&](auto par_c, bool fold_prev) {
+        constexpr int P = decltype(par_c)::value;
+        using Q = std::integral_constant<int, 1 - P>;
+        __syncthreads();
+        buf = next_buf(buf);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(H0{});
+        __builtin_amdgcn_sched_barrier(0);
+        read_b(buf, H0{});
+        __builtin_amdgcn_sched_barrier(0);
+        if (fold_prev) fold(H1{}, Q{});
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(H1{});
+        __builtin_amdgcn_sched_barrier(0);
+        read_a(buf);
+        read_b(buf, H1{});
+        __builtin_amdgcn_sched_barrier(0);
+        fold(H0{}, par_c);
+        __builtin_amdgcn_sched_barrier(0);
+        read_scales(buf, Q{});
+    };
+
+    __syncthreads();                               // stage 0 is published
+    read_a(0);
+    read_b(0, H0{});
+    read_b(0, H1{});
+    read_scales(0, std::integral_constant<int, 0>{});
+    step(std::integral_constant<int, 0>{}, false);
+    int s = 1;
+    for (; s + 1 < nst; s += 2) {
+        step(std::integral_constant<int, 1>{}, true);
+        step(std::integral_constant<int, 0>{}, true);
+    }
+    if (s < nst) {                                 // an even number of stages: one more, of odd parity
+        step(std::integral_constant<int, 1>{}, true);
+        fold(H1{}, std::integral_constant<int, 1>{});
+    } else {
+        fold(H1{}, std::integral_constant<int, 0>{});
+    }
+
+    const float div = (float)(1.0 / (127.0 * 127.0));
+    const bool has_bias = !SPLIT && g.bias != nullptr;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int64_t n = n0 + cg * 16 * NJ + j * 16 + r16;
+        const bool n_ok = n < g.N;
+        const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < NI; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = rg * 16 * NI + i * 16 + 4 * q + r;
+                const int64_t m = m0 + row;
+                if constexpr (SPLIT) {
+                    float *slab = g.ws + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * (BM * BN);
+                    if (n_ok && m < g.M) slab_store(slab + row * BN + cg * 16 * NJ + j * 16 + r16, acc[i][j][r] * div);
+                } else {
+                    if (n_ok && m < g.M) store_c<CDT>(g.C, m * g.ldc + n, acc[i][j][r] * div, has_bias, bias);
+                }
+            }
+    }
+}
+
+// SPLIT: K in gridDim.y pieces of GemmArgs::split_stages stages; workgroup (t, y) writes the fp32 sums of its piece, scaled,
+// without bias, to slab t * gridDim.y + y of the workspace ([BM][BN] each), and splitk_reduce adds a tile's slabs.
+template <int BLK, int CDT, int NJ, int CG = 1, bool SPLIT = false, int NI = 1>
+__global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
+    static_assert(!SPLIT || CDT == BI8_F32, "the slabs are fp32 sums");
+    static_assert(BLK == 128 || BLK == 64, "a K-block is one or two MFMAs of 64 bytes of K");
+    static_assert(NJ >= 1 && NJ <= 4 && (CG == 1 || CG == 2 || CG == 4), "16 ... 64 columns per wave, one, two or four waves side by side");
+    static_assert(NI == 1 || (NI == 2 && CG == 2 && NJ % 2 == 0), "two row subtiles per wave: the square form, its columns in two halves");
+    constexpr int NBS = kStageK / BLK;
+    using L = PanelLds<NBS, NJ, CG, NI>;
+    constexpr int BM = L::BM, BN = L::BN;
+    constexpr int kBufs = L::kBufs;
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t lds_base = bi8_lds_address(lds);
+    const int tile_m = (int)blockIdx.x / g.tiles_n, tile_n = (int)blockIdx.x - tile_m * g.tiles_n;
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int stage_lo = SPLIT ? (int)blockIdx.y * g.split_stages : 0;          // this workgroup's first stage of K, and how many
+    const int nst = SPLIT ? ((int)(g.K / kStageK) - stage_lo < g.split_stages ? (int)(g.K / kStageK) - stage_lo : g.split_stages)
+                          : (int)(g.K / kStageK);
+    auto wait_vm = [&](auto pending_c) {
+        constexpr int kPending = decltype(pending_c)::value;
+        static_assert(kPending < 64, "vmcnt is a 6-bit field");
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (kPending & 15) | ((kPending >> 4) << 14));
+    };
+    auto next_buf = [](int buf) { return buf + 1 == kBufs ? 0 : buf + 1; };      // the ring's buffer after `buf`
+
+    if (wave >= 8) {
+        // ---- the loading waves.  A stage is a list of wave-instructions: BM / 8 of rows of A and BN / 8 of rows of W (an
+        // instruction covers tile rows 8i .. 8i+7, lane -> row 8i + lane/8, LDS chunk lane%8, which holds source chunk
+        // (lane%8) ^ ((row >> 1) & 7)), then per K-block the row scales and the column scales, 64 floats per instruction.
+        // Loader P takes items P, P + 4, ... (all its row items have the parity of P); which item is of which kind is known
+        // at compile time, one copy of the code per loader.  Stages past the end of K are loaded from beyond the buffers'
+        // ranges (zeros, no memory access), so a loader's count of loads in flight never changes.
+        constexpr int kAItems = BM / 8, kWItems = BN / 8;
+        constexpr int kSAParts = L::kSARow / 64, kSWParts = L::kSWRow / 64, kSParts = kSAParts + kSWParts;
+        constexpr int kItems = kAItems + kWItems + kSParts * NBS, kSlots = (kItems + kPanelLoaders - 1) / kPanelLoaders;
+        static_assert(kAItems % 2 == 0 && kPanelLoaders % 2 == 0, "the swizzle term of a loader's row items does not depend on the slot");
+        static_assert((kBufs - 1) * kSlots < 64, "a loader's loads in flight fit the counter");
+        const int64_t nblk = g.K / BLK;
+        const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM, w_rows = g.N - n0 < BN ? g.N - n0 : BN;
+        const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
+        const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
+        const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
+        const bi8_rsrc sw_rsrc = bi8_make_rsrc(g.sW + n0, ((nblk - 1) * g.N + (g.N - n0)) * 4);
+        const uint32_t sa_row = (uint32_t)(g.M * 4), sw_row = (uint32_t)(g.N * 4);          // bytes from one K-block's scales to the next
+        auto loader = [&](auto p_c) {
+            constexpr int P = decltype(p_c)::value;
+            constexpr int kMine = (kItems - P + kPanelLoaders - 1) / kPanelLoaders;          // this loader's items per stage
+            const int ld_row = lane >> 3;
+            const int ld_chunk = (lane & 7) ^ ((4 * (P & 1) + (lane >> 4)) & 7);
+            const uint32_t a_lane = (uint32_t)(ld_row * g.lda + ld_chunk * 16), w_lane = (uint32_t)(ld_row * g.ldw + ld_chunk * 16);
+            const uint32_t a_item = (uint32_t)(8 * g.lda), w_item = (uint32_t)(8 * g.ldw);  // from one row item to the next
+            const uint32_t s_lane = (uint32_t)(lane * 4);
+            auto issue_stage = [&](int buf, int s) {   // both wave-uniform
+                const bool real = s < nst;
+                const uint32_t k_pos = real ? (uint32_t)((stage_lo + s) * kStageK) : (uint32_t)kBufOut;
+                const uint32_t kb0 = (uint32_t)((stage_lo + s) * NBS);
+#pragma unroll
+                for (int e = 0; e < kMine; ++e) {
+                    constexpr int kA = kAItems, kW = kWItems;
+                    const int item = e * kPanelLoaders + P;            // a constant after unrolling
+                    if (item < kA) {
+                        bi8_buffer_to_lds16_sum(a_rsrc, lds_base + L::kAReg + buf * L::kABuf + item * 1024, a_lane, k_pos, (uint32_t)item * a_item);
+                    } else if (item < kA + kW) {
+                        bi8_buffer_to_lds16_sum(w_rsrc, lds_base + L::kWReg + buf * L::kWBuf + (item - kA) * 1024, w_lane, k_pos, (uint32_t)(item - kA) * w_item);
+                    } else {
+                        const int sc = item - kA - kW, kb = sc / kSParts, r = sc % kSParts;
+                        if (r < kSAParts) {
+                            const uint32_t pos = real ? (kb0 + kb) * sa_row + r * 256 : (uint32_t)kBufOut;
+                            bi8_buffer_to_lds4(sa_rsrc, lds_base + L::kSAReg + buf * L::kSABuf + (kb * L::kSARow + r * 64) * 4, s_lane, pos);
+                        } else {
+                            const uint32_t pos = real ? (kb0 + kb) * sw_row + (r - kSAParts) * 256 : (uint32_t)kBufOut;
+                            bi8_buffer_to_lds4(sw_rsrc, lds_base + L::kSWReg + buf * L::kSWBuf + (kb * L::kSWRow + (r - kSAParts) * 64) * 4, s_lane, pos);
+                        }
+                    }
+                }
+            };
+#pragma unroll
+            for (int s = 0; s < kBufs - 1; ++s) issue_stage(s, s);
+            wait_vm(std::integral_constant<int, (kBufs - 2) * kMine>{});                 // stage 0 has landed
+            __syncthreads();
+            int fill = kBufs - 1;
+            for (int s = 0; s < nst; ++s) {
+                wait_vm(std::integral_constant<int, (kBufs - 3) * kMine>{});             // stage s + 1 has landed
+                __syncthreads();                   // ... for every loader: published; and the computing waves have left stage s - 1
+                issue_stage(fill, s + kBufs - 1);
+                fill = next_buf(fill);
+            }
+            wait_vm(std::integral_constant<int, 0>{});     // (the loads past the end of K) nothing may still be writing LDS when the wave ends
+        };
+        static_assert(kPanelLoaders == 4, "one copy of the loader per loading wave");
+        if (wave == 8) loader(std::integral_constant<int, 0>{});
+        else if (wave == 9) loader(std::integral_constant<int, 1>{});
+        else if (wave == 10) loader(std::integral_constant<int, 2>{});
+        else loader(std::integral_constant<int, 3>{});
+        return;
+    }
+
+    if constexpr (NI == 2) panel_compute_square<BLK, CDT, NJ, SPLIT>(g, lds, wave, lane, m0, n0, nst);
+    else panel_compute_rows<BLK, CDT, NJ, CG, SPLIT>(g, lds, wave, lane, m0, n0, nst);
 }
 
 // ---- 256x256 tile, block 128 ------------------------------------------------------------------------------------
@@ -2616,6 +2789,8 @@ constexpr int64_t kPanelSplitFewRowsMinStages = 64, kPanelSplitFewRowsTwoStages 
 constexpr int64_t kPanelSplitFewRowsMinGroups = 192;                                       // ... and this many workgroups
 constexpr int64_t kPanelSplit64RowsMinStages = 40, kPanelSplit64RowsMaxTiles = 32;         // on tiles of 64 rows: K from 5120 on, up to 2048 columns
 constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024
+constexpr int64_t kPanelSquareSplitMinTiles = 100, kPanelSquareSplitMinStages = 64;     // the square form on two pieces of K: 100 ... 128 tiles, K from 8192 on
+constexpr int64_t kPanelSquareMinTiles = 176;  // the square form outright from this many tiles on; with fewer only where nothing splits K
 constexpr int64_t kPanelFewRows = 32;          // up to 32 rows: tiles of 32 rows x (64 ... 256) columns ...
 constexpr int64_t kPanelFewRowsMinCols = 6144; // ... from this many columns on (fewer leave most CUs without a tile)
 // the widest tile, in 16-column subtiles (block 64 at 64 columns needs more registers than a wave has)
@@ -2647,6 +2822,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     if (!tile_ok) return p;
     // few tiles and scratch memory: split K over the workgroups, then sum the slabs
     bool panel_if_no_split = false;                // gemm_panel's tiles would give one round, but K is beyond what it is given outright
+    bool square_if_no_split = false;               // its square tiles would, but they are few enough that a split of K may be ahead
     auto try_split = [&](bool few_rows_split = false) {
         if (partials || ws_bytes <= 0) return false;
         // 65 ... 128 rows and K up to 12288: gemm_panel on pieces of K, tiles of 128 rows x 64 columns (block 64: 32).  Measured
@@ -2689,6 +2865,25 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
             }
         }
         if (few_rows_split) return false;          // (asked ahead of gemv_staged: only for that rule)
+        // more than 128 rows, 100 to 128 square tiles (128 x 128, block 64: 128 x 64) and K from 8192 on: two pieces per tile on
+        // gemm_panel's square form.  Measured against the split 256x128 tiles, block 128, W from HBM, us at K = 8192 / 11008 /
+        // 16384: 512 x 4096 38.2 -> 34.0, 45.2 -> 42.7, 59.2 -> 56.4; 1024 x 2048 37.7 -> 33.1, 45.5 -> 43.7, 59.6 -> 55.7; 256 x 8192
+        // 39.1 -> 35.7, 47.1 -> 47.0, 62.8 -> 60.9.  With fewer tiles and more pieces it is level with or behind the split tile
+        // kernels (256 x 4096: 25.9 -> 26.5, 30.5 -> 31.7; 512 x 1024: 21.2 -> 18.4, 22.3 -> 21.3, 25.0 -> 28.7): not taken there.
+        if (block != 32 && M > 128 && !rest_of_cut && K / kStageK >= kPanelSquareSplitMinStages && (K / block + 1) * max_mn * 4 < kBufOut) {
+            const int64_t bn = block == 64 ? 64 : 128, t = ((M + 127) / 128) * ((N + bn - 1) / bn), nst = K / kStageK;
+            if (t >= kPanelSquareSplitMinTiles && t <= kCus / 2) {
+                const int64_t stages = (nst + 1) / 2, need = t * 2 * 128 * bn * 4;
+                if (need <= ws_bytes) {
+                    p.kernel = kKSplitPanel;
+                    p.splits = (int)(t * 2);
+                    p.split_stages = (int)stages;
+                    p.split_per_tile = 2;
+                    p.ws_need = need;
+                    return true;
+                }
+            }
+        }
         // 256x128 tiles on gemm_wide's loop, split evenly, where that puts most of the CUs to work
         if (block != 32 && M > 128 && wide_addressable(M, N, K, lda, ldw, block)) {
             const int64_t t = ((M + 255) / 256) * ((N + 127) / 128), nst = K / kStageK;
@@ -2775,6 +2970,20 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
                 p.kernel = kKPanel;
                 return p;
             }
+            // more rows of tiles than that: the square form, tiles of 128 x 128 (block 64: 128 x 64), where that is one round.
+            // Measured against the 128x128 tile kernel, W from HBM, us: block 128 1024 x 4096 x 1024 / 4096 / 11008 12.7 -> 11.2,
+            // 33.1 -> 28.2, 74.2 -> 61.7; 256 x 11008 x 4096 27.5 -> 26.0; 1024 x 3072 x 16384 (split) 89.0 -> 74.9; block 64
+            // 512 x 4096 x 768 / 4096 9.9 -> 7.1, 25.7 -> 19.4; 1024 x 2048 x 3072 22.9 -> 15.5.  With fewer than 176 tiles a split
+            // of K, where the rules below find one, is level or ahead (1024 x 2176 x 8192 / 11008 / 16384, 136 tiles, against
+            // the split 256x128 tiles: 41.5 -> 40.1, 50.1 -> 60.9, 68.1 -> 68.4; 160 tiles: 42.1 -> 38.3, 52.6 -> 56.7, 70.4 -> 68.9).
+            if (!one_round && M > 128) {
+                const int64_t bn = block == 64 ? 64 : 128, sq = rows * ((N + bn - 1) / bn);
+                if (sq <= kCus && sq >= kPanelSquareMinTiles) {
+                    p.kernel = kKPanel;
+                    return p;
+                }
+                square_if_no_split = sq <= kCus;
+            }
             panel_if_no_split = one_round;
         }
         if (M <= 32) {
@@ -2834,7 +3043,7 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
     // a long K and nothing to split it with (no scratch memory, or too little): one round of narrow tiles is still ahead of a
     // few 128x128 tiles (measured without scratch memory, block 128, us, K = 8192 / 16384: 128 x 768 45.0 -> 13.9, 88.6 -> 35.9;
     // 128 x 11008 48.7 -> 32.2, 90.3 -> 57.6; 512 x 4096 49.7 -> 34.9, 88.5 -> 63.2; 1024 x 256 at K = 32768 167 -> 53)
-    if (panel_if_no_split) {
+    if (panel_if_no_split || square_if_no_split) {     // (the square tiles: 12-18 % ahead of the 128x128 tile kernel on the same grid)
         p.kernel = kKPanel;
         return p;
     }
@@ -2876,11 +3085,11 @@ template <int BLK, int CDT> int launch_staged(const GemmArgs &g, hipStream_t st)
 }
 
 // gemm_panel on the narrowest tiles that give at most one per CU
-template <int BLK, int CDT, int NJ, int CG> int launch_panel_as(GemmArgs g, hipStream_t st) {
-    using L = PanelLds<kStageK / BLK, NJ, CG>;
+template <int BLK, int CDT, int NJ, int CG, int NI = 1> int launch_panel_as(GemmArgs g, hipStream_t st) {
+    using L = PanelLds<kStageK / BLK, NJ, CG, NI>;
     g.tiles_m = (int)((g.M + L::BM - 1) / L::BM);
     g.tiles_n = (int)((g.N + L::BN - 1) / L::BN);
-    auto kern = gemm_panel<BLK, CDT, NJ, CG>;
+    auto kern = gemm_panel<BLK, CDT, NJ, CG, false, NI>;
     static LdsOptIn opted;                         // one per kernel instantiation
     const int rc = opted.ensure((const void *)kern, L::kBytes);
     if (rc != BI8_OK) return rc;
@@ -2897,13 +3106,13 @@ template <int BLK, int CDT, int CG> int launch_panel_cg(const GemmArgs &g, hipSt
     return BI8_ERR_UNSUPPORTED;                    // (the plan sends no other problem here)
 }
 // the split form: tiles of 128 rows x 64 columns (block 64: 32), split_per_tile pieces of split_stages stages each, then the sum
-template <int BLK, int CDT, int NJ, int CG> int launch_panel_split_as(GemmArgs g, hipStream_t st) {
-    using L = PanelLds<kStageK / BLK, NJ, CG>;
+template <int BLK, int CDT, int NJ, int CG, int NI = 1> int launch_panel_split_as(GemmArgs g, hipStream_t st) {
+    using L = PanelLds<kStageK / BLK, NJ, CG, NI>;
     g.tiles_m = (int)((g.M + L::BM - 1) / L::BM);
     g.tiles_n = (int)((g.N + L::BN - 1) / L::BN);
     g.tile_m0 = g.tile_n0 = 0;
     if (g.split_per_tile < 2 || g.split_per_tile > kSplitMax || (int64_t)g.tiles_m * g.tiles_n * g.split_per_tile > 2 * kCus) return BI8_ERR_UNSUPPORTED;
-    auto kern = gemm_panel<BLK, BI8_F32, NJ, CG, true>;
+    auto kern = gemm_panel<BLK, BI8_F32, NJ, CG, true, NI>;
     static LdsOptIn opted;                         // one per kernel instantiation
     const int rc = opted.ensure((const void *)kern, L::kBytes);
     if (rc != BI8_OK) return rc;
@@ -2913,14 +3122,19 @@ template <int BLK, int CDT, int NJ, int CG> int launch_panel_split_as(GemmArgs g
     hipLaunchKernelGGL((splitk_reduce<CDT, L::BM, L::BN>), dim3((unsigned)(g.tiles_m * g.tiles_n), L::BM / (256 / (L::BN / 4))), dim3(256), 0, st, g);
     return bi8_launch_rc();
 }
-// (the tiles the plan has counted: 32 rows x 64 columns up to 32 rows, 64 x 64 up to 64, else 128 x 64, at block 64 128 x 32)
+// (the tiles the plan has counted: 32 rows x 64 columns up to 32 rows, 64 x 64 up to 64, 128 x 64 -- at block 64 128 x 32 -- up to
+// 128, and beyond that the square form's 128 x 128, at block 64 128 x 64)
 template <int BLK, int CDT> int launch_panel_split(const GemmArgs &g, hipStream_t st) {
     if (g.M <= kPanelFewRows) return launch_panel_split_as<BLK, CDT, 1, 4>(g, st);
     if (g.M <= kPanelMinRows) return launch_panel_split_as<BLK, CDT, 2, 2>(g, st);
+    if (g.M > 128) return launch_panel_split_as<BLK, CDT, BLK == 64 ? 2 : 4, 2, 2>(g, st);
     return launch_panel_split_as<BLK, CDT, BLK == 64 ? 2 : 4, 1>(g, st);
 }
 template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) {
     if (g.M <= kPanelFewRows) return launch_panel_cg<BLK, CDT, 4>(g, st);
+    // (more rows of narrow tiles than one round: the plan has counted the square form's)
+    if (g.M > 128 && ((g.M + 127) / 128) * ((g.N + 16 * panel_max_subtiles(BLK) - 1) / (16 * panel_max_subtiles(BLK))) > kCus)
+        return launch_panel_as<BLK, CDT, BLK == 64 ? 2 : 4, 2, 2>(g, st);
     return g.M <= 64 ? launch_panel_cg<BLK, CDT, 2>(g, st) : launch_panel_cg<BLK, CDT, 1>(g, st);
 }
 

@@ -240,14 +240,24 @@ def test_kernel_choice_by_shape():
     assert name(2048, 4096, 4096, 128) == "gemm_wide_256x128"        # 128 tiles of 256x256: one round of 256x128 tiles
     assert name(2048, 4096, 512, 64) == "gemm_wide_256x128" and name(2048, 2304, 512, 64) == "gemm_wide_256x128"
     assert name(2048, 4096, 4096, 128, 0, 1 << 21, 4096) == "gemm_tile_256x128"     # rows 2 MiB apart: beyond its 32-bit offsets
-    assert name(1500, 1500, 512, 128) == "gemm_tile_128x128" and name(48, 5000, 640, 32) == "gemm_tile_64x128"
+    assert name(1500, 1500, 512, 32) == "gemm_tile_128x128" and name(48, 5000, 640, 32) == "gemm_tile_64x128"
+    assert name(1024, 3072, 4096, 64) == "gemm_tile_128x128"         # block 64: 384 tiles of 128 x 64 are more than one round of the square form
+    # more than 128 rows, more narrow tiles than one round, at most 256 tiles of 128 x 128 (block 64: 128 x 64): gemm_panel's square form
+    assert name(1024, 4096, 4096, 128) == "gemm_panel" and name(256, 11008, 4096, 128, 1 << 30) == "gemm_panel" and name(1024, 4096, 16384, 128, 1 << 30) == "gemm_panel"
+    assert name(512, 4096, 4096, 64, 1 << 30) == "gemm_panel" and name(1024, 2048, 3072, 64) == "gemm_panel" and name(2048, 1024, 768, 64) == "gemm_panel"
+    assert name(1500, 1500, 512, 128) == "gemm_panel" and name(1500, 1500, 16384, 128) == "gemm_panel"     # 144 tiles: where nothing splits K
+    assert name(1500, 1500, 16384, 128, 1 << 30) == "gemm_wide_256x128_splitk" and name(1500, 1500, 16384, 32, 1 << 30) == "gemm_tile_128x128_splitk"
+    # ... and on two pieces of K for 100 to 128 such tiles and K from 8192 on
+    assert name(512, 4096, 11008, 128, 1 << 30) == "gemm_panel_splitk" and name(1024, 2048, 8192, 128, 1 << 30) == "gemm_panel_splitk"
+    assert name(1024, 1024, 8192, 64, 1 << 30) == "gemm_panel_splitk" and name(512, 4096, 8064, 128, 1 << 30) == "gemm_wide_256x128_splitk"
+    assert name(512, 3072, 11008, 128, 1 << 30) == "gemm_wide_256x128_splitk"      # 96 tiles
     # more than 64 rows, at most one tile of 128 x (16 ... 64) per CU and K up to 4096: narrow tiles, the whole K in one workgroup
     assert name(300, 500, 512, 128) == "gemm_panel" and name(128, 4096, 4096, 128) == "gemm_panel" and name(65, 64, 128, 64) == "gemm_panel"
     assert name(128, 4096, 4096, 128, 1 << 30) == "gemm_panel" and name(512, 4096, 4096, 128, 1 << 30) == "gemm_panel"
     assert name(128, 11008, 4096, 64, 1 << 30) == "gemm_panel" and name(1024, 2048, 4096, 128) == "gemm_panel"
     assert name(128, 1024, 4096, 128) == "gemm_panel" and name(128, 16, 4096, 128, 1 << 30) == "gemm_panel"      # however few the tiles
     assert name(128, 4096, 4224, 128, 1 << 30) == "gemm_panel_splitk" and name(256, 4096, 4224, 128, 1 << 30) == "gemm_tile_128x128_splitk"   # a longer K: split, given scratch memory
-    assert name(512, 4096, 4096, 64) == "gemm_tile_128x128"          # block 64 stops at 48 columns: 4 x 86 tiles are more than one round
+    assert name(512, 4096, 4096, 64) == "gemm_panel"                 # block 64 stops at 48 columns, 4 x 86 tiles are more than one round: the square form
     assert name(300, 500, 512, 32) == "gemm_tile_128x128"            # block 32: not its
     # 33 to 64 rows: the same on tiles of 64 rows x 32 ... 128 columns, where gemv_staged (below) does not apply or K is at most 1024
     assert name(64, 5000, 640, 128) == "gemm_panel" and name(48, 11008, 4096, 128, 1 << 30) == "gemm_panel" and name(33, 16384, 4096, 64) == "gemm_panel"
@@ -285,12 +295,12 @@ def test_kernel_choice_by_shape():
     assert name(128, 4096, 8192, 128) == "gemm_panel" and name(128, 32768, 8192, 128) == "gemm_tile_128x128"   # no scratch memory: one pass
     # few tiles of 256x128 and a long K: pieces of every tile on the 256x256 kernel's loop (the GPT-2 grad-weight GEMMs)
     assert name(3072, 768, 8192, 64, 1 << 25) == "gemm_wide_256x128_splitk" and name(3072, 768, 8192, 64) == "gemm_tile_128x128"
-    assert name(1024, 4096, 4096, 128, 1 << 25) == "gemm_tile_128x128"        # two pieces of 16 stages: the slabs would cost more
+    assert name(1024, 4096, 4096, 128, 1 << 25) == "gemm_panel"               # 256 tiles of 128 x 128: nothing to split
     ws = lib.bi8_gemm_workspace_bytes(128, 2048, 16384, 128)
     # 32 tiles of 64x128, eight workgroups each: one fp32 slab of a tile per workgroup
     assert ws == 8 * 128 * 2048 * 4 and name(128, 2048, 16384, 128, ws) == "gemm_tile_64x128_splitk"
     assert name(128, 2048, 16384, 128, ws - 1) == "gemm_panel"            # too small a workspace is not used: one pass on narrow tiles
-    assert name(512, 4096, 8192, 128, 1 << 30) == "gemm_wide_256x128_splitk" and name(512, 4096, 4096, 64, 1 << 30) == "gemm_tile_128x128_splitk"
+    assert name(256, 4096, 11008, 128, 1 << 30) == "gemm_tile_128x128_splitk"         # 64 tiles, four pieces each
     # 144 tiles of 128x128: runs that end inside tiles fill the chip when K is long enough to pay for the second kernel
     assert name(3072, 768, 8192, 32, 1 << 30) == "gemm_tile_128x128_splitk" and name(3072, 768, 2048, 32, 1 << 30) == "gemm_tile_128x128"
     assert name(2048, 1408, 16384, 64, 1 << 30) == "gemm_tile_128x128_splitk"      # 176 tiles: too many for pieces of 256x128 tiles

@@ -81,19 +81,22 @@ def test_split_matches_checker_and_one_pass(lib, M, N, K, block, out):
 
 @pytest.mark.parametrize("M,N,K,block,kernel", [
     # 129 to 255 tiles of 128x128 and a long K: 256 workgroups, each a run of (tile, stage) pairs that ends inside a tile
-    (2048, 1408, 16384, 64, "gemm_tile_128x128_splitk"), (2000, 1400, 16384, 128, "gemm_tile_128x128_splitk"),
+    (2048, 1408, 16384, 64, "gemm_tile_128x128_splitk"), (1900, 1400, 16384, 128, "gemm_tile_128x128_splitk"),
     (3000, 700, 8192, 32, "gemm_tile_128x128_splitk"),
-    # few tiles of 256x128 and a long K: three or four pieces per tile on the 256x256 kernel's loop (72 tiles x 3 pieces of 22,
-    # 22 and 20 stages; 77 x 3 pieces of 44, 44, 40; 54 x 4 of 16 stages, ragged edges)
+    # few tiles of 256x128 and a long K: three pieces per tile on the 256x256 kernel's loop (72 tiles x 3 pieces of 22,
+    # 22 and 20 stages; 77 x 3 pieces of 44, 44, 40)
     (3072, 768, 8192, 64, "gemm_wide_256x128_splitk"), (1700, 1300, 16384, 128, "gemm_wide_256x128_splitk"),
-    (2200, 700, 8192, 128, "gemm_wide_256x128_splitk")])
+    # 100 to 128 tiles of 128x128 and K from 8192 on: two pieces per tile on gemm_panel's square form (18 x 6 tiles, ragged edges)
+    (2200, 700, 8192, 128, "gemm_panel_splitk")])
 def test_more_tiles_than_half_the_chip(lib, M, N, K, block, kernel):
     """The splits of problems that fill more than half of the chip with tiles.  The checker on sampled rows (every row of
     tiles is hit), the one-pass kernel on everything."""
     A, W, sa, sw, bias = _problem(M, N, K, block, seed=M + N + K)
     want = lib.bi8_gemm_workspace_bytes(M, N, K, block)
     assert lib.bi8_gemm_kernel_name(M, N, K, K, K, block, want).decode() == kernel
-    if "wide" in kernel:
+    if "panel" in kernel:
+        assert want == -(-M // 128) * -(-N // 128) * 2 * 128 * 128 * 4
+    elif "wide" in kernel:
         tiles = -(-M // 256) * -(-N // 128)
         assert want % (256 * 128 * 4) == 0 and 160 <= want // (256 * 128 * 4) <= 256 and (want // (256 * 128 * 4)) % tiles == 0
     else:

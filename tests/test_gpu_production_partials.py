@@ -101,7 +101,8 @@ CASES = [
     # software-pipelined block-128 instantiation, and its three-buffer form at block 64 (sixth entry: row pitch of A)
     (600, 11008, 256, 128, "gemm_tile_256x128", (1 << 22) - 128),
     (600, 11008, 256, 64, "gemm_tile_256x128", (1 << 22) - 128),
-    (1500, 1500, 512, 128, "gemm_tile_128x128"),
+    (1500, 1500, 512, 32, "gemm_tile_128x128"),
+    (1024, 3072, 640, 64, "gemm_tile_128x128"),     # block 64: more tiles of 128 x 64 than one round of gemm_panel's square form
     (300, 500, 512, 32, "gemm_tile_128x128"),
     # narrow tiles, the whole K in one workgroup: 16, 32, 48 and 64 columns per tile, one to eight rows of tiles, one stage of
     # K to thirty-two, odd and even numbers of stages, ragged edges
@@ -158,6 +159,14 @@ CASES = [
     (24, 500, 2048, 32, "gemm_tile_64x128_splitk"),
     (16, 300, 1024, 32, "gemm_skinny"),
     (128, 1024, 16384, 128, "gemm_tile_64x128_splitk"),
+    # the square form (more than 128 rows): 4 x 2 waves of 32 x 64, tiles of 128 x 128, at block 64 (waves of 32 x 32) 128 x 64
+    (1024, 4096, 1024, 128, "gemm_panel"),          # 256 tiles, eight stages
+    (1500, 1500, 640, 128, "gemm_panel"),           # 144 tiles, ragged on both edges, five stages
+    (300, 10000, 128, 128, "gemm_panel"),           # 3 x 79 tiles, one stage
+    (512, 4000, 1152, 64, "gemm_panel"),            # 4 x 63 tiles of 128 x 64, two K-blocks per stage, nine stages
+    (2000, 1000, 256, 64, "gemm_panel"),            # 16 x 16 tiles
+    (512, 4096, 8192, 128, "gemm_panel_splitk"),    # 128 tiles, two pieces of 32 stages
+    (1000, 1000, 8320, 64, "gemm_panel_splitk"),    # 8 x 16 tiles, two pieces of 33 and 32 stages
     # narrow tiles on pieces of K (65 to 128 rows, K from 4224 to 12288): 128 x 64 tiles, at block 64 128 x 32
     (128, 1024, 8192, 128, "gemm_panel_splitk"),    # 16 tiles, eight pieces of eight stages
     (65, 4100, 4224, 128, "gemm_panel_splitk"),     # 65 tiles (the last 4 columns wide), three pieces of 11 stages
@@ -168,7 +177,7 @@ CASES = [
     (30, 8192, 10240, 128, "gemm_panel_splitk"),    # 128 tiles, two pieces of 40 stages
     (64, 2048, 11008, 128, "gemm_panel_splitk"),    # 32 tiles of 64 x 64, eight pieces of 11 stages
     (33, 2000, 5120, 64, "gemm_panel_splitk"),      # 32 tiles (the last 16 columns wide), five pieces of eight stages
-    (512, 4096, 4096, 64, "gemm_tile_128x128_splitk"),
+    (256, 2048, 8192, 64, "gemm_tile_128x128_splitk"),
 ]
 
 
