@@ -237,11 +237,12 @@ def bench_extras(pkg, torch):
                 out[f"decode_linear_M1_K{K}_N{N}"] = {"one_kernel_us": round(t1 * 1e3, 2), "two_launches_us": round(t2 * 1e3, 2)}
         del ws
 
-    # The Llama-7B GEMM shapes at 2048 and at 128 rows of activations (prefill; a decode batch), and 512 tokens against
-    # GPT-2-small's layers: through the entry point that takes scratch memory, as the Python operator calls it (problems
+    # The Llama-7B GEMM shapes at 2048 (and, against 4096 columns, 1024) and at 128 rows of activations (prefill; a decode
+    # batch), and 512 tokens against GPT-2-small's layers: through the entry point that takes scratch memory, as the Python operator calls it (problems
     # of few tiles run on narrow tiles, one per CU, or split K over the workgroups)
     shapes = [(M, K, N) for M in (2048, 128) for (K, N) in ((4096, 4096), (4096, 11008), (11008, 4096), (4096, 12288))]
     shapes += [(512, 768, 2304), (512, 768, 3072), (512, 3072, 768)]
+    shapes += [(1024, 4096, 4096), (1024, 11008, 4096)]          # 1024 tokens against N = 4096: 256 tiles of 128 x 128
     for (M, K, N) in shapes:
         if True:
             x = torch.randint(-127, 128, (M, K), device="cuda", dtype=torch.int8)
@@ -262,7 +263,7 @@ def bench_extras(pkg, torch):
             for _ in range(100 if M < 1024 else 20):          # (short kernels: the clock needs a few hundred microseconds of work to settle)
                 gp()
             t = median_ms(gp, 30)
-            out[f"{'prefill' if M == 2048 else 'batch128' if M == 128 else 'tokens512'}_gemm_M{M}_K{K}_N{N}"] = {
+            out[f"{'prefill' if M >= 1024 else 'batch128' if M == 128 else 'tokens512'}_gemm_M{M}_K{K}_N{N}"] = {
                 "us": round(t * 1e3, 1), "TOPS": round(2.0 * M * N * K / t / 1e9, 1),
                 "frac_int8_peak": round(2.0 * M * N * K / t / 1e9 / INT8_PEAK_TOPS, 4),
                 "kernel": lib.bi8_gemm_kernel_name(M, N, K, K, K, B, need).decode()}
