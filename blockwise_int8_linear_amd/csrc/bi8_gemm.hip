@@ -170,6 +170,9 @@ struct GemmArgs {
     // a launch that computes part of the output only: tiles_m x tiles_n tiles from tile (tile_m0, tile_n0) on (M, N and
     // the pointers stay those of the whole problem)
     int tile_m0, tile_n0;
+    // gemm_panel: columns from one tile to the next where that is less than the tile's width (0: its width): the tile's
+    // remaining columns are loaded as zeros, from beyond the buffer's range, and not stored
+    int panel_pitch;
 };
 // The rectangle of the output that one launch computes (the whole of it unless the plan cuts the problem in two).
 struct Part {
@@ -770,7 +773,7 @@ constexpr int kPanelThreads = (8 + kPanelLoaders) * 64;
 // The computing waves of the forms with one 16-row subtile per wave: `wave` = row group rg (16 rows), column group cg
 // (16 * NJ columns).
 template <int BLK, int CDT, int NJ, int CG, bool SPLIT>
-__device__ __forceinline__ void panel_compute_rows(const GemmArgs &g, uint8_t *lds, int wave, int lane, int64_t m0, int64_t n0, int nst) {
+__device__ __forceinline__ void panel_compute_rows(const GemmArgs &g, uint8_t *lds, int wave, int lane, int64_t m0, int64_t n0, int64_t n_end, int nst) {
     constexpr int NBS = kStageK / BLK;
     using L = PanelLds<NBS, NJ, CG>;
     constexpr int BM = L::BM, BN = L::BN, RG = 8 / CG, kBufs = L::kBufs;     // RG = row groups of 16 rows
@@ -881,7 +884,7 @@ __device__ __forceinline__ void panel_compute_rows(const GemmArgs &g, uint8_t *l
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const int64_t n = n0 + cg * 16 * NJ + j * 16 + r16;
-        const bool n_ok = n < g.N;
+        const bool n_ok = n < n_end;
         const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -903,7 +906,7 @@ __device__ __forceinline__ void panel_compute_rows(const GemmArgs &g, uint8_t *l
 // right behind the MFMAs that were the last to read the registers it goes into, so that the LDS reads run under MFMAs and
 // folds (the order of a stage: at `step` below).
 template <int BLK, int CDT, int NJ, bool SPLIT>
-__device__ __forceinline__ void panel_compute_square(const GemmArgs &g, uint8_t *lds, int wave, int lane, int64_t m0, int64_t n0, int nst) {
+__device__ __forceinline__ void panel_compute_square(const GemmArgs &g, uint8_t *lds, int wave, int lane, int64_t m0, int64_t n0, int64_t n_end, int nst) {
     constexpr int NBS = kStageK / BLK, NI = 2, CG = 2, RG = 4, NH = NJ / 2;
     using L = PanelLds<NBS, NJ, CG, NI>;
     constexpr int BM = L::BM, BN = L::BN, kBufs = L::kBufs;
@@ -1038,7 +1041,7 @@ __device__ __forceinline__ void panel_compute_square(const GemmArgs &g, uint8_t 
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
         const int64_t n = n0 + cg * 16 * NJ + j * 16 + r16;
-        const bool n_ok = n < g.N;
+        const bool n_ok = n < n_end;
         const float bias = (has_bias && n_ok) ? load_bias(g, n) : 0.0f;
 #pragma unroll
         for (int i = 0; i < NI; ++i)
@@ -1075,7 +1078,9 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t lds_base = bi8_lds_address(lds);
     const int tile_m = (int)blockIdx.x / g.tiles_n, tile_n = (int)blockIdx.x - tile_m * g.tiles_n;
-    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * BN;
+    const int pitch = !SPLIT && g.panel_pitch > 0 ? g.panel_pitch : BN;
+    const int64_t m0 = (int64_t)tile_m * BM, n0 = (int64_t)tile_n * pitch;
+    const int64_t n_end = g.N - n0 < pitch ? g.N : n0 + pitch;                  // the tile's columns: n0 ... n_end - 1
     const int stage_lo = SPLIT ? (int)blockIdx.y * g.split_stages : 0;          // this workgroup's first stage of K, and how many
     const int nst = SPLIT ? ((int)(g.K / kStageK) - stage_lo < g.split_stages ? (int)(g.K / kStageK) - stage_lo : g.split_stages)
                           : (int)(g.K / kStageK);
@@ -1099,7 +1104,7 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
         static_assert(kAItems % 2 == 0 && kPanelLoaders % 2 == 0, "the swizzle term of a loader's row items does not depend on the slot");
         static_assert((kBufs - 1) * kSlots < 64, "a loader's loads in flight fit the counter");
         const int64_t nblk = g.K / BLK;
-        const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM, w_rows = g.N - n0 < BN ? g.N - n0 : BN;
+        const int64_t a_rows = g.M - m0 < BM ? g.M - m0 : BM, w_rows = n_end - n0;
         const bi8_rsrc a_rsrc = bi8_make_rsrc(g.A + m0 * g.lda, (a_rows - 1) * g.lda + g.K);
         const bi8_rsrc w_rsrc = bi8_make_rsrc(g.W + n0 * g.ldw, (w_rows - 1) * g.ldw + g.K);
         const bi8_rsrc sa_rsrc = bi8_make_rsrc(g.sA + m0, ((nblk - 1) * g.M + (g.M - m0)) * 4);
@@ -1158,8 +1163,8 @@ __global__ __launch_bounds__(kPanelThreads) void gemm_panel(const GemmArgs g) {
         return;
     }
 
-    if constexpr (NI == 2) panel_compute_square<BLK, CDT, NJ, SPLIT>(g, lds, wave, lane, m0, n0, nst);
-    else panel_compute_rows<BLK, CDT, NJ, CG, SPLIT>(g, lds, wave, lane, m0, n0, nst);
+    if constexpr (NI == 2) panel_compute_square<BLK, CDT, NJ, SPLIT>(g, lds, wave, lane, m0, n0, n_end, nst);
+    else panel_compute_rows<BLK, CDT, NJ, CG, SPLIT>(g, lds, wave, lane, m0, n0, n_end, nst);
 }
 
 // ---- 256x256 tile, block 128 ------------------------------------------------------------------------------------
@@ -2792,7 +2797,7 @@ constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_sta
 constexpr int64_t kPanelSquareSplitMinTiles = 100, kPanelSquareSplitMinStages = 64;     // the square form on two pieces of K: 100 ... 128 tiles, K from 8192 on
 constexpr int64_t kPanelSquareMinTiles = 176;  // the square form outright from this many tiles on; with fewer only where nothing splits K
 constexpr int64_t kPanelFewRows = 32;          // up to 32 rows: tiles of 32 rows x (64 ... 256) columns ...
-constexpr int64_t kPanelFewRowsMinCols = 6144; // ... from this many columns on (fewer leave most CUs without a tile)
+constexpr int64_t kPanelFewRowsMinCols = 5120; // ... from this many columns on (fewer leave most CUs without a tile)
 // the widest tile, in 16-column subtiles (block 64 at 64 columns needs more registers than a wave has)
 constexpr int panel_max_subtiles(int block) { return block == 64 ? 3 : 4; }
 constexpr int64_t kStagedMaxRows = 32;         // gemv_staged: one or two groups of 16 rows whatever the shape ...
@@ -2947,7 +2952,10 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
         // workgroups of 16 columns run in several rounds (measured, block 128, W from HBM, us, gemv_staged -> gemm_panel at
         // K = 1024 / 4096: 16 rows N = 6144 7.2 -> 4.2, 10.4 -> 9.4; N = 11008 6.1 -> 4.7, 13.6 -> 11.9; N = 32000 13.8 -> 9.1, 31.8 -> 29.8;
         // 32 rows N = 8192 5.7 -> 4.1, 12.3 -> 11.4; N = 11008 7.8 -> 4.3, 16.4 -> 12.5; N = 16384 10.1 -> 5.0, 21.6 -> 16.3; N = 32000
-        // 17.9 -> 8.1, 37.3 -> 30.0; at N = 4096 the 64 tiles leave most CUs idle: 16 rows 6.5 -> 9.1, 32 rows 7.9 -> 9.9 at K = 4096)
+        // 17.9 -> 8.1, 37.3 -> 30.0.  A tile's columns are a multiple of 16 (the tile's remaining subtiles stay empty: panel_pitch), as
+        // few as give one tile per CU: N = 6144 / 8192 at K = 4096 on 192 / 256 tiles of 32 columns instead of 96 / 128 of 64: 16 rows
+        // 9.9 -> 8.6, 10.5 -> 9.8; 32 rows 10.8 -> 9.0, 11.3 -> 10.2; N = 5120 (gemv_staged before) 9.2 -> 8.2, 10.9 -> 8.6; at N = 4096
+        // gemv_staged stays ahead: 16 rows 6.4 -> 8.5, 32 rows 7.8 -> 8.6 at K = 4096)
         if (M > kRowsMax && M <= kPanelFewRows && N >= kPanelFewRowsMinCols && (block == 64 || block == 128) &&
             (K / block + 1) * max_mn * 4 < kBufOut && K / kStageK <= kPanelMaxStages) {
             const int64_t widest = 64 * panel_max_subtiles(block);
@@ -3087,8 +3095,10 @@ template <int BLK, int CDT> int launch_staged(const GemmArgs &g, hipStream_t st)
 // gemm_panel on the narrowest tiles that give at most one per CU
 template <int BLK, int CDT, int NJ, int CG, int NI = 1> int launch_panel_as(GemmArgs g, hipStream_t st) {
     using L = PanelLds<kStageK / BLK, NJ, CG, NI>;
+    const int pitch = g.panel_pitch > 0 ? g.panel_pitch : L::BN;
+    if (pitch > L::BN) return BI8_ERR_UNSUPPORTED;
     g.tiles_m = (int)((g.M + L::BM - 1) / L::BM);
-    g.tiles_n = (int)((g.N + L::BN - 1) / L::BN);
+    g.tiles_n = (int)((g.N + pitch - 1) / pitch);
     auto kern = gemm_panel<BLK, CDT, NJ, CG, false, NI>;
     static LdsOptIn opted;                         // one per kernel instantiation
     const int rc = opted.ensure((const void *)kern, L::kBytes);
@@ -3096,14 +3106,22 @@ template <int BLK, int CDT, int NJ, int CG, int NI = 1> int launch_panel_as(Gemm
     hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(kPanelThreads), L::kBytes, st, g);
     return bi8_launch_rc();
 }
-template <int BLK, int CDT, int CG> int launch_panel_cg(const GemmArgs &g, hipStream_t st) {
-    const int64_t rows = (g.M + 128 / CG - 1) / (128 / CG), w = 16 * CG;       // rows of tiles; columns of a tile per subtile of a wave
-    if (rows * ((g.N + w - 1) / w) <= kCus) return launch_panel_as<BLK, CDT, 1, CG>(g, st);
-    if (rows * ((g.N + 2 * w - 1) / (2 * w)) <= kCus) return launch_panel_as<BLK, CDT, 2, CG>(g, st);
-    if (rows * ((g.N + 3 * w - 1) / (3 * w)) <= kCus) return launch_panel_as<BLK, CDT, 3, CG>(g, st);
-    if constexpr (panel_max_subtiles(BLK) >= 4)
-        if (rows * ((g.N + 4 * w - 1) / (4 * w)) <= kCus) return launch_panel_as<BLK, CDT, 4, CG>(g, st);
-    return BI8_ERR_UNSUPPORTED;                    // (the plan sends no other problem here)
+template <int BLK, int CDT, int CG> int launch_panel_cg(GemmArgs g, hipStream_t st) {
+    const int64_t rows = (g.M + 128 / CG - 1) / (128 / CG);                    // rows of tiles
+    // the fewest 16-column subtiles per tile that give at most one tile per CU; the narrowest kernel form that holds them
+    // (two or four waves side by side: the tile's last subtiles may then be empty)
+    const int64_t sub = (g.N + 15) / 16, across = kCus / rows;
+    const int64_t per_tile = across > 0 ? (sub + across - 1) / across : 0;
+    if (per_tile < 1 || per_tile > CG * panel_max_subtiles(BLK)) return BI8_ERR_UNSUPPORTED;        // (the plan sends no other problem here)
+    g.panel_pitch = (int)(16 * per_tile);
+    switch ((per_tile + CG - 1) / CG) {
+    case 1: return launch_panel_as<BLK, CDT, 1, CG>(g, st);
+    case 2: return launch_panel_as<BLK, CDT, 2, CG>(g, st);
+    case 3: return launch_panel_as<BLK, CDT, 3, CG>(g, st);
+    default:
+        if constexpr (panel_max_subtiles(BLK) >= 4) return launch_panel_as<BLK, CDT, 4, CG>(g, st);
+        return BI8_ERR_UNSUPPORTED;
+    }
 }
 // the split form: tiles of 128 rows x 64 columns (block 64: 32), split_per_tile pieces of split_stages stages each, then the sum
 template <int BLK, int CDT, int NJ, int CG, int NI = 1> int launch_panel_split_as(GemmArgs g, hipStream_t st) {

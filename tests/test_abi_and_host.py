@@ -263,10 +263,10 @@ def test_kernel_choice_by_shape():
     assert name(64, 5000, 640, 128) == "gemm_panel" and name(48, 11008, 4096, 128, 1 << 30) == "gemm_panel" and name(33, 16384, 4096, 64) == "gemm_panel"
     assert name(48, 700, 640, 128) == "gemm_panel" and name(64, 4096, 1024, 64) == "gemm_panel" and name(64, 4096, 1152, 64) == "gemv_staged"
     assert name(64, 33000, 768, 128) == "gemm_wide"                  # too many columns for one round
-    # 3 to 32 rows against 6144 columns or more: the same on tiles of 32 rows x 64 ... 256 columns
-    assert name(32, 11008, 768, 128) == "gemm_panel" and name(16, 11008, 4096, 64) == "gemm_panel" and name(3, 6144, 4096, 128, 1 << 30) == "gemm_panel"
+    # 3 to 32 rows against 5120 columns or more: the same on tiles of 32 rows x 64 ... 256 columns
+    assert name(32, 11008, 768, 128) == "gemm_panel" and name(16, 11008, 4096, 64) == "gemm_panel" and name(3, 5120, 4096, 128, 1 << 30) == "gemm_panel"
     assert name(32, 11008, 4096, 64, 1 << 30) == "gemm_panel" and name(16, 32000, 4096, 128) == "gemm_panel" and name(8, 50257, 768, 128) == "gemm_panel"
-    assert name(16, 6143, 4096, 128) == "gemv_staged" and name(16, 11008, 4224, 128) == "gemv_staged" and name(2, 11008, 4096, 128) == "gemv_rows"
+    assert name(16, 5119, 4096, 128) == "gemv_staged" and name(16, 11008, 4224, 128) == "gemv_staged" and name(2, 11008, 4096, 128) == "gemv_rows"
     assert name(16, 50257, 768, 64) == "gemv_staged" and name(16, 65537, 768, 128) == "gemv_staged"      # 262 tiles of 192 / 257 of 256 columns
     assert name(1, 4096, 4096, 128) == "gemv_rows" and name(2, 11008, 4096, 64) == "gemv_rows"   # weight rows read as runs
     assert name(3, 4096, 4096, 128) == "gemv_staged" and name(16, 4096, 11008, 64) == "gemv_staged"

@@ -122,20 +122,24 @@ CASES = [
     (48, 700, 640, 64, "gemm_panel"),
     (64, 4096, 1024, 128, "gemm_panel"),            # 128 tiles of 32 columns
     (33, 64, 128, 128, "gemm_panel"),               # one stage, one tile of which the second wave column is empty
-    (64, 11008, 4096, 128, "gemm_panel"),           # 172 tiles of 64 columns, 32 stages
+    (64, 11008, 4096, 128, "gemm_panel"),           # 230 tiles of 48 columns in the 64-column form, 32 stages
     (50, 24000, 256, 128, "gemm_panel"),            # 250 tiles of 96 columns
     (40, 24000, 384, 64, "gemm_panel"),             # ... two K-blocks per stage
     (64, 32000, 384, 128, "gemm_panel"),            # 250 tiles of 128 columns
-    # ... and for 3 to 32 rows against 6144 columns or more tiles of 32 rows, the waves as 2 x 4: 64, 128, 192 and 256 columns per tile
-    (7, 8192, 2048, 128, "gemm_panel"),             # 128 tiles of 64 columns, the second row group empty
-    (12, 11008, 2048, 64, "gemm_panel"),            # 172 tiles
+    (60, 30000, 256, 128, "gemm_panel"),            # 235 tiles of 128 columns; (48, 20000): 250 of 80 in the 96-column form
+    (48, 20000, 256, 128, "gemm_panel"),
+    # ... and for 3 to 32 rows against 5120 columns or more tiles of 32 rows, the waves as 2 x 4 (64, 128, 192 or 256 columns),
+    # of which a tile takes as few 16-column subtiles as give one tile per CU
+    (7, 8192, 2048, 128, "gemm_panel"),             # 256 tiles of 32 columns (the waves' last two columns and second row group empty)
+    (12, 11008, 2048, 64, "gemm_panel"),            # 230 tiles of 48 columns
     (17, 8192, 2048, 128, "gemm_panel"),
     (29, 11008, 1024, 64, "gemm_panel"),
-    (32, 6144, 4096, 128, "gemm_panel"),            # 96 tiles, 32 stages
-    (5, 6150, 256, 128, "gemm_panel"),              # the last tile 6 columns wide
+    (32, 6144, 4096, 128, "gemm_panel"),            # 192 tiles of 32 columns, 32 stages
+    (5, 6150, 256, 128, "gemm_panel"),              # 193 tiles, the last 6 columns wide
+    (16, 5120, 640, 128, "gemm_panel"),             # 160 tiles of 32 columns
     (24, 30000, 384, 128, "gemm_panel"),            # 235 tiles of 128 columns
-    (20, 40000, 384, 64, "gemm_panel"),             # 209 tiles of 192 columns, two K-blocks per stage
-    (3, 50000, 128, 128, "gemm_panel"),             # 196 tiles of 256 columns, one stage
+    (20, 40000, 384, 64, "gemm_panel"),             # 250 tiles of 160 columns in the 192-column form, two K-blocks per stage
+    (3, 50000, 128, 128, "gemm_panel"),             # 241 tiles of 208 columns in the 256-column form, one stage
     (2304, 2304, 256, 32, "gemm_tile_128x128"),
     (48, 5000, 640, 32, "gemm_tile_64x128"),
     (48, 700, 1280, 64, "gemv_staged"),             # four groups of 16 rows
