@@ -2796,6 +2796,7 @@ constexpr int64_t kPanelSplit64RowsMinStages = 40, kPanelSplit64RowsMaxTiles = 3
 constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024
 constexpr int64_t kPanelSquareSplitMinTiles = 100, kPanelSquareSplitMinStages = 64;     // the square form on two pieces of K: 100 ... 128 tiles, K from 8192 on
 constexpr int64_t kPanelSquareMinTiles = 176;  // the square form outright from this many tiles on; with fewer only where nothing splits K
+constexpr int64_t kPanelHalfHeightMaxSubtiles = 4;     // more than 64 rows on tiles of 64 rows: where those are at most 64 columns wide
 constexpr int64_t kPanelFewRows = 32;          // up to 32 rows: tiles of 32 rows x (64 ... 256) columns ...
 constexpr int64_t kPanelFewRowsMinCols = 5120; // ... from this many columns on (fewer leave most CUs without a tile)
 // the widest tile, in 16-column subtiles (block 64 at 64 columns needs more registers than a wave has)
@@ -3153,7 +3154,16 @@ template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) 
     // (more rows of narrow tiles than one round: the plan has counted the square form's)
     if (g.M > 128 && ((g.M + 127) / 128) * ((g.N + 16 * panel_max_subtiles(BLK) - 1) / (16 * panel_max_subtiles(BLK))) > kCus)
         return launch_panel_as<BLK, CDT, BLK == 64 ? 2 : 4, 2, 2>(g, st);
-    return g.M <= 64 ? launch_panel_cg<BLK, CDT, 2>(g, st) : launch_panel_cg<BLK, CDT, 1>(g, st);
+    if (g.M <= 64) return launch_panel_cg<BLK, CDT, 2>(g, st);
+    // more than 64 rows: tiles of 64 rows where one round of them is at most 64 columns wide, else of 128 rows.  A workgroup
+    // streams its tile's rows of A and of W, and what bounds these problems is that traffic: 256 tiles of 64 x 32 move a third
+    // less than 256 of 128 x 16.  Measured, block 128, W from HBM, us at K = 1024 / 4096, tiles of 128 -> 64 rows: 128 x 768
+    // 4.7 -> 4.2, 8.6 -> 7.8; 128 x 4096 5.1 -> 4.5, 12.4 -> 9.8; 128 x 8192 6.1 -> 5.6, 15.7 -> 15.1; 256 x 2048 5.1 -> 4.5, 9.5 -> 8.3;
+    // 256 x 4096 5.8 -> 5.6, 14.2 -> 12.9; 512 x 768 5.0 -> 4.4, 9.0 -> 8.3; but 128 x 11008 (tiles of 64 x 96) 7.3 -> 8.0, 18.1 -> 19.4;
+    // tiles of 32 rows: the same as 64 at up to 4096 columns, behind from there (128 x 8192 x 4096 16.5, 128 x 11008 x 4096 29.3).
+    const int64_t across = kCus / ((g.M + 63) / 64);
+    if (across >= 1 && ((g.N + 15) / 16 + across - 1) / across <= kPanelHalfHeightMaxSubtiles) return launch_panel_cg<BLK, CDT, 2>(g, st);
+    return launch_panel_cg<BLK, CDT, 1>(g, st);
 }
 
 template <int BLK, int CDT> int launch_rows(const GemmArgs &g, hipStream_t st) {

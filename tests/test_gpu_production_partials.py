@@ -104,19 +104,20 @@ CASES = [
     (1500, 1500, 512, 32, "gemm_tile_128x128"),
     (1024, 3072, 640, 64, "gemm_tile_128x128"),     # block 64: more tiles of 128 x 64 than one round of gemm_panel's square form
     (300, 500, 512, 32, "gemm_tile_128x128"),
-    # narrow tiles, the whole K in one workgroup: 16, 32, 48 and 64 columns per tile, one to eight rows of tiles, one stage of
-    # K to thirty-two, odd and even numbers of stages, ragged edges
-    (300, 500, 512, 128, "gemm_panel"),             # 3 x 32 tiles of 16 columns, the last row of tiles 44 rows, the last column 4
-    (128, 4096, 1024, 128, "gemm_panel"),           # 256 tiles of 16 columns
+    # narrow tiles, the whole K in one workgroup: tiles of 128 rows x 16, 32, 48 or 64 columns, or -- where one round of them is at
+    # most 64 columns wide -- of 64 rows x 16 ... 64 columns; one to many rows of tiles, one stage of K to thirty-two, odd and even
+    # numbers of stages, ragged edges
+    (300, 500, 512, 128, "gemm_panel"),             # 5 x 32 tiles of 64 x 16, the last row of tiles 44 rows, the last column 4
+    (128, 4096, 1024, 128, "gemm_panel"),           # 2 x 128 tiles of 64 x 32
     (128, 64, 128, 128, "gemm_panel"),              # a single stage
     (100, 48, 256, 64, "gemm_panel"),
-    (100, 8000, 640, 128, "gemm_panel"),            # 250 tiles of 32 columns, five stages
-    (200, 3000, 1152, 64, "gemm_panel"),            # 2 x 94 tiles of 32 columns, two K-blocks per stage, nine stages
-    (128, 11008, 384, 64, "gemm_panel"),            # 230 tiles of 48 columns
-    (65, 16000, 256, 128, "gemm_panel"),            # 250 tiles of 64 columns
-    (512, 4090, 4096, 128, "gemm_panel"),           # 4 x 64 tiles of 64 columns, 32 stages
-    (1000, 500, 384, 128, "gemm_panel"),            # 8 x 32 tiles
-    (30000, 16, 256, 128, "gemm_panel"),            # 235 x 1 tiles: tall and one tile wide
+    (100, 8000, 640, 128, "gemm_panel"),            # 2 x 125 tiles of 64 x 64, five stages
+    (200, 3000, 1152, 64, "gemm_panel"),            # 4 x 63 tiles of 64 x 48, two K-blocks per stage, nine stages
+    (128, 11008, 384, 64, "gemm_panel"),            # 230 tiles of 128 x 48
+    (65, 16000, 256, 128, "gemm_panel"),            # 250 tiles of 128 x 64
+    (512, 4090, 4096, 128, "gemm_panel"),           # 4 x 64 tiles of 128 x 64, 32 stages
+    (1000, 500, 384, 128, "gemm_panel"),            # 16 x 16 tiles of 64 x 32
+    (30000, 16, 256, 128, "gemm_panel"),            # 235 x 1 tiles of 128 x 16: tall and one tile wide
     # ... and for 33 to 64 rows tiles of 64 rows, the waves as 4 x 2: 32, 64, 96 and 128 columns per tile
     (48, 5000, 640, 64, "gemm_panel"),              # 157 tiles of 32 columns, the last 8 columns wide
     (48, 700, 640, 64, "gemm_panel"),
