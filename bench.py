@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0          # HBM3E, 8 TB/s
 # WRITE_SIZE of rocprofv3 --pmc runs of this file, scaled by what the same counters read for a 256 MiB copy
 # (x2.0 and x1.0); the runs and figures are in profiles/gemm_wide_8192x8192x8192_block128.md.  Counters cannot be read
 # from inside the process, so this is a constant from those runs, labelled as such in the output ("traffic_source").
-GEMM_8192_TRAFFIC_BYTES = 966812913
+GEMM_8192_TRAFFIC_BYTES = 966965985
 GEMM_8192_TRAFFIC_SOURCE = ("profiles/gemm_wide_8192x8192x8192_block128.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
                             "command, scaled by a 256 MiB copy; a constant, not measured in this run")
 PREROLL_MAX = 400              # launches

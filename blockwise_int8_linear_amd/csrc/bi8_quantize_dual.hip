@@ -76,6 +76,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
 
     const int tid = threadIdx.x;
     const char *xb = (const char *)x;
+    const bool wide_q = (((uintptr_t)q | (uintptr_t)ldq) & 15) == 0;     // rows of q on 16-byte boundaries: 16-byte code stores
     const int lr = tid / LPR;                      // row inside a pass
     const int cc = (tid % LPR) * VEC;              // first column of this lane inside a half
 
@@ -141,6 +142,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
 #pragma unroll
                 for (int h = 0; h < NH; ++h) m[h] = bi8_group_max<LB>(m[h]);
             }
+            // (16-bit inputs, two halves, aligned: a lane's 8 codes of each half are exchanged with its neighbour's so that the
+            // even lane stores 16 consecutive codes of the left half and the odd lane 16 of the right half -- the eight lanes of
+            // a row then write the row's whole 128-byte line in one instruction instead of two halves in two)
+            constexpr bool kPairStores = ALIGNED && VEC == 8 && NH == 2;
+            bi8_v2u wq[NH];
 #pragma unroll
             for (int h = 0; h < NH; ++h) {
                 const int64_t col = cbase + h * kTC + cc;
@@ -156,7 +162,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) code[e] = bi8_code_fast<NCORR>(f[h][e], m[h], y);
                 }
-                if (live) {
+                if constexpr (kPairStores) {
+                    wq[h] = bi8_v2u{bi8_pack4(code[0], code[1], code[2], code[3]), bi8_pack4(code[4], code[5], code[6], code[7])};
+                    if (!wide_q && live) __builtin_nontemporal_store(wq[h], (bi8_v2u *)(q + row * ldq + col));
+                } else if (live) {
                     int8_t *dst = q + row * ldq + col;
                     if (ALIGNED || col + VEC <= C) {
                         if constexpr (VEC == 4) {
@@ -172,6 +181,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(DT == 
 #pragma unroll
                         for (int e = 0; e < VEC; ++e)
                             if (col + e < C) dst[e] = (int8_t)(code[e] & 0xffu);
+                    }
+                }
+            }
+            if constexpr (kPairStores) {
+                if (wide_q) {
+                    const bool odd = (tid & 1) != 0;
+                    const bi8_v2u send = odd ? wq[0] : wq[1];              // what the neighbour stores of this lane's codes
+                    bi8_v2u recv;
+                    recv[0] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send[0], 0xB1, 0xf, 0xf, false);   // quad_perm [1,0,3,2]
+                    recv[1] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)send[1], 0xB1, 0xf, 0xf, false);
+                    const bi8_v4u w = odd ? bi8_v4u{recv[0], recv[1], wq[1][0], wq[1][1]} : bi8_v4u{wq[0][0], wq[0][1], recv[0], recv[1]};
+                    const int64_t col = cbase + (odd ? kTC + cc - VEC : cc);       // 16 consecutive codes from here
+                    if (row < R && col < C) {
+                        int8_t *dst = q + row * ldq + col;
+                        if (col + 2 * VEC <= C) __builtin_nontemporal_store(w, (bi8_v4u *)dst);
+                        else __builtin_nontemporal_store(bi8_v2u{w[0], w[1]}, (bi8_v2u *)dst);      // (C is a multiple of 8: the row ends after the first 8)
                     }
                 }
             }
