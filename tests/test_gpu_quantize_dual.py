@@ -141,3 +141,18 @@ def test_dual_with_column_sums_special_and_empty(ops):
     e = torch.empty(0, 128, device=DEV, dtype=torch.bfloat16)
     out = ops.quantize_block_dual_colsum(e, 128)
     assert out[0].shape == (0, 128) and out[4].shape == (128,) and (out[4] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16", "f32"])
+def test_padded_code_buffers_hold_the_same_codes(ops, dtype):
+    """The training path keeps the codes in buffers whose rows are padded to whole K-blocks, i.e. rows that start on 16-byte
+    boundaries whatever the column count: there the row codes of 16-bit inputs leave as 16-byte stores (a row's whole line in
+    one instruction), also where a row ends after the first 8 codes of such a store.  Same codes and scales as unpadded."""
+    from blockwise_int8_linear_amd import ops as _ops
+    for (R, C, block) in [(300, 1000, 128), (1000, 72, 64), (64, 520, 128), (257, 136, 128), (128, 8, 64)]:
+        x = outlier_tensor(R, C, DTYPES[dtype], seed=R + C).to(DEV)
+        q, s, qt, st = ops.quantize_block_dual(x, block)
+        qp, sp, qtp, stp, q_store, qt_store = _ops._quantize_block_dual(x, block, True)
+        assert q_store.shape[1] % 16 == 0 and q_store.shape[1] >= C and q_store.data_ptr() % 16 == 0
+        assert torch.equal(qp, q) and torch.equal(qtp, qt) and _same(sp, s) and _same(stp, st)
+        assert (q_store[:, C:] == 0).all() and (qt_store[:, R:] == 0).all()          # the padding stays zero
