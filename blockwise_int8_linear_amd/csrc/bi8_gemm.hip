@@ -2793,7 +2793,8 @@ constexpr int64_t kPanelSplitFewRowsMin = 16;  // the split form on tiles of 32 
 constexpr int64_t kPanelSplitFewRowsMinStages = 64, kPanelSplitFewRowsTwoStages = 80;      // ... K from 8192 on; two pieces per tile from 10240 on, ...
 constexpr int64_t kPanelSplitFewRowsMinGroups = 192;                                       // ... and this many workgroups
 constexpr int64_t kPanelSplit64RowsMinStages = 40, kPanelSplit64RowsMaxTiles = 32;         // on tiles of 64 rows: K from 5120 on, up to 2048 columns
-constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024
+constexpr int64_t kPanelOverStagedStages = 8;  // 33 ... 64 rows inside gemv_staged's band: only up to K = 1024 ...
+constexpr int64_t kPanelOverStagedMinCols = 3072;      // ... or from this many columns on
 constexpr int64_t kPanelSquareSplitMinTiles = 100, kPanelSquareSplitMinStages = 64;     // the square form on two pieces of K: 100 ... 128 tiles, K from 8192 on
 constexpr int64_t kPanelSquareMinTiles = 176;  // the square form outright from this many tiles on; with fewer only where nothing splits K
 constexpr int64_t kPanelHalfHeightMaxSubtiles = 4;     // more than 64 rows on tiles of 64 rows: where those are at most 64 columns wide
@@ -2939,11 +2940,14 @@ static GemmPlan plan_gemm(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t 
         // unless gemv_staged's four groups of rows apply, which are ahead from K = 1152 on (measured, 64 rows, block 128, W from
         // HBM, us, gemv_staged or the split 64x128 tiles -> gemm_panel, K = 768 / 2048 / 4096 / 8192: N = 4096 5.7 -> 4.7,
         // 6.0 -> 7.2, 10.1 -> 11.6, 16.9 -> 19.6; N = 8192 7.1 -> 5.0, 12.4 -> 7.9, 15.5 -> 13.1, 21.1 -> 23.1; N = 11008 7.5 -> 5.9,
-        // 13.6 -> 10.2, 17.4 -> 16.2, 29.4 -> 28.0; N = 16384 8.0 -> 6.6, 15.5 -> 12.5, 22.4 -> 19.4, 39.4 -> 33.5)
+        // 13.6 -> 10.2, 17.4 -> 16.2, 29.4 -> 28.0; N = 16384 8.0 -> 6.6, 15.5 -> 12.5, 22.4 -> 19.4, 39.4 -> 33.5).  With tiles of as few
+        // 16-column subtiles as give one tile per CU, and of 32 rows where those are at most 32 columns wide (launch_panel), the
+        // kernel is ahead of gemv_staged from 3072 columns on whatever K up to 4096: N = 4096 at K = 2048 / 4096, 48 rows 5.6 -> 5.4,
+        // 9.4 -> 8.3, 64 rows 5.9 -> 5.4, 10.0 -> 8.5; level at N = 2048 (5.5 -> 5.4, 7.6 -> 7.7), behind at N = 1024 (7.2 -> 7.6)
         const bool staged_band = M <= kStagedWideRows && (N + 15) / 16 <= kStagedWideMaxGroups && M * K <= kStagedWideMaxCodes;
         if (M > kStagedMaxRows && M <= kPanelMinRows && (block == 64 || block == 128) && (K / block + 1) * max_mn * 4 < kBufOut) {
             const int64_t widest = 32 * panel_max_subtiles(block), nst = K / kStageK;
-            if ((N + widest - 1) / widest <= kCus && nst <= kPanelMaxStages && (!staged_band || nst <= kPanelOverStagedStages)) {
+            if ((N + widest - 1) / widest <= kCus && nst <= kPanelMaxStages && (!staged_band || nst <= kPanelOverStagedStages || N >= kPanelOverStagedMinCols)) {
                 p.kernel = kKPanel;
                 return p;
             }
@@ -3154,7 +3158,12 @@ template <int BLK, int CDT> int launch_panel(const GemmArgs &g, hipStream_t st) 
     // (more rows of narrow tiles than one round: the plan has counted the square form's)
     if (g.M > 128 && ((g.M + 127) / 128) * ((g.N + 16 * panel_max_subtiles(BLK) - 1) / (16 * panel_max_subtiles(BLK))) > kCus)
         return launch_panel_as<BLK, CDT, BLK == 64 ? 2 : 4, 2, 2>(g, st);
-    if (g.M <= 64) return launch_panel_cg<BLK, CDT, 2>(g, st);
+    if (g.M <= 64) {
+        // 33 ... 64 rows: two rows of 32-row tiles where one round of them is at most 32 columns wide (a fifth less traffic into
+        // LDS than one row of 64 x 16 tiles: 64 x 4096 x 4096 9.1 -> 8.5 us, 48 rows 8.7 -> 8.3; level at 8192 columns, behind beyond)
+        if ((g.N + 15) / 16 <= 2 * (kCus / 2)) return launch_panel_cg<BLK, CDT, 4>(g, st);
+        return launch_panel_cg<BLK, CDT, 2>(g, st);
+    }
     // more than 64 rows: tiles of 64 rows where one round of them is at most 64 columns wide, else of 128 rows.  A workgroup
     // streams its tile's rows of A and of W, and what bounds these problems is that traffic: 256 tiles of 64 x 32 move a third
     // less than 256 of 128 x 16.  Measured, block 128, W from HBM, us at K = 1024 / 4096, tiles of 128 -> 64 rows: 128 x 768

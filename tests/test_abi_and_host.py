@@ -261,7 +261,7 @@ def test_kernel_choice_by_shape():
     assert name(300, 500, 512, 32) == "gemm_tile_128x128"            # block 32: not its
     # 33 to 64 rows: the same on tiles of 64 rows x 32 ... 128 columns, where gemv_staged (below) does not apply or K is at most 1024
     assert name(64, 5000, 640, 128) == "gemm_panel" and name(48, 11008, 4096, 128, 1 << 30) == "gemm_panel" and name(33, 16384, 4096, 64) == "gemm_panel"
-    assert name(48, 700, 640, 128) == "gemm_panel" and name(64, 4096, 1024, 64) == "gemm_panel" and name(64, 4096, 1152, 64) == "gemv_staged"
+    assert name(48, 700, 640, 128) == "gemm_panel" and name(64, 2048, 1024, 64) == "gemm_panel" and name(64, 2048, 1152, 64) == "gemv_staged"
     assert name(64, 33000, 768, 128) == "gemm_wide"                  # too many columns for one round
     # 3 to 32 rows against 5120 columns or more: the same on tiles of 32 rows x 64 ... 256 columns
     assert name(32, 11008, 768, 128) == "gemm_panel" and name(16, 11008, 4096, 64) == "gemm_panel" and name(3, 5120, 4096, 128, 1 << 30) == "gemm_panel"
@@ -275,7 +275,9 @@ def test_kernel_choice_by_shape():
     assert name(24, 4096, 4096, 128) == "gemv_staged" and name(32, 4096, 11008, 64) == "gemv_staged"   # two groups of 16 rows
     assert name(24, 4096, 4096, 32, 1 << 30) == "gemm_tile_64x128_splitk"      # block 32 with scratch memory: the split tiles are ahead
     # 33 to 64 rows: one pass over W where one round of workgroups covers the columns and K is short, else the split tiles
-    assert name(33, 4096, 4096, 128, 1 << 30) == "gemv_staged" and name(64, 4096, 4096, 64) == "gemv_staged" and name(48, 700, 1280, 128) == "gemv_staged"
+    assert name(33, 3071, 4096, 128, 1 << 30) == "gemv_staged" and name(64, 2048, 4096, 64) == "gemv_staged" and name(48, 700, 1280, 128) == "gemv_staged"
+    assert name(33, 3072, 4096, 128, 1 << 30) == "gemm_panel" and name(64, 4096, 4096, 64) == "gemm_panel"      # from 3072 columns on: narrow tiles
+    assert name(64, 4096, 4224, 64) == "gemv_staged"                 # ... up to K = 4096
     assert name(48, 11008, 8192, 128, 1 << 30) == "gemm_tile_64x128_splitk" and name(48, 4096, 11008, 128, 1 << 30) == "gemm_tile_64x128_splitk"
     # 33 to 64 rows, K from 5120 to 12288, up to 2048 columns: narrow tiles of 64 rows on pieces of K
     assert name(48, 2048, 11008, 128, 1 << 30) == "gemm_panel_splitk" and name(64, 1024, 5120, 64, 1 << 30) == "gemm_panel_splitk"

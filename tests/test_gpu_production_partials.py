@@ -129,6 +129,10 @@ CASES = [
     (64, 32000, 384, 128, "gemm_panel"),            # 250 tiles of 128 columns
     (60, 30000, 256, 128, "gemm_panel"),            # 235 tiles of 128 columns; (48, 20000): 250 of 80 in the 96-column form
     (48, 20000, 256, 128, "gemm_panel"),
+    # ... and, up to 4096 columns, two rows of 32-row tiles
+    (64, 4096, 2048, 128, "gemm_panel"),            # 2 x 128 tiles of 32 x 32
+    (48, 3072, 4096, 64, "gemm_panel"),             # 2 x 96 tiles, the second row of tiles 16 rows, 32 stages
+    (33, 3100, 640, 128, "gemm_panel"),             # 2 x 97 tiles, the second row of tiles a single row, the last column 28 wide
     # ... and for 3 to 32 rows against 5120 columns or more tiles of 32 rows, the waves as 2 x 4 (64, 128, 192 or 256 columns),
     # of which a tile takes as few 16-column subtiles as give one tile per CU
     (7, 8192, 2048, 128, "gemm_panel"),             # 256 tiles of 32 columns (the waves' last two columns and second row group empty)
@@ -144,7 +148,7 @@ CASES = [
     (2304, 2304, 256, 32, "gemm_tile_128x128"),
     (48, 5000, 640, 32, "gemm_tile_64x128"),
     (48, 700, 1280, 64, "gemv_staged"),             # four groups of 16 rows
-    (64, 4096, 2048, 128, "gemv_staged"),
+    (64, 2048, 2048, 128, "gemv_staged"),
     (33, 1000, 2048 + 128, 128, "gemv_staged"),
     (1, 384, 512, 128, "gemv_rows"),
     (2, 1000, 4096 + 384, 128, "gemv_rows"),        # more than four runs of 1 KiB per row, the last one partial
