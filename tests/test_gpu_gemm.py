@@ -449,7 +449,7 @@ def test_infinite_and_nan_scales(ops, shape):
     """A block that held an infinity has scale inf.  The reference's sw * (sx * (P * div)) (triton_functions.py:120)
     then gives +-inf where the block partial P is not 0 and NaN where it is.  A ROW scale of inf or NaN gives exactly
     that in every kernel.  A COLUMN scale of inf gives it in the few-row and general kernels; the tiled kernels
-    (M > 32, and gemm_panel's 32-row tiles for 3 rows or more against 6144 columns or more), whose fold computes fma(1.5*2^23 + P, b, -1.5*2^23 * b), give NaN for the whole column instead of +-inf:
+    (M > 32, and gemm_panel's 32-row tiles for 3 rows or more against 5120 columns or more), whose fold computes fma(1.5*2^23 + P, b, -1.5*2^23 * b), give NaN for the whole column instead of +-inf:
     the one place where non-finite results differ from the reference's, pinned here.  Everything else stays finite."""
     from blockwise_int8_linear_amd import _lib
     M, N, K, family = shape[:4]
