@@ -93,3 +93,44 @@ def test_random_shape(case):
     scale = full.double().abs().max().item()
     unit = {"f32": 2e-6, "bf16": 8e-3, "f16": 1e-3}[out]         # one rounding of the output type at the largest magnitude, and the summation order
     assert not torch.isnan(C).any() and err.max().item() <= unit * scale, f"{kernel}: {err.max().item():.3e} of {scale:.3e}"
+
+
+@pytest.mark.parametrize("M,N,K,block", [(16, 11008, 4096, 128), (32, 6144, 2048, 64), (64, 4096, 4096, 128), (128, 4096, 4096, 128),
+                                         (300, 500, 512, 128), (1024, 4096, 2048, 128), (512, 4096, 1152, 64),
+                                         (32, 4096, 11008, 128), (64, 2048, 8192, 128), (128, 4096, 11008, 128), (512, 4096, 8192, 128)])
+def test_narrow_tile_kernels_call_after_call(M, N, K, block):
+    """gemm_panel's forms (tiles of 32, 64 and 128 rows, the square form, the pieces of K) stream their operands through rings of
+    LDS buffers filled by waves of their own, with hand-counted waits: a buffer reused too early would show now and then, not
+    always.  Fresh operands three times, twelve calls each with other work on the GPU in between: every call gives the bits of
+    the first (the kernels are deterministic), and the first matches a float64 product on the device."""
+    from blockwise_int8_linear_amd import _lib
+    lib = _lib.load()
+    need = lib.bi8_gemm_workspace_bytes(M, N, K, block)
+    kernel = lib.bi8_gemm_kernel_name(M, N, K, K, K, block, need).decode()
+    assert kernel in ("gemm_panel", "gemm_panel_splitk")
+    ws = torch.empty(max(need, 16), device=DEV, dtype=torch.uint8)
+    st = torch.cuda.current_stream().cuda_stream
+    for ds in range(3):
+        g = torch.Generator(device=DEV).manual_seed(1000 * ds + M)
+        A = torch.randint(-127, 128, (M, K), device=DEV, dtype=torch.int8, generator=g)
+        W = torch.randint(-127, 128, (N, K), device=DEV, dtype=torch.int8, generator=g)
+        sa = torch.rand(K // block, M, device=DEV, generator=g) + 0.5
+        sw = torch.rand(K // block, N, device=DEV, generator=g) * 0.02
+        first = None
+        for rep in range(12):
+            C = torch.full((M, N), float("nan"), device=DEV, dtype=torch.float32)
+            rc = lib.bi8_gemm_nt_dequant_ws(A.data_ptr(), W.data_ptr(), sa.data_ptr(), sw.data_ptr(), None, 0, C.data_ptr(), 0,
+                                            M, N, K, K, K, N, block, ws.data_ptr(), need, st)
+            assert rc == 0, kernel
+            if rep % 4 == 0:
+                _ = (W[:64].float() @ W[:64].float().t()).sum()
+            if first is None:
+                first = C
+            else:
+                assert torch.equal(C, first), f"{kernel}: call {rep} of data set {ds} differs from the first"
+        full = torch.zeros(M, N, device=DEV, dtype=torch.float64)
+        for j in range(K // block):
+            p = A[:, j * block:(j + 1) * block].double() @ W[:, j * block:(j + 1) * block].double().t()
+            full += p * sa[j].double()[:, None] * sw[j].double()[None, :]
+        full /= 127.0 * 127.0
+        assert (first.double() - full).abs().max().item() <= 3e-6 * full.abs().max().item(), kernel
